@@ -1,0 +1,292 @@
+"""Stand-ins for the wire.  The hot path of this package is the *local* half of
+every primitive (pack, unpack, shard compute); what the reference sends through
+MPI or NCCL between those halves is supplied here by one of two transports:
+
+``LoopbackTransport``
+    every rank of a :class:`SimWorld` runs in its own thread of this process and
+    messages are handed over through a mailbox, device buffer to device buffer.
+    Semantics are those of the reference's exchange (post receives, pack, send,
+    unpack), so whole layers can be checked against their sequential
+    counterparts without MPI.
+
+``SoloTransport``
+    one live rank; peers are absent.  Receive buffers keep whatever the caller
+    seeded them with, gathers return registered peer contributions (or mirror
+    the live rank), and metadata assumes that every peer holds a shard shaped
+    like the live rank's.  This is the configuration timed by the benchmark:
+    exactly one rank's share of the work.
+"""
+
+import threading
+
+import numpy as np
+
+
+class TransportError(RuntimeError):
+    pass
+
+
+# ---------------------------------------------------------------------------
+# Solo
+# ---------------------------------------------------------------------------
+
+class SoloTransport:
+
+    # Receive buffers are filled before a layer runs, so a layer may consume all
+    # ghost slabs of all dimensions in one fused pass.
+    ghosts_preloaded = True
+
+    def __init__(self, world):
+        self.world = world
+        self._gather_providers = {}
+        self._shape_provider = None
+
+    # -- configuration by tests / benchmarks --------------------------------
+
+    def set_gather_provider(self, tag, fn):
+        """``fn(P, tensor) -> list of P.size tensors`` supplies what the peers
+        would contribute to a gather carrying ``tag`` (entry ``P.rank`` is
+        replaced by the live tensor)."""
+        self._gather_providers[tag] = fn
+
+    def set_peer_shape_provider(self, fn):
+        """``fn(P, index, my_shape) -> shape`` of the shard held by the peer at
+        Cartesian ``index``; default: same as the live rank's."""
+        self._shape_provider = fn
+
+    # -- metadata -----------------------------------------------------------
+
+    def subtensor_shapes(self, P, local_shape):
+        from ...utilities.slicing import range_index
+        table = np.zeros(list(P.shape) + [P.dim], dtype=int)
+        mine = np.asarray(local_shape, dtype=int)
+        for index in range_index(P.shape):
+            if self._shape_provider is not None and tuple(index) != tuple(P.index):
+                table[tuple(index)] = np.asarray(self._shape_provider(P, index, mine), dtype=int)
+            else:
+                table[tuple(index)] = mine
+        return table
+
+    def broadcast_data(self, P, data, root, P_data):
+        if data is None:
+            raise TransportError("solo transport: this rank does not hold the data being broadcast")
+        return data
+
+    def allgather_data(self, P, data):
+        return np.stack([np.asarray(data)] * P.size)
+
+    def allreduce_data(self, P, data, op):
+        data = np.asarray(data)
+        if op == "sum":
+            return data * P.size
+        return data
+
+    # -- tensors ------------------------------------------------------------
+
+    def exchange(self, P, sends, recvs):
+        """Nothing leaves and nothing arrives: receive buffers hold what the
+        caller seeded them with."""
+        return None
+
+    def allgather(self, P, tensor, tag=None):
+        import torch
+        fn = self._gather_providers.get(tag)
+        if fn is None:
+            parts = [tensor] * P.size
+        else:
+            parts = list(fn(P, tensor))
+            if len(parts) != P.size:
+                raise TransportError(f"gather provider for {tag!r} returned {len(parts)} parts for {P.size} workers")
+            parts[P.rank] = tensor
+        return torch.stack(parts)
+
+    def broadcast(self, P_src, P_dst, tensor, tag=None):
+        if P_src.active:
+            return tensor
+        raise TransportError("solo transport: the live rank is not a source of this broadcast")
+
+
+# ---------------------------------------------------------------------------
+# Loopback
+# ---------------------------------------------------------------------------
+
+class _Mailbox:
+
+    def __init__(self, timeout):
+        self.cv = threading.Condition()
+        self.slots = {}
+        self.failed = None
+        self.timeout = timeout
+
+    def put(self, key, value, readers=1):
+        with self.cv:
+            if key in self.slots:
+                raise TransportError(f"mailbox key {key!r} posted twice")
+            self.slots[key] = [value, readers]
+            self.cv.notify_all()
+
+    def take(self, key):
+        with self.cv:
+            ok = self.cv.wait_for(lambda: key in self.slots or self.failed is not None, timeout=self.timeout)
+            if self.failed is not None:
+                raise TransportError(f"another rank failed: {self.failed!r}")
+            if not ok:
+                raise TransportError(f"timed out waiting for {key!r}")
+            slot = self.slots[key]
+            slot[1] -= 1
+            if slot[1] == 0:
+                del self.slots[key]
+            return slot[0]
+
+    def fail(self, exc):
+        with self.cv:
+            if self.failed is None:
+                self.failed = exc
+            self.cv.notify_all()
+
+
+class LoopbackTransport:
+
+    ghosts_preloaded = False
+
+    def __init__(self, world, timeout=120.0):
+        self.world = world
+        self.mail = _Mailbox(timeout)
+        self._seq = {}
+        self._seq_lock = threading.Lock()
+
+    @classmethod
+    def run(cls, world, fn, timeout=120.0):
+        transport = cls(world, timeout)
+        previous = world.transport
+        world.transport = transport
+        results = [None] * world.size
+        errors = [None] * world.size
+
+        def body(rank):
+            try:
+                results[rank] = fn(world.partition(rank))
+            except BaseException as exc:  # noqa: B902 - re-raised below
+                errors[rank] = exc
+                transport.mail.fail(exc)
+
+        threads = [threading.Thread(target=body, args=(r,), name=f"sim-rank-{r}") for r in range(world.size)]
+        try:
+            for t in threads:
+                t.start()
+            for t in threads:
+                t.join()
+        finally:
+            world.transport = previous
+        for rank, exc in enumerate(errors):
+            if exc is not None and not isinstance(exc, TransportError):
+                raise exc
+        for exc in errors:
+            if exc is not None:
+                raise exc
+        return results
+
+    def _next(self, me, group, kind):
+        key = (me, group, kind)
+        with self._seq_lock:
+            n = self._seq.get(key, 0)
+            self._seq[key] = n + 1
+        return n
+
+    # -- collectives on host data ---------------------------------------------
+
+    def _allgather_obj(self, P, obj, kind):
+        group = P._ranks
+        seq = self._next(P._me, group, kind)
+        self.mail.put((kind, group, seq, P._me), obj, readers=len(group))
+        return [self.mail.take((kind, group, seq, r)) for r in group]
+
+    def subtensor_shapes(self, P, local_shape):
+        shapes = self._allgather_obj(P, tuple(int(s) for s in local_shape), "shapes")
+        table = np.zeros(list(P.shape) + [P.dim], dtype=int)
+        for rank, shape in enumerate(shapes):
+            table[tuple(P.index_of_rank(rank))] = np.asarray(shape, dtype=int)
+        return table
+
+    def broadcast_data(self, P, data, root, P_data):
+        if P_data is not None:
+            source = P_data._ranks[0] if P_data._ranks is not None else getattr(P_data, "_ranks_released", (None,))[0]
+        else:
+            source = P._ranks[root]
+        everyone = self._allgather_obj(P, data, "bcast")
+        return everyone[P._ranks.index(source)]
+
+    def allgather_data(self, P, data):
+        return np.stack([np.asarray(d) for d in self._allgather_obj(P, data, "gather")])
+
+    def allreduce_data(self, P, data, op):
+        parts = [np.asarray(d) for d in self._allgather_obj(P, data, "reduce")]
+        if op == "sum":
+            return np.sum(parts, axis=0)
+        if op == "max":
+            return np.max(parts, axis=0)
+        if op == "min":
+            return np.min(parts, axis=0)
+        raise ValueError(f"unknown reduction {op!r}")
+
+    # -- tensors ------------------------------------------------------------
+
+    def exchange(self, P, sends, recvs):
+        """``sends`` / ``recvs``: lists of ``(peer_rank_in_P, tensor, tag)``.
+        All sends are posted, then receives are completed in list order (the
+        copy is enqueued on the current stream, after the sender's pack), then
+        the sender waits until every peer has taken its message so that the
+        buffer may be reused."""
+        group = P._ranks
+        me = P._me
+        acks = []
+        for peer, tensor, tag in sends:
+            dst = group[peer]
+            seq = self._next(me, group, ("send", dst, tag))
+            self.mail.put(("p2p", group, me, dst, tag, seq), tensor)
+            acks.append(("ack", group, me, dst, tag, seq))
+        for peer, tensor, tag in recvs:
+            src = group[peer]
+            seq = self._next(me, group, ("recv", src, tag))
+            payload = self.mail.take(("p2p", group, src, me, tag, seq))
+            if tuple(payload.shape) != tuple(tensor.shape) or payload.dtype != tensor.dtype:
+                raise TransportError(f"message {tuple(payload.shape)}/{payload.dtype} does not fit receive buffer "
+                                     f"{tuple(tensor.shape)}/{tensor.dtype}")
+            tensor.copy_(payload)
+            self.mail.put(("ack", group, src, me, tag, seq), True)
+        for key in acks:
+            self.mail.take(key)
+
+    def allgather(self, P, tensor, tag=None):
+        import torch
+        parts = self._allgather_obj(P, tensor, ("tgather", tag))
+        out = torch.stack(parts)
+        # Nobody may overwrite its contribution before everyone has stacked it.
+        self._allgather_obj(P, None, ("tgather-done", tag))
+        return out
+
+    def broadcast(self, P_src, P_dst, tensor, tag=None):
+        """Every worker of ``P_dst`` receives the tensor held by the worker of
+        ``P_src`` that shares its index in the dimensions ``P_src`` spans
+        (weights stored on a sub-grid, used on the full grid)."""
+        union = P_src.create_partition_union(P_dst)
+        key = ("tbcast", tag)
+        payload = (tuple(int(i) for i in P_src.index), tensor) if P_src.active else None
+        everyone = self._allgather_obj(union, payload, key)
+        out = tensor
+        if P_dst.active and not P_src.active:
+            mine = [int(i) for i in P_dst.index]
+            match = None
+            for item in everyone:
+                if item is None:
+                    continue
+                index, t = item
+                src_shape = [int(s) for s in P_src.shape]
+                if all(src_shape[d] == 1 or index[d] == mine[d] for d in range(len(src_shape))):
+                    match = t
+                    break
+            if match is None:
+                raise TransportError("broadcast: no source worker matches this destination index")
+            out = match.clone()
+        self._allgather_obj(union, None, ("tbcast-done", tag))
+        return out

@@ -1,0 +1,93 @@
+// DistributedEmbedding shard gather (reference: nn/embedding.py:244-246,
+// torch.nn.functional.embedding on the local table).  out[t] is row ids[t]-lo of
+// the table when lo <= ids[t] < hi and a row of zero bits otherwise.  Rows are
+// opaque bytes: one wavefront moves one token's row as 16-byte vectors, eight
+// vectors per lane in flight; misses issue no loads at all.
+#include "ddl_common.h"
+
+namespace ddl {
+namespace {
+
+constexpr int kWave = 64;
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / kWave;
+constexpr int kInFlight = 8;
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+template <typename V, typename IdT>
+__global__ __launch_bounds__(kBlock) void gather_rows(const char* __restrict__ weight, int64_t ldw_bytes, int64_t nvec,
+                                                      const IdT* __restrict__ ids, int64_t n_ids, int64_t lo, int64_t hi,
+                                                      char* __restrict__ out) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + threadIdx.x / kWave;
+    if (t >= n_ids) return;
+    const int64_t id = static_cast<int64_t>(ids[t]);
+    const bool hit = id >= lo && id < hi;
+    V* dst = reinterpret_cast<V*>(out + t * nvec * static_cast<int64_t>(sizeof(V)));
+    if (!hit) {
+        V z;
+        __builtin_memset(&z, 0, sizeof(V));
+        for (int64_t c = lane; c < nvec; c += kWave) __builtin_nontemporal_store(z, dst + c);
+        return;
+    }
+    const V* src = reinterpret_cast<const V*>(weight + (id - lo) * ldw_bytes);
+    for (int64_t c0 = 0; c0 < nvec; c0 += kWave * kInFlight) {
+        V v[kInFlight];
+#pragma unroll
+        for (int k = 0; k < kInFlight; ++k) {
+            const int64_t c = c0 + lane + k * kWave;
+            if (c < nvec) v[k] = src[c];
+        }
+#pragma unroll
+        for (int k = 0; k < kInFlight; ++k) {
+            const int64_t c = c0 + lane + k * kWave;
+            if (c < nvec) __builtin_nontemporal_store(v[k], dst + c);
+        }
+    }
+}
+
+template <typename V>
+int launch_gather(const void* w, int64_t ldw_bytes, int64_t row_bytes, const void* ids, int i64, int64_t n, int64_t lo,
+                  int64_t hi, void* out, hipStream_t s) {
+    const int64_t nvec = row_bytes / static_cast<int64_t>(sizeof(V));
+    const int64_t blocks = (n + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (blocks > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "embedding gather: more than 2^33 ids in one call");
+    if (i64)
+        hipLaunchKernelGGL((gather_rows<V, int64_t>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, s,
+                           static_cast<const char*>(w), ldw_bytes, nvec, static_cast<const int64_t*>(ids), n, lo, hi,
+                           static_cast<char*>(out));
+    else
+        hipLaunchKernelGGL((gather_rows<V, int32_t>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, s,
+                           static_cast<const char*>(w), ldw_bytes, nvec, static_cast<const int32_t*>(ids), n, lo, hi,
+                           static_cast<char*>(out));
+    return check_launch("gather_rows");
+}
+
+}  // namespace
+}  // namespace ddl
+
+extern "C" int ddl_embedding_gather(const void* weight, int64_t dim, int64_t ldw, int elem_size, const void* ids,
+                                    int ids_is_i64, int64_t n_ids, int64_t lo, int64_t hi, void* out, void* stream) {
+    using namespace ddl;
+    if (dim < 1 || ldw < dim || n_ids < 0 || hi < lo)
+        return fail(DDL_E_ARG, "embedding gather: dim=%lld ldw=%lld n_ids=%lld window=[%lld,%lld)", (long long)dim,
+                    (long long)ldw, (long long)n_ids, (long long)lo, (long long)hi);
+    if (elem_size != 1 && elem_size != 2 && elem_size != 4 && elem_size != 8)
+        return fail(DDL_E_ARG, "embedding gather: element size %d not in {1,2,4,8}", elem_size);
+    if (n_ids == 0) return 0;
+    if (!ids || !out || (!weight && hi > lo)) return fail(DDL_E_ARG, "embedding gather: null pointer");
+    if (!aligned_to(ids, ids_is_i64 ? 8 : 4)) return fail(DDL_E_ALIGN, "embedding gather: ids misaligned");
+    if (!aligned_to(out, elem_size) || !aligned_to(weight, elem_size))
+        return fail(DDL_E_ALIGN, "embedding gather: table or output not aligned to the element size");
+    const int64_t row_bytes = dim * elem_size, ldw_bytes = ldw * elem_size;
+    const uint64_t bits = static_cast<uint64_t>(row_bytes) | static_cast<uint64_t>(ldw_bytes) |
+                          reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(out);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if ((bits & 15) == 0) return launch_gather<u32x4>(weight, ldw_bytes, row_bytes, ids, ids_is_i64, n_ids, lo, hi, out, s);
+    if ((bits & 7) == 0) return launch_gather<u32x2>(weight, ldw_bytes, row_bytes, ids, ids_is_i64, n_ids, lo, hi, out, s);
+    if ((bits & 3) == 0) return launch_gather<uint32_t>(weight, ldw_bytes, row_bytes, ids, ids_is_i64, n_ids, lo, hi, out, s);
+    if ((bits & 1) == 0) return launch_gather<uint16_t>(weight, ldw_bytes, row_bytes, ids, ids_is_i64, n_ids, lo, hi, out, s);
+    return launch_gather<uint8_t>(weight, ldw_bytes, row_bytes, ids, ids_is_i64, n_ids, lo, hi, out, s);
+}

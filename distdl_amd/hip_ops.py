@@ -1,0 +1,319 @@
+"""Torch-tensor front end of the C ABI: device checks, pointer extraction and
+the current HIP stream.  Nothing here computes; every function ends in one call
+into ``libdistdl_hip.so`` and raises when that is impossible.
+"""
+
+import ctypes
+
+import torch
+
+from . import _lib
+
+_ADD_DTYPES = {
+    torch.float32: _lib.DDL_DT_F32,
+    torch.float64: _lib.DDL_DT_F64,
+    torch.bfloat16: _lib.DDL_DT_BF16,
+    torch.float16: _lib.DDL_DT_F16,
+}
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _require_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "distdl_amd: tensor on %s; the HIP path only accepts GPU tensors and there is no CPU fallback"
+                % (t.device,))
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+class BoxPlan:
+    """Box geometry of one strided tensor, converted to C arrays once.
+
+    ``boxes`` is a list of ``(start, shape)`` pairs (or ``None`` for an absent
+    box) in the coordinates of a tensor with the given shape / strides; the
+    contiguous buffers on the other side are supplied per call.  Built where the
+    reference builds its overlap lists (the forward pre-hook), used on every
+    forward and adjoint call.
+    """
+
+    def __init__(self, tensor_shape, tensor_strides, boxes):
+        self.ndim = len(tensor_shape)
+        if self.ndim < 1 or self.ndim > _lib.DDL_MAX_DIMS:
+            raise ValueError(f"tensors of rank {self.ndim} are not supported (1..{_lib.DDL_MAX_DIMS})")
+        self.tensor_shape = tuple(int(s) for s in tensor_shape)
+        self.tensor_strides = tuple(int(s) for s in tensor_strides)
+        self.shape_arr = _lib.i64_array(self.tensor_shape)
+        self.stride_arr = _lib.i64_array(self.tensor_strides)
+        self.present = [b is not None for b in boxes]
+        starts, shapes = [], []
+        for b in boxes:
+            if b is None:
+                starts += [0] * self.ndim
+                shapes += [0] * self.ndim
+            else:
+                starts += list(b[0])
+                shapes += list(b[1])
+        self.nbox = len(boxes)
+        self.box_shapes = [None if b is None else tuple(int(v) for v in b[1]) for b in boxes]
+        self.start_arr = _lib.i64_array(starts)
+        self.boxshape_arr = _lib.i64_array(shapes)
+
+    @classmethod
+    def from_slices(cls, tensor, slice_list):
+        boxes = []
+        for sl in slice_list:
+            if sl is None:
+                boxes.append(None)
+            else:
+                boxes.append(([int(s.start) for s in sl], [int(s.stop) - int(s.start) for s in sl]))
+        return cls(tensor.shape, tensor.stride(), boxes)
+
+    def matches(self, tensor):
+        return tuple(tensor.shape) == self.tensor_shape and tuple(tensor.stride()) == self.tensor_strides
+
+    def _buf_ptrs(self, bufs, dtype, device):
+        if len(bufs) != self.nbox:
+            raise ValueError(f"expected {self.nbox} buffers, got {len(bufs)}")
+        ptrs = []
+        for buf, shape in zip(bufs, self.box_shapes):
+            if buf is None or shape is None:
+                ptrs.append(None)
+                continue
+            _require_gpu(buf)
+            if buf.dtype != dtype or not buf.is_contiguous() or tuple(buf.shape) != shape:
+                raise ValueError(f"buffer {tuple(buf.shape)}/{buf.dtype} does not match box {shape}/{dtype} "
+                                 "or is not contiguous")
+            ptrs.append(buf.data_ptr())
+        return _lib.ptr_array(ptrs)
+
+    def pack(self, tensor, bufs):
+        """bufs[b][...] = tensor[box b]"""
+        _require_gpu(tensor)
+        if not self.matches(tensor):
+            raise ValueError("tensor structure differs from the one this plan was built for")
+        if self.nbox == 0:
+            return
+        ptrs = self._buf_ptrs(bufs, tensor.dtype, tensor.device)
+        rc = _lib.load().ddl_pack_boxes(tensor.data_ptr(), self.shape_arr, self.stride_arr, self.ndim,
+                                        tensor.element_size(), self.nbox, self.start_arr, self.boxshape_arr,
+                                        ptrs, _stream())
+        _lib.check(rc, "ddl_pack_boxes")
+
+    def unpack(self, tensor, bufs, accumulate=False):
+        """tensor[box b] = bufs[b]   (+= when accumulate)"""
+        _require_gpu(tensor)
+        if not self.matches(tensor):
+            raise ValueError("tensor structure differs from the one this plan was built for")
+        if self.nbox == 0:
+            return
+        ptrs = self._buf_ptrs(bufs, tensor.dtype, tensor.device)
+        op, dt = _lib.DDL_OP_COPY, _lib.DDL_DT_BITS
+        if accumulate:
+            if tensor.dtype not in _ADD_DTYPES:
+                raise ValueError(f"accumulating unpack is not available for {tensor.dtype}")
+            op, dt = _lib.DDL_OP_ADD, _ADD_DTYPES[tensor.dtype]
+        rc = _lib.load().ddl_unpack_boxes(tensor.data_ptr(), self.shape_arr, self.stride_arr, self.ndim,
+                                          tensor.element_size(), self.nbox, self.start_arr, self.boxshape_arr,
+                                          ptrs, op, dt, _stream())
+        _lib.check(rc, "ddl_unpack_boxes")
+
+    def zero(self, tensor):
+        """tensor[box b] = 0 for every box"""
+        _require_gpu(tensor)
+        if not self.matches(tensor):
+            raise ValueError("tensor structure differs from the one this plan was built for")
+        if self.nbox == 0:
+            return
+        rc = _lib.load().ddl_zero_boxes(tensor.data_ptr(), self.shape_arr, self.stride_arr, self.ndim,
+                                        tensor.element_size(), self.nbox, self.start_arr, self.boxshape_arr, _stream())
+        _lib.check(rc, "ddl_zero_boxes")
+
+
+def copy_box(src, src_slices, dst, dst_slices, accumulate=False):
+    """dst[dst_slices] (+)= src[src_slices]; both strided, same box shape."""
+    _require_gpu(src, dst)
+    if src.dtype != dst.dtype:
+        raise ValueError("copy_box: dtype mismatch")
+    nd = src.dim()
+    if dst.dim() != nd or len(src_slices) != nd or len(dst_slices) != nd:
+        raise ValueError("copy_box: rank mismatch")
+    box = _lib.ddl_box_t()
+    box.ndim = nd
+    soff = doff = 0
+    for d in range(nd):
+        n = int(src_slices[d].stop) - int(src_slices[d].start)
+        if n != int(dst_slices[d].stop) - int(dst_slices[d].start):
+            raise ValueError("copy_box: source and destination boxes differ in shape")
+        if src_slices[d].start < 0 or src_slices[d].stop > src.shape[d] or \
+           dst_slices[d].start < 0 or dst_slices[d].stop > dst.shape[d]:
+            raise ValueError("copy_box: box outside tensor")
+        box.shape[d] = n
+        box.src_stride[d] = src.stride(d)
+        box.dst_stride[d] = dst.stride(d)
+        soff += int(src_slices[d].start) * src.stride(d)
+        doff += int(dst_slices[d].start) * dst.stride(d)
+    es = src.element_size()
+    box.src = src.data_ptr() + soff * es
+    box.dst = dst.data_ptr() + doff * es
+    op, dt = _lib.DDL_OP_COPY, _lib.DDL_DT_BITS
+    if accumulate:
+        op, dt = _lib.DDL_OP_ADD, _ADD_DTYPES[src.dtype]
+    rc = _lib.load().ddl_copy_boxes(ctypes.byref(box), 1, es, op, dt, _stream())
+    _lib.check(rc, "ddl_copy_boxes")
+
+
+class HaloPadPlan:
+    """Geometry of the fused pad + ghost fill + bulk pack call for one shard shape."""
+
+    def __init__(self, x_shape, pad, recv, send):
+        self.x_shape = tuple(int(s) for s in x_shape)
+        self.ndim = len(self.x_shape)
+        self.pad = [[int(p[0]), int(p[1])] for p in pad]
+        self.recv = [[int(p[0]), int(p[1])] for p in recv]
+        self.send = [[int(p[0]), int(p[1])] for p in send]
+        self.padded_shape = tuple(s + p[0] + p[1] for s, p in zip(self.x_shape, self.pad))
+        self.shape_arr = _lib.i64_array(self.x_shape)
+        self.pad_arr = _lib.i64_array([v for p in self.pad for v in p])
+        self.recv_arr = _lib.i64_array([v for p in self.recv for v in p])
+        self.send_arr = _lib.i64_array([v for p in self.send for v in p])
+
+    def slab_shape(self, dim, side, kind):
+        """Shape of the ghost (kind='ghost') or bulk slab of (dim, side); None if empty."""
+        widths = self.recv if kind == "ghost" else self.send
+        w = widths[dim][side]
+        if w == 0:
+            return None
+        shape = []
+        for j in range(self.ndim):
+            if j < dim:
+                shape.append(self.padded_shape[j])
+            elif j == dim:
+                shape.append(w)
+            else:
+                shape.append(self.padded_shape[j] - self.recv[j][0] - self.recv[j][1])
+        return tuple(shape)
+
+    def run(self, x, ghost_bufs, bulk_bufs, out=None):
+        """ghost_bufs / bulk_bufs: ``[ndim][2]`` nested lists of tensors or None."""
+        _require_gpu(x)
+        if tuple(x.shape) != self.x_shape or not x.is_contiguous():
+            raise ValueError("halo_pad_exchange: input must be contiguous with the planned shape")
+        if out is None:
+            out = torch.empty(self.padded_shape, dtype=x.dtype, device=x.device)
+        elif tuple(out.shape) != self.padded_shape or not out.is_contiguous() or out.dtype != x.dtype:
+            raise ValueError("halo_pad_exchange: bad output tensor")
+        gptr, bptr = [], []
+        for d in range(self.ndim):
+            for s in range(2):
+                for kind, bufs, ptrs in (("ghost", ghost_bufs, gptr), ("bulk", bulk_bufs, bptr)):
+                    buf = None if bufs is None else bufs[d][s]
+                    shape = self.slab_shape(d, s, kind)
+                    if buf is None or shape is None:
+                        ptrs.append(None)
+                        continue
+                    _require_gpu(buf)
+                    if tuple(buf.shape) != shape or not buf.is_contiguous() or buf.dtype != x.dtype:
+                        raise ValueError(f"halo_pad_exchange: {kind} slab ({d},{s}) must be contiguous {shape}, "
+                                         f"got {tuple(buf.shape)}")
+                    ptrs.append(buf.data_ptr())
+        rc = _lib.load().ddl_halo_pad_exchange(x.data_ptr(), out.data_ptr(), self.shape_arr, self.ndim,
+                                               x.element_size(), self.pad_arr, self.recv_arr, self.send_arr,
+                                               _lib.ptr_array(gptr), _lib.ptr_array(bptr), _stream())
+        _lib.check(rc, "ddl_halo_pad_exchange")
+        return out
+
+
+def ln_partial_stats(x2d, out=None):
+    """{mean, M2} per row of a [rows, cols] fp32 view (last stride 1)."""
+    _require_gpu(x2d)
+    if x2d.dtype != torch.float32 or x2d.dim() != 2 or (x2d.shape[1] > 1 and x2d.stride(1) != 1):
+        raise ValueError("ln_partial_stats: need a 2-D fp32 tensor with unit column stride")
+    rows, cols = x2d.shape
+    if out is None:
+        out = torch.empty((rows, 2), dtype=torch.float32, device=x2d.device)
+    rc = _lib.load().ddl_ln_partial_stats_f32(x2d.data_ptr(), rows, cols, x2d.stride(0) if rows > 1 else cols,
+                                              out.data_ptr(), _stream())
+    _lib.check(rc, "ddl_ln_partial_stats_f32")
+    return out
+
+
+def ln_normalize_affine(x2d, part_stats, part_cols, gamma, beta, eps, want_stats=False):
+    """Combines [P, rows, 2] partial statistics and normalises x2d; returns y (and mean, rstd)."""
+    _require_gpu(x2d, part_stats, gamma, beta)
+    if x2d.dtype != torch.float32 or x2d.dim() != 2 or (x2d.shape[1] > 1 and x2d.stride(1) != 1):
+        raise ValueError("ln_normalize_affine: need a 2-D fp32 tensor with unit column stride")
+    rows, cols = x2d.shape
+    nparts = len(part_cols)
+    if part_stats.dtype != torch.float32 or tuple(part_stats.shape) != (nparts, rows, 2) or \
+       not part_stats.is_contiguous():
+        raise ValueError(f"ln_normalize_affine: part_stats must be contiguous fp32 [{nparts}, {rows}, 2]")
+    for p in (gamma, beta):
+        if p is not None and (p.dtype != torch.float32 or p.numel() != cols or not p.is_contiguous()):
+            raise ValueError("ln_normalize_affine: gamma / beta must be contiguous fp32 with `cols` elements")
+    y = torch.empty((rows, cols), dtype=torch.float32, device=x2d.device)
+    mean = rstd = None
+    if want_stats:
+        mean = torch.empty((rows,), dtype=torch.float32, device=x2d.device)
+        rstd = torch.empty((rows,), dtype=torch.float32, device=x2d.device)
+    rc = _lib.load().ddl_ln_normalize_affine_f32(x2d.data_ptr(), rows, cols, x2d.stride(0) if rows > 1 else cols,
+                                                 part_stats.data_ptr(), nparts, _lib.i64_array(part_cols),
+                                                 _ptr(gamma), _ptr(beta), float(eps), y.data_ptr(), cols,
+                                                 _ptr(mean), _ptr(rstd), _stream())
+    _lib.check(rc, "ddl_ln_normalize_affine_f32")
+    return (y, mean, rstd) if want_stats else y
+
+
+def embedding_gather(weight, ids, lo, hi, out=None):
+    """out[t] = weight[ids[t] - lo] if lo <= ids[t] < hi else 0."""
+    _require_gpu(weight, ids)
+    if weight.dim() != 2 or (weight.shape[1] > 1 and weight.stride(1) != 1):
+        raise ValueError("embedding_gather: weight must be 2-D with unit column stride")
+    if ids.dtype not in (torch.int64, torch.int32):
+        raise ValueError("embedding_gather: ids must be int32 or int64")
+    if weight.shape[0] != hi - lo:
+        raise ValueError(f"embedding_gather: table has {weight.shape[0]} rows but the window is [{lo},{hi})")
+    ids_c = ids.contiguous()
+    dim = weight.shape[1]
+    if out is None:
+        out = torch.empty(tuple(ids.shape) + (dim,), dtype=weight.dtype, device=weight.device)
+    elif not out.is_contiguous() or out.numel() != ids.numel() * dim or out.dtype != weight.dtype:
+        raise ValueError("embedding_gather: bad output tensor")
+    rc = _lib.load().ddl_embedding_gather(weight.data_ptr(), dim, weight.stride(0) if weight.shape[0] > 1 else dim,
+                                          weight.element_size(), ids_c.data_ptr(),
+                                          1 if ids.dtype == torch.int64 else 0, ids_c.numel(), int(lo), int(hi),
+                                          out.data_ptr(), _stream())
+    _lib.check(rc, "ddl_embedding_gather")
+    return out
+
+
+def linear_bf16(x, weight, bias=None, out=None):
+    """y = x @ weight.T + bias; bf16 operands, fp32 accumulation, bf16 result."""
+    _require_gpu(x, weight, bias)
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or (bias is not None and bias.dtype != torch.bfloat16):
+        raise ValueError("linear_bf16: operands must be bfloat16")
+    if weight.dim() != 2 or x.shape[-1] != weight.shape[1]:
+        raise ValueError(f"linear_bf16: x[..., {x.shape[-1]}] does not match weight {tuple(weight.shape)}")
+    n, k = weight.shape
+    x2 = x.reshape(-1, k)
+    if x2.stride(1) != 1 and k > 1:
+        x2 = x2.contiguous()
+    if weight.stride(1) != 1 and k > 1:
+        weight = weight.contiguous()
+    if bias is not None and (bias.numel() != n or not bias.is_contiguous()):
+        raise ValueError("linear_bf16: bias must be contiguous with out_features elements")
+    m = x2.shape[0]
+    if out is None:
+        out = torch.empty(tuple(x.shape[:-1]) + (n,), dtype=torch.bfloat16, device=x.device)
+    elif not out.is_contiguous() or out.numel() != m * n or out.dtype != torch.bfloat16:
+        raise ValueError("linear_bf16: bad output tensor")
+    rc = _lib.load().ddl_linear_bf16(x2.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(), m, n, k,
+                                     x2.stride(0) if m > 1 else k, weight.stride(0) if n > 1 else k, n, _stream())
+    _lib.check(rc, "ddl_linear_bf16")
+    return out

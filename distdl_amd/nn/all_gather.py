@@ -1,0 +1,34 @@
+"""AllGather layer stand-in (reference: nn/all_gather.py).  Under the solo
+transport the caller supplies the already gathered activation and the layer is
+the identity; under loopback the shards are concatenated along the axis."""
+
+import numpy as np
+import torch
+
+from .module import Module
+
+
+class AllGather(Module):
+
+    def __init__(self, P_x, axes_all_gather=None, axes_keep=None, scale_backward=None):
+        super().__init__()
+        self.P_x = P_x
+        if not P_x.active:
+            return
+        if axes_all_gather is None:
+            axes_all_gather = [d for d in range(P_x.dim) if d not in [int(a) for a in axes_keep]]
+        self.axes = tuple(int(a) for a in axes_all_gather)
+        keep = [d in self.axes for d in range(P_x.dim)]
+        self.P_allgather = P_x.create_cartesian_subtopology_partition(keep)
+        self.identity = int(np.prod(self.P_allgather.shape)) == 1
+
+    def forward(self, input):
+        if not self.P_x.active or self.identity:
+            return input
+        transport = self.P_x._world.transport
+        if getattr(transport, "ghosts_preloaded", False):
+            return input  # solo: the input already is the gathered tensor
+        if len(self.axes) != 1:
+            raise NotImplementedError("AllGather along several axes is not part of this build")
+        parts = transport.allgather(self.P_allgather, input.detach(), tag="all_gather")
+        return torch.cat(list(parts), dim=self.axes[0])

@@ -1,0 +1,248 @@
+"""Feature-space partitioned convolution (reference: nn/conv_feature.py:16-466).
+
+What this build accelerates is the input staging in front of the local
+convolution (reference forward, :399-410): zero padding on global boundaries,
+halo exchange with the neighbours, cropping to the needed range.  When every
+ghost slab is available before the call (solo transport) the padding, the ghost
+fill and the packing of the outgoing slabs run as ONE kernel
+(``ddl_halo_pad_exchange``); otherwise the padding kernel is followed by the
+dimension-ordered HaloExchange layer.  The convolution itself stays the stock
+``torch.nn.ConvNd`` the reference calls (:411).
+"""
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+from .. import hip_ops
+from ..utilities.slicing import assemble_slices
+from ..utilities.slicing import compute_nd_slice_shape
+from ..utilities.torch import TensorStructure
+from ..utilities.torch import zero_volume_tensor
+from .broadcast import Broadcast
+from .halo_exchange import HaloExchange
+from .mixins.conv_mixin import ConvMixin
+from .mixins.halo_mixin import HaloMixin
+from .module import Module
+
+
+class _HaloStaging(torch.autograd.Function):
+    """pad + exchange of one shard through the fused kernel."""
+
+    @staticmethod
+    def forward(ctx, input, plan, ghost_bufs, bulk_bufs):
+        x = input.detach()
+        if not x.is_contiguous():
+            x = x.contiguous()
+        return plan.run(x, ghost_bufs, bulk_bufs)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        raise NotImplementedError("the adjoint of the fused halo staging is not part of this build")
+
+
+class DistributedFeatureConvBase(Module, HaloMixin, ConvMixin):
+    r"""Convolution over a tensor partitioned in feature space only:
+    ``P_x ~ 1 x 1 x P_{d-1} x ... x P_0``; the output reuses ``P_x``.  Weights
+    live on worker 0 and are broadcast.  Arguments as the reference (and as the
+    wrapped ``torch.nn.ConvNd``)."""
+
+    TorchConvType = None
+    num_dimensions = None
+
+    def __init__(self, P_x, in_channels, out_channels, kernel_size, stride=1, padding=0, padding_mode='zeros',
+                 dilation=1, groups=1, bias=True, buffer_manager=None, collect_state=False):
+        super().__init__()
+        self.P_x = P_x
+        if buffer_manager is None:
+            buffer_manager = self._distdl_backend.BufferManager()
+        elif not isinstance(buffer_manager, self._distdl_backend.BufferManager):
+            raise ValueError("Buffer manager type does not match backend.")
+        self.buffer_manager = buffer_manager
+        if not self.P_x.active:
+            return
+        if padding_mode != 'zeros':
+            raise NotImplementedError("only zero padding is staged by the HIP kernels")
+
+        self.in_channels = in_channels
+        self.out_channels = out_channels
+        self.kernel_size = self._expand_parameter(kernel_size)
+        self.stride = self._expand_parameter(stride)
+        self.padding = self._expand_parameter(padding)
+        self.padding_mode = padding_mode
+        self.dilation = self._expand_parameter(dilation)
+        self.groups = groups
+        self.use_bias = bias
+        self.collect_state = collect_state
+
+        # A stock layer provides the default initialisation of the parameters;
+        # only worker 0 keeps them, the others receive them by broadcast.
+        template = self.TorchConvType(in_channels=in_channels, out_channels=out_channels,
+                                      kernel_size=self.kernel_size, stride=self.stride, padding=0,
+                                      padding_mode='zeros', dilation=self.dilation, groups=groups, bias=bias,
+                                      device=P_x.device)
+        self._conv_fn = {1: F.conv1d, 2: F.conv2d, 3: F.conv3d}[self.num_dimensions]
+
+        dims = len(self.P_x.shape)
+        self.global_padding = np.concatenate([np.zeros(dims - len(self.padding), dtype=int),
+                                              np.asarray(self.padding, dtype=int)])
+        self.local_padding = self._compute_local_padding(np.stack([self.global_padding, self.global_padding], axis=1))
+
+        P_wb = self.P_x.create_partition_inclusive([0])
+        self.P_wb_cart = P_wb.create_cartesian_topology_partition([1])
+        P_wb.deactivate()
+        if self.P_wb_cart.active:
+            self.weight = torch.nn.Parameter(template.weight.detach().clone())
+            if bias:
+                self.bias = torch.nn.Parameter(template.bias.detach().clone())
+            else:
+                self.register_buffer('bias', None)
+        else:
+            self.register_buffer('weight', zero_volume_tensor(device=P_x.device))
+            if bias:
+                self.register_buffer('bias', zero_volume_tensor(device=P_x.device))
+            else:
+                self.register_buffer('bias', None)
+
+        self.w_broadcast = Broadcast(self.P_wb_cart, self.P_x, preserve_batch=False)
+        if bias:
+            self.b_broadcast = Broadcast(self.P_wb_cart, self.P_x, preserve_batch=False)
+
+        self.needed_slices = None
+        self.halo_layer = None
+        self._staging_plan = None
+        self._distdl_is_setup = False
+        self._input_tensor_structure = TensorStructure()
+
+    def _expand_parameter(self, param):
+        param = np.atleast_1d(param)
+        if len(param) == 1:
+            param = np.ones(self.num_dimensions, dtype=int) * param[0]
+        elif len(param) != self.num_dimensions:
+            raise ValueError('Invalid parameter: ' + str(param))
+        return tuple(int(p) for p in param)
+
+    def _compute_local_padding(self, padding):
+        """Explicit zero padding exists only on the sides of the shard that lie
+        on the global boundary (reference :367-377)."""
+        on_left = [k == 0 for k in self.P_x.index]
+        on_right = [k == d - 1 for k, d in zip(self.P_x.index, self.P_x.shape)]
+        return np.where(np.stack((on_left, on_right), axis=1), padding, 0)
+
+    def _distdl_module_setup(self, input):
+        """Halo geometry for the structure of ``input[0]``, computed on the
+        explicitly padded global tensor with padding 0 (reference :263-328)."""
+        self._distdl_is_setup = True
+        self._input_tensor_structure = TensorStructure(input[0])
+        if not self.P_x.active:
+            return
+        backend = self._distdl_backend
+        x_global_structure = backend.assemble_global_tensor_structure(input[0], self.P_x)
+        x_global_shape_after_pad = np.asarray(x_global_structure.shape) + 2 * self.global_padding
+        padded = TensorStructure(input[0])
+        padded.shape = np.asarray(input[0].shape) + np.sum(self.local_padding, axis=1)
+        subtensor_shapes = backend.tensor_decomposition.compute_subtensor_shapes_unbalanced(padded, self.P_x)
+
+        halo_shape, recv_buffer_shape, send_buffer_shape, needed_ranges = self._compute_exchange_info(
+            x_global_shape_after_pad, self.kernel_size, self.stride, self._expand_parameter(0), self.dilation,
+            self.P_x.active, self.P_x.shape, self.P_x.index, subtensor_shapes=subtensor_shapes)
+        self.halo_shape = halo_shape
+        self.recv_buffer_shape = recv_buffer_shape
+        self.send_buffer_shape = send_buffer_shape
+        self.halo_layer = HaloExchange(self.P_x, halo_shape, recv_buffer_shape, send_buffer_shape,
+                                       buffer_manager=self.buffer_manager)
+        self.needed_slices = assemble_slices(needed_ranges[:, 0], needed_ranges[:, 1])
+
+        total_padding = self.local_padding + self.halo_shape
+        self._pad_only_plan = hip_ops.HaloPadPlan(input[0].shape, total_padding,
+                                                  np.zeros_like(total_padding), np.zeros_like(total_padding))
+        self._staging_plan = hip_ops.HaloPadPlan(input[0].shape, total_padding, recv_buffer_shape, send_buffer_shape)
+
+    def _distdl_module_teardown(self, input):
+        self.needed_slices = None
+        self.halo_layer = None
+        self._staging_plan = None
+        self._distdl_is_setup = False
+        self._input_tensor_structure = TensorStructure()
+
+    def _distdl_input_changed(self, input):
+        return self._input_tensor_structure != TensorStructure(input[0])
+
+    def _slab_views(self, padded_shape):
+        """Ghost and bulk buffers of the halo layer as ``[dim][side]`` tables."""
+        layer = self.halo_layer
+        if layer.slices is None:
+            SliceTable = self._distdl_backend.functional.halo_exchange.SliceTable
+            layer.slices = SliceTable(layer._assemble_slices(padded_shape, layer.recv_buffer_shape,
+                                                             layer.send_buffer_shape))
+            layer.buffers = layer.allocate_halo_exchange_buffers(layer.buffer_manager, layer.slices,
+                                                                 layer.recv_buffer_shape, layer.send_buffer_shape,
+                                                                 self._input_tensor_structure.dtype)
+        ghost, bulk = [], []
+        for i in range(len(padded_shape)):
+            lbs, lgs, rbs, rgs = layer.slices[i]
+            lbb, lgb, rbb, rgb = layer.buffers[i]
+
+            def view(buf, sl):
+                return None if buf is None else buf.get_view(compute_nd_slice_shape(sl))
+            ghost.append([view(lgb, lgs), view(rgb, rgs)])
+            bulk.append([view(lbb, lbs), view(rbb, rbs)])
+        return ghost, bulk
+
+    def stage_input(self, input):
+        """Padded, exchanged and cropped input of the local convolution."""
+        total_padding = self.local_padding + self.halo_shape
+        transport = self.P_x._world.transport
+        if total_padding.sum() == 0 and self.P_x.size == 1:
+            return input
+        if getattr(transport, "ghosts_preloaded", False):
+            # The four pooled halo buffers are shared by all dimensions
+            # (reference buffer_allocator.py:69-74), so a fused pass over all
+            # dimensions needs its own slab per (dimension, side).
+            ghost, bulk = self._fused_slabs(input)
+            exchanged = _HaloStaging.apply(input, self._staging_plan, ghost, bulk)
+        else:
+            padded = _HaloStaging.apply(input, self._pad_only_plan, None, None)
+            exchanged = self.halo_layer(padded)
+        return exchanged[self.needed_slices]
+
+    def _fused_slabs(self, input):
+        plan = self._staging_plan
+        slabs = getattr(self, "_fused_slab_cache", None)
+        key = (tuple(input.shape), input.dtype)
+        if slabs is None or slabs[0] != key:
+            ghost, bulk = [], []
+            for d in range(plan.ndim):
+                grow, brow = [], []
+                for s in range(2):
+                    gs, bs = plan.slab_shape(d, s, "ghost"), plan.slab_shape(d, s, "bulk")
+                    grow.append(None if gs is None else torch.zeros(gs, dtype=input.dtype, device=input.device))
+                    brow.append(None if bs is None else torch.empty(bs, dtype=input.dtype, device=input.device))
+                ghost.append(grow)
+                bulk.append(brow)
+            slabs = self._fused_slab_cache = (key, ghost, bulk)
+        return slabs[1], slabs[2]
+
+    def forward(self, input):
+        if not self.P_x.active:
+            return input
+        weight = self.w_broadcast(self.weight)
+        bias = self.b_broadcast(self.bias) if self.use_bias else None
+        # The local convolution is the stock one the reference calls (:411).
+        return self._conv_fn(self.stage_input(input), weight, bias, stride=self.stride, padding=0,
+                             dilation=self.dilation, groups=self.groups)
+
+
+class DistributedFeatureConv1d(DistributedFeatureConvBase):
+    TorchConvType = torch.nn.Conv1d
+    num_dimensions = 1
+
+
+class DistributedFeatureConv2d(DistributedFeatureConvBase):
+    TorchConvType = torch.nn.Conv2d
+    num_dimensions = 2
+
+
+class DistributedFeatureConv3d(DistributedFeatureConvBase):
+    TorchConvType = torch.nn.Conv3d
+    num_dimensions = 3

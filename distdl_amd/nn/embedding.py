@@ -1,0 +1,131 @@
+"""DistributedEmbedding (reference: nn/embedding.py:12-246).
+
+The table is partitioned along the embedding dimension as in the reference
+(every id hits, :113-115); the lookup ``torch.nn.functional.embedding``
+(:244-246) is replaced by the HIP gather kernel.  ``vocab_shard=(lo, hi)`` is an
+extension for vocabulary-sharded tables: the local table then holds rows
+``lo..hi-1`` and ids outside that window produce zero rows.
+"""
+
+import torch
+
+from .. import hip_ops
+from ..utilities.slicing import compute_subshape
+from ..utilities.slicing import worker_layout
+from ..utilities.torch import zero_volume_tensor
+from .broadcast import Broadcast
+from .module import Module
+
+
+class _EmbeddingShard(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, weight, ids, lo, hi):
+        return hip_ops.embedding_gather(weight.detach(), ids, lo, hi)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        raise NotImplementedError("the backward pass of DistributedEmbedding is not part of this build")
+
+
+class DistributedEmbedding(Module):
+    r"""Lookup table of ``num_embeddings`` vectors of size ``embedding_dim``
+    whose last dimension is partitioned by the last dimension of ``P_x``.
+
+    Signature of the reference; ``max_norm`` (in-place renormalisation of the
+    table during the lookup) is refused, ``padding_idx``, ``scale_grad_by_freq``
+    and ``sparse`` only concern gradients and are stored.
+    """
+
+    def __init__(self, P_x, num_embeddings, embedding_dim, padding_idx=None,
+                 max_norm=None, norm_type=2., scale_grad_by_freq=False, sparse=False,
+                 _weight=None, _freeze=False, collect_state=False, device=None,
+                 dtype=None, scale_backward=None, vocab_shard=None):
+        super().__init__()
+        self.num_embeddings = num_embeddings
+        self.embedding_dim = embedding_dim
+        if padding_idx is not None:
+            if padding_idx > 0:
+                assert padding_idx < self.num_embeddings, 'Padding_idx must be within num_embeddings'
+            elif padding_idx < 0:
+                assert padding_idx >= -self.num_embeddings, 'Padding_idx must be within num_embeddings'
+                padding_idx = self.num_embeddings + padding_idx
+        if max_norm is not None:
+            raise NotImplementedError("max_norm renormalises the table in place; not part of this build")
+        if collect_state:
+            raise NotImplementedError("collect_state=True is not part of this build")
+        self.padding_idx = padding_idx
+        self.max_norm = max_norm
+        self.norm_type = norm_type
+        self.scale_grad_by_freq = scale_grad_by_freq
+        self.sparse = sparse
+        self.collect_state = collect_state
+        self.dtype = dtype
+        self.P_x = P_x
+        if not self.P_x.active:
+            return
+
+        if vocab_shard is None:
+            vocab_shard = (0, num_embeddings)
+        self.vocab_lo, self.vocab_hi = int(vocab_shard[0]), int(vocab_shard[1])
+        if not 0 <= self.vocab_lo <= self.vocab_hi <= num_embeddings:
+            raise ValueError(f"vocab_shard {vocab_shard} is not inside [0, {num_embeddings}]")
+        rows_local = self.vocab_hi - self.vocab_lo
+
+        # Workers with index 0 in every dimension but the last store the table.
+        weight_partition_shape = [1] * P_x.dim
+        weight_partition_shape[-1] = int(P_x.shape[-1])
+        index_weight = [slice(0, 1)] * P_x.dim
+        index_weight[-1] = slice(0, int(P_x.shape[-1]))
+        weight_workers = worker_layout(P_x.shape)[tuple(index_weight)].reshape(-1).tolist()
+        P_weight_base = P_x.create_partition_inclusive(weight_workers)
+        self.P_weight = P_weight_base.create_cartesian_topology_partition(weight_partition_shape)
+        P_weight_base.deactivate()
+        self.broadcast = Broadcast(self.P_weight, self.P_x, scale_backward=scale_backward)
+
+        embedding_dim_local = int(compute_subshape(P_x.shape[-1], P_x.index[-1], [embedding_dim])[0])
+        dev = P_x.device if device is None else device
+        if _weight is not None:
+            assert _weight.shape[-1] == embedding_dim_local
+            assert _weight.shape[-2] == rows_local
+            if self.P_weight.active:
+                self.weight = torch.nn.Parameter(_weight, requires_grad=not _freeze)
+        elif self.P_weight.active:
+            self.weight = torch.nn.Parameter(torch.empty((rows_local, embedding_dim_local), device=dev, dtype=dtype),
+                                             requires_grad=not _freeze)
+            self.reset_parameters()
+        else:
+            self.register_buffer('weight', zero_volume_tensor(device=dev, requires_grad=True, dtype=self.dtype))
+        self.weight_buffer = None
+
+    def reset_parameters(self, mean=0.0, std=1.0):
+        """Every storing worker draws its own columns (the reference draws the
+        whole table on the root worker and scatters it, :150-160)."""
+        if self.P_weight.active:
+            with torch.no_grad():
+                torch.nn.init.normal_(self.weight, mean=mean, std=std)
+        self._fill_padding_idx_with_zero()
+
+    def extra_repr(self) -> str:
+        return f'num_embeddings={self.num_embeddings}, embedding_dim={self.embedding_dim}'
+
+    def _fill_padding_idx_with_zero(self):
+        if self.padding_idx is not None and self.P_weight.active:
+            if self.vocab_lo <= self.padding_idx < self.vocab_hi:
+                with torch.no_grad():
+                    self.weight[self.padding_idx - self.vocab_lo].fill_(0)
+
+    def prefetch_weights(self):
+        if self.P_x.size == 1:
+            return
+        self.weight_buffer = self.broadcast(self.weight)
+
+    def forward(self, input):
+        if not self.P_x.active:
+            return zero_volume_tensor(device=self.P_x.device, dtype=self.dtype)
+        if self.weight_buffer is None:
+            weight = self.broadcast(self.weight)
+        else:
+            weight = self.weight_buffer
+            self.weight_buffer = None
+        return _EmbeddingShard.apply(weight, input, self.vocab_lo, self.vocab_hi)

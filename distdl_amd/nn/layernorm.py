@@ -1,0 +1,167 @@
+"""DistributedLayerNorm (reference: nn/layernorm.py:15-321).
+
+Constructor and ``forward`` signature are the reference's.  The arithmetic of
+the distributed branch (reference :295-309: local mean, all-reduce, local mean
+of squared deviations, all-reduce, normalise, affine -- six or more elementwise
+kernels and two collectives) runs here as two HIP kernels around ONE gather of
+per-row ``{mean, M2}`` pairs; the combination rule reproduces the reference's
+mean of local means and mean of local variances exactly.
+"""
+
+import numbers
+
+import numpy as np
+import torch
+
+from .. import hip_ops
+from ..utilities.slicing import compute_subshape
+from ..utilities.slicing import range_index
+from ..utilities.slicing import worker_layout
+from ..utilities.torch import zero_volume_tensor
+from .all_sum_reduce import AllSumReduce
+from .broadcast import Broadcast
+from .module import Module
+
+STATS_TAG = "layernorm_stats"
+
+
+class _LayerNormShard(torch.autograd.Function):
+    """Local shard of a layer norm whose statistics span ``P_reduce``."""
+
+    @staticmethod
+    def forward(ctx, input, weight, bias, P_reduce, part_cols, eps):
+        x = input.detach()
+        cols = int(part_cols[P_reduce.rank if P_reduce.active else 0])
+        x2d = x.reshape(-1, cols)
+        if x2d.shape[1] > 1 and x2d.stride(1) != 1:
+            x2d = x2d.contiguous()
+        stats = hip_ops.ln_partial_stats(x2d)
+        if len(part_cols) > 1:
+            gathered = P_reduce._world.transport.allgather(P_reduce, stats, tag=STATS_TAG)
+            gathered = gathered.contiguous()
+        else:
+            gathered = stats.unsqueeze(0)
+        gamma = None if weight is None else weight.detach().reshape(-1)
+        beta = None if bias is None else bias.detach().reshape(-1)
+        y = hip_ops.ln_normalize_affine(x2d, gathered, part_cols, gamma, beta, eps)
+        return y.view(input.shape)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        raise NotImplementedError("the backward pass of DistributedLayerNorm is not part of this build")
+
+
+class DistributedLayerNorm(Module):
+    r"""Layer normalisation over the last ``len(normalized_shape)`` dimensions of
+    a tensor partitioned by ``P_x``; those dimensions may themselves be
+    partitioned.
+
+    Parameters
+    ----------
+    P_x :
+        Partition of the input (and output) tensor.
+    normalized_shape :
+        Global extent(s) of the normalised dimensions.
+    elementwise_affine, eps :
+        As ``torch.nn.LayerNorm``.
+    collect_state, device, dtype, scale_backward :
+        Accepted for signature compatibility; ``collect_state=True`` (gathering
+        the parameters into the state dict) is not part of this build.
+    """
+
+    def __init__(self, P_x, normalized_shape, elementwise_affine=True, eps=1e-5,
+                 collect_state=False, device=None, dtype=None, scale_backward=None):
+        super().__init__()
+        self.P_x = P_x
+        if not self.P_x.active:
+            return
+        if collect_state:
+            raise NotImplementedError("collect_state=True is not part of this build")
+        if device is None:
+            device = P_x.device
+        self.eps = eps
+        self.elementwise_affine = elementwise_affine
+        self.collect_state = collect_state
+        self.dtype = dtype
+        if isinstance(normalized_shape, numbers.Integral):
+            normalized_shape = (normalized_shape,)
+        self.normalized_shape = tuple(int(n) for n in normalized_shape)
+        num_dim = len(self.normalized_shape)
+
+        # Dimensions the statistics run over, and the workers sharing them.
+        self.dim_reduce = tuple(range(P_x.dim))[-num_dim:]
+        self.allreduce = AllSumReduce(P_x, axes_reduce=self.dim_reduce)
+        self.dim_reduce_slice = slice(P_x.dim - num_dim, P_x.dim)
+        self.dim_bcast_slice = slice(0, P_x.dim - num_dim)
+        reduce_shape = np.asarray(P_x.shape[self.dim_reduce_slice]).astype(int)
+        self.num_reduce = int(np.prod(reduce_shape))
+
+        # Columns held by every worker of the reduction group, in group order.
+        self.part_cols = [int(np.prod(compute_subshape(reduce_shape, idx, self.normalized_shape)))
+                          for idx in range_index(reduce_shape)]
+        local_norm_shape = compute_subshape(reduce_shape, P_x.index[self.dim_reduce_slice], self.normalized_shape)
+
+        if self.elementwise_affine:
+            # Parameters live on the workers with index 0 in every dimension that
+            # is not normalised, and are broadcast along those dimensions.
+            weight_partition_shape = np.copy(P_x.shape)
+            weight_partition_shape[self.dim_bcast_slice] = 1
+            index = [0] * P_x.dim
+            for i in range(self.dim_reduce_slice.start, self.dim_reduce_slice.stop):
+                index[i] = slice(0, int(P_x.shape[i]))
+            storage_workers = worker_layout(P_x.shape)[tuple(index)].reshape(-1).tolist()
+            P_w_base = P_x.create_partition_inclusive(storage_workers)
+            P_w = P_w_base.create_cartesian_topology_partition(weight_partition_shape)
+            P_w_base.deactivate()
+            self.P_w = P_w
+            self.broadcast = Broadcast(P_w, P_x, scale_backward=scale_backward)
+
+            shape_local = [1] * P_x.dim
+            shape_local[self.dim_reduce_slice] = [int(n) for n in local_norm_shape]
+            if P_w.active:
+                self.weight = torch.nn.Parameter(torch.empty(tuple(shape_local), device=device, dtype=dtype))
+                self.bias = torch.nn.Parameter(torch.empty(tuple(shape_local), device=device, dtype=dtype))
+            else:
+                self.register_buffer('weight', zero_volume_tensor(device=device, requires_grad=True, dtype=dtype))
+                self.register_buffer('bias', zero_volume_tensor(device=device, requires_grad=True, dtype=dtype))
+            self.weight_buffer = None
+            self.bias_buffer = None
+        else:
+            self.register_parameter('weight', None)
+            self.register_parameter('bias', None)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        if self.elementwise_affine and self.P_w.active:
+            torch.nn.init.ones_(self.weight)
+            torch.nn.init.zeros_(self.bias)
+
+    def extra_repr(self) -> str:
+        return f'normalized_shape={self.normalized_shape}'
+
+    def prefetch_weights(self):
+        """Fetches the parameters ahead of ``forward`` (reference :249-263)."""
+        if self.P_x.size == 1 or not self.elementwise_affine:
+            return
+        self.weight_buffer = self.broadcast(self.weight)
+        self.bias_buffer = self.broadcast(self.bias)
+
+    def forward(self, input):
+        if not self.P_x.active:
+            return input
+        weight = bias = None
+        if self.elementwise_affine:
+            if self.weight_buffer is None:
+                weight = self.broadcast(self.weight)
+                bias = self.broadcast(self.bias)
+            else:
+                weight, bias = self.weight_buffer, self.bias_buffer
+                self.weight_buffer = self.bias_buffer = None
+        if input.dtype != torch.float32:
+            raise NotImplementedError(f"DistributedLayerNorm kernels are fp32 only, got {input.dtype}")
+        local_cols = int(np.prod(input.shape[self.dim_reduce_slice.start - self.P_x.dim:]))
+        mine = self.allreduce.P_allreduce.rank if self.num_reduce > 1 else 0
+        if local_cols != self.part_cols[mine]:
+            raise ValueError(f"input shard has {local_cols} normalised elements, the partition of "
+                             f"normalized_shape={self.normalized_shape} gives this worker {self.part_cols[mine]}")
+        return _LayerNormShard.apply(input, weight, bias, self.allreduce.P_allreduce, self.part_cols, self.eps)

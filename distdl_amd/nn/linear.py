@@ -1,0 +1,63 @@
+"""DistributedLinear (reference: nn/linear.py:11-108): broadcast x over the rows
+of the weight partition, apply the local ``[out/P_fo, in/P_fi]`` shard, sum-reduce
+the partial outputs.  The local apply (reference :103, ``self.sublinear(x)``) is
+the bf16 MFMA kernel."""
+
+__all__ = ["DistributedLinear"]
+
+import torch
+
+from .. import hip_ops
+from ..utilities.slicing import compute_subshape
+from .broadcast import Broadcast
+from .module import Module
+from .sum_reduce import SumReduce
+
+
+class _LinearShard(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        return hip_ops.linear_bf16(x.detach(), weight.detach(), None if bias is None else bias.detach())
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        raise NotImplementedError("the backward pass of the linear shard is not part of this build")
+
+
+def linear_shard(x, weight, bias):
+    """``x @ weight.T + bias`` on the HIP kernel (bf16 operands only)."""
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise NotImplementedError(f"the linear shard kernel is bf16 only (got x {x.dtype}, weight {weight.dtype}); "
+                                  "convert the layer with .to(torch.bfloat16)")
+    return _LinearShard.apply(x, weight, bias)
+
+
+class DistributedLinear(Module):
+    r"""Affine layer with ``P_x ~ 1 x P_fi``, ``P_y ~ 1 x P_fo`` and
+    ``P_w ~ P_fo x P_fi``; ``in_features`` / ``out_features`` are global."""
+
+    def __init__(self, P_x, P_y, P_w, in_features, out_features, bias=True):
+        super().__init__()
+        self.P_x = P_x
+        self.P_y = P_y
+        self.P_w = P_w
+        self.bias = bias
+        self.x_broadcast = Broadcast(self.P_x, self.P_w, preserve_batch=True)
+        if self.P_w.active:
+            local_in_features = compute_subshape(P_w.shape[1], P_w.index[1], in_features)
+            local_out_features = compute_subshape(P_w.shape[0], P_w.index[0], out_features)
+            # Only column 0 of the weight partition adds the bias, so that the
+            # sum-reduce counts it once.
+            bias = self.bias if (self.P_w.index[-1] == 0) else False
+            self.sublinear = torch.nn.Linear(int(local_in_features[0]), int(local_out_features[0]), bias=bias,
+                                             device=P_w.device)
+        self.y_sum_reduce = SumReduce(self.P_w, self.P_y, transpose_src=True, preserve_batch=True)
+
+    def forward(self, input):
+        if not (self.P_x.active or self.P_y.active or self.P_w.active):
+            return input
+        x = self.x_broadcast(input)
+        if self.P_w.active:
+            x = linear_shard(x, self.sublinear.weight, self.sublinear.bias)
+        return self.y_sum_reduce(x)

@@ -1,0 +1,217 @@
+/*
+ * distdl_hip.h -- C ABI of libdistdl_hip.so (gfx950 / MI355X).
+ *
+ * One rank's local share of the DistDL data-parallel hot path: the strided
+ * pack / unpack copies of Repartition and HaloExchange, and the local-shard
+ * compute of DistributedLayerNorm, DistributedEmbedding and DistributedLinear.
+ *
+ * Conventions (every entry point):
+ *   - plain pointers and sizes only; every pointer named "device" is a device
+ *     address owned by the caller, every other pointer is host memory that is
+ *     only read during the call;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); work
+ *     is enqueued asynchronously, nothing synchronises, nothing allocates;
+ *   - the return value is 0 on success, a positive hipError_t if the runtime
+ *     refused a launch, or a negative DDL_E_* code for a rejected argument;
+ *     ddl_last_error() gives the message of the calling thread's last failure;
+ *   - shapes, starts and strides are int64 counts of ELEMENTS, row-major order
+ *     of dimensions (dimension 0 slowest) unless strides say otherwise.
+ *
+ * Citations are paths below the reference's src/distdl/ (or tests/, examples/).
+ */
+#ifndef DISTDL_HIP_H
+#define DISTDL_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DDL_MAX_DIMS 8
+
+#define DDL_E_ARG      (-1)  /* null pointer, negative size, bad enum        */
+#define DDL_E_DIMS     (-2)  /* ndim outside [1, DDL_MAX_DIMS]               */
+#define DDL_E_ALIGN    (-3)  /* pointer not aligned to the element size      */
+#define DDL_E_SHAPE    (-4)  /* box outside its tensor / inconsistent shape  */
+#define DDL_E_UNSUPP   (-5)  /* valid request this build does not implement  */
+
+/* Library identification: "distdl_hip <version> gfx950". */
+const char* ddl_version(void);
+
+/* Message for the last non-zero return on the calling thread ("" if none). */
+const char* ddl_last_error(void);
+
+/* ------------------------------------------------------------------------ *
+ * Box copies (Repartition / HaloExchange pack, unpack, self-copy)
+ * ------------------------------------------------------------------------ */
+
+/* One rectangular box copied between two strided device tensors.  `src` and
+ * `dst` point at the FIRST element of the box on each side. */
+typedef struct ddl_box {
+    const void* src;                   /* device */
+    void*       dst;                   /* device */
+    int32_t     ndim;                  /* 1..DDL_MAX_DIMS */
+    int32_t     reserved;
+    int64_t     shape[DDL_MAX_DIMS];
+    int64_t     src_stride[DDL_MAX_DIMS];
+    int64_t     dst_stride[DDL_MAX_DIMS];
+} ddl_box_t;
+
+#define DDL_OP_COPY 0   /* dst  = src                                          */
+#define DDL_OP_ADD  1   /* dst += src  (needs `dtype`; boxes must not alias)   */
+
+#define DDL_DT_BITS 0   /* opaque elements of elem_size bytes (copy only)      */
+#define DDL_DT_F32  1
+#define DDL_DT_F64  2
+#define DDL_DT_BF16 3
+#define DDL_DT_F16  4
+
+/* Copies (or accumulates) `nbox` boxes in as few launches as possible (16
+ * boxes per launch).  Boxes of one call must not overlap each other on the
+ * destination side.  Zero-volume boxes are skipped.
+ *
+ * Replaces the strided self-copy of Repartition,
+ *   backends/mpi_numpy/functional/repartition.py:179-190 (np.copyto(output[ysl], input[xsl])),
+ *   backends/nccl_cupy/functional/repartition.py:186,
+ * and, with DDL_OP_ADD, the adjoint accumulation of HaloExchange,
+ *   backends/mpi_numpy/functional/halo_exchange.py:138,140 (grad_output[lbs] += lbb). */
+int ddl_copy_boxes(const ddl_box_t* boxes, int nbox, int elem_size,
+                   int op, int dtype, void* stream);
+
+/* Pack: for b in [0,nbox): bufs[b] (contiguous, C order, shape box_shape[b])
+ *       = tensor[box_start[b] : box_start[b]+box_shape[b]].
+ * `tensor_strides` are the element strides of the (possibly non-contiguous)
+ * source tensor whose extent is `tensor_shape`.  box_start / box_shape are
+ * [nbox][ndim] row-major.  bufs[b] may be NULL to skip a box.
+ *
+ * Replaces  np.copyto(xfer_buff, input.detach()[sl].cpu().numpy())
+ *   backends/mpi_numpy/functional/repartition.py:158-171 (forward), :300-312 (adjoint),
+ *   xfer_buff.copy_(input.detach()[sl])  backends/nccl_cupy/functional/repartition.py:164,
+ * and the halo bulk-slab pack
+ *   backends/mpi_numpy/functional/halo_exchange.py:50-53 (forward), :115-119 (adjoint). */
+int ddl_pack_boxes(const void* tensor, const int64_t* tensor_shape,
+                   const int64_t* tensor_strides, int ndim, int elem_size,
+                   int nbox, const int64_t* box_start, const int64_t* box_shape,
+                   void* const* bufs, void* stream);
+
+/* Unpack: tensor[box_start[b] : +box_shape[b]] (op)= bufs[b]; the mirror of
+ * ddl_pack_boxes.  op = DDL_OP_COPY or DDL_OP_ADD (then `dtype` != DDL_DT_BITS).
+ *
+ * Replaces  np.copyto(output[sl], xfer_buff)
+ *   backends/mpi_numpy/functional/repartition.py:192-208 (forward), :335-349 (adjoint),
+ *   output[sl] = xfer_buff.detach().clone()  backends/nccl_cupy/functional/repartition.py:205,
+ * and the halo ghost-slab unpack
+ *   backends/mpi_numpy/functional/halo_exchange.py:70-74 (forward), :136-140 (adjoint, add). */
+int ddl_unpack_boxes(void* tensor, const int64_t* tensor_shape,
+                     const int64_t* tensor_strides, int ndim, int elem_size,
+                     int nbox, const int64_t* box_start, const int64_t* box_shape,
+                     const void* const* bufs, int op, int dtype, void* stream);
+
+/* Sets every element of each box of `tensor` to zero bits.
+ * Replaces  grad_output[lgs] = 0.0  backends/mpi_numpy/functional/halo_exchange.py:116,119
+ * and the zero initialisation of the Repartition output, repartition.py:175-177. */
+int ddl_zero_boxes(void* tensor, const int64_t* tensor_shape,
+                   const int64_t* tensor_strides, int ndim, int elem_size,
+                   int nbox, const int64_t* box_start, const int64_t* box_shape,
+                   void* stream);
+
+/* ------------------------------------------------------------------------ *
+ * Fused halo staging: zero-pad + ghost fill + send-slab pack in one pass
+ * ------------------------------------------------------------------------ */
+
+/* Writes the padded, exchanged tensor `xpad` (contiguous, shape
+ * x_shape[d] + pad[d][0] + pad[d][1]) from the local shard `x` (contiguous,
+ * shape x_shape) and, in the same pass, the send slabs.
+ *
+ *   pad   [ndim][2]  total padding = explicit zero padding + halo width
+ *   recv  [ndim][2]  ghost (receive) widths, left/right, in xpad coordinates
+ *   send  [ndim][2]  bulk  (send)    widths, left/right
+ *   ghost_bufs [ndim][2]  contiguous received slabs (NULL where width is 0)
+ *   bulk_bufs  [ndim][2]  contiguous slabs to send   (NULL where width is 0)
+ *
+ * Slab geometry is that of HaloExchange._assemble_slices, nn/halo_exchange.py:37-99:
+ * for exchange dimension i, dimensions j<i span all of xpad, j==i the
+ * ghost/bulk strip, j>i the bulk range [recv[j][0], size-recv[j][1]).
+ * The result equals F.pad (nn/conv_feature.py:400-407) followed by the
+ * dimension-ordered pack / unpack loop of
+ * backends/mpi_numpy/functional/halo_exchange.py:30-76 when the ghost slabs
+ * are those the neighbours send: an element lying in the ghost strips of
+ * several dimensions takes the slab of the highest such dimension, and a bulk
+ * slab of dimension i sees the ghosts of dimensions < i.
+ * Only when every ghost slab is available before the call (one-GPU stub
+ * exchange, or `ghost_bufs` all NULL for phase 0 of a real exchange). */
+int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x_shape,
+                          int ndim, int elem_size,
+                          const int64_t* pad, const int64_t* recv,
+                          const int64_t* send,
+                          const void* const* ghost_bufs, void* const* bulk_bufs,
+                          void* stream);
+
+/* ------------------------------------------------------------------------ *
+ * DistributedLayerNorm local shard (fp32)
+ * ------------------------------------------------------------------------ */
+
+/* Per-row partial statistics of the local shard x[rows, cols] (row stride
+ * `ld` elements): stats[r] = { mean_r, M2_r } with M2 = sum (x - mean_r)^2,
+ * fp32 accumulation.  One read of x.
+ *
+ * Replaces the local halves of DistributedLayerNorm._compute_mean / _compute_var,
+ *   nn/layernorm.py:230 (input.mean(dim, keepdim)) and :246-247. */
+int ddl_ln_partial_stats_f32(const float* x, int64_t rows, int64_t cols,
+                             int64_t ld, float* stats /*[rows][2]*/,
+                             void* stream);
+
+/* Combines the partial statistics of the `nparts` workers that share a row and
+ * normalises the local shard:
+ *   mean = (1/P) sum_p mean_p
+ *   var  = (1/P) sum_p (M2_p + n_p (mean_p - mean)^2) / n_p      (biased)
+ *   y    = (x - mean) / sqrt(var + eps) [* gamma + beta]
+ * which is the reference's mean-of-local-means / mean-of-local-variances,
+ *   nn/layernorm.py:230-233, :246-247, :298-302, :309,
+ * with the two all-reduces replaced by one gather of {mean, M2}.
+ *   part_stats [nparts][rows][2]  (this worker's own partials included)
+ *   part_cols  [nparts]           host array: columns n_p held by each worker
+ *   gamma/beta [cols] or NULL (both or neither)
+ *   mean_out/rstd_out [rows] or NULL: the combined statistics, for backward. */
+int ddl_ln_normalize_affine_f32(const float* x, int64_t rows, int64_t cols,
+                                int64_t ld, const float* part_stats,
+                                int nparts, const int64_t* part_cols,
+                                const float* gamma, const float* beta,
+                                float eps, float* y, int64_t ldy,
+                                float* mean_out, float* rstd_out,
+                                void* stream);
+
+/* ------------------------------------------------------------------------ *
+ * DistributedEmbedding shard gather
+ * ------------------------------------------------------------------------ */
+
+/* out[t, :] = (lo <= ids[t] < hi) ? weight[ids[t] - lo, :] : 0   for t < n_ids.
+ * `weight` is [hi-lo, dim] row-major with row stride `ldw`; rows are moved as
+ * opaque bytes (elem_size 1, 2, 4 or 8).  ids are int64 (ids_is_i64 = 1) or
+ * int32.  With lo = 0 and hi = num_embeddings this is
+ *   torch.nn.functional.embedding(input, weight)   nn/embedding.py:244-246;
+ * a narrower window is the vocabulary-sharded variant whose misses give zero
+ * rows.  An id outside [0, num_embeddings) is a caller error the kernel does
+ * not detect beyond the window test. */
+int ddl_embedding_gather(const void* weight, int64_t dim, int64_t ldw,
+                         int elem_size, const void* ids, int ids_is_i64,
+                         int64_t n_ids, int64_t lo, int64_t hi,
+                         void* out, void* stream);
+
+/* ------------------------------------------------------------------------ *
+ * DistributedLinear shard GEMM (bf16 in, fp32 accumulate, bf16 out)
+ * ------------------------------------------------------------------------ */
+
+/* y[M, N] = x[M, K] . w[N, K]^T + bias[N]   (bias may be NULL).
+ * x, w, y row-major with leading dimensions ldx, ldw, ldy (elements).
+ * Replaces  self.sublinear(x)  nn/linear.py:103  and
+ *   torch.nn.functional.linear(input, weight, bias)  nn/linear_ag.py:486. */
+int ddl_linear_bf16(const void* x, const void* w, const void* bias, void* y,
+                    int64_t M, int64_t N, int64_t K,
+                    int64_t ldx, int64_t ldw, int64_t ldy, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DISTDL_HIP_H */

@@ -1,0 +1,34 @@
+"""ORACLE -- test infrastructure, not product code.  Only tests/,
+__graft_entry__.smoke() and bench.py's cpu_baseline leg may import it.
+
+The local apply of the reference's linear layers (nn/linear.py:103,
+nn/linear_ag.py:486: torch.nn.functional.linear(input, weight, bias)) as
+y = x . w^T + b in fp32 (or fp64) on operands given as bf16 bit patterns.
+
+The reference's tests check only forward/adjoint consistency of these layers
+(tests/layers/test_linear.py:48-305), never forward values -- parity is
+unpinned by the reference; here it is pinned by torch.nn.functional.linear on
+CPU, by exact small-integer cases and by an fp64 evaluation.
+"""
+
+import numpy as np
+
+
+def bf16_bits_to_f32(bits):
+    return (np.asarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_bf16_bits(x):
+    """Round to nearest even, NaN -> 0x7FC0."""
+    u = np.asarray(x, dtype=np.float32).view(np.uint32)
+    rounded = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    return np.where(np.isnan(np.asarray(x, dtype=np.float32)), np.uint16(0x7FC0), rounded)
+
+
+def linear(x_bits, w_bits, bias_bits=None, dtype=np.float32):
+    x = bf16_bits_to_f32(x_bits).astype(dtype)
+    w = bf16_bits_to_f32(w_bits).astype(dtype)
+    y = x.reshape(-1, x.shape[-1]) @ w.T
+    if bias_bits is not None:
+        y = y + bf16_bits_to_f32(bias_bits).astype(dtype)
+    return y.reshape(x.shape[:-1] + (w.shape[0],))

