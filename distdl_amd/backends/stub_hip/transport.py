@@ -164,8 +164,14 @@ class LoopbackTransport:
         errors = [None] * world.size
 
         def body(rank):
+            import torch
             try:
-                results[rank] = fn(world.partition(rank))
+                # Backward passes of GPU tensors normally all run on the single
+                # autograd thread of the device; a rank blocking there for a
+                # message would stall every other rank.  With multithreading
+                # off, each rank's backward runs on its own thread.
+                with torch.autograd.set_multithreading_enabled(False):
+                    results[rank] = fn(world.partition(rank))
             except BaseException as exc:  # noqa: B902 - re-raised below
                 errors[rank] = exc
                 transport.mail.fail(exc)

@@ -114,6 +114,9 @@ class Repartition(Module):
 
         backend = self._distdl_backend
         self.input_tensor_structure = TensorStructure(input[0])
+        if self.P_x.active and len(input[0].shape) != len(self.P_x_shape):
+            raise ValueError(f"Input partition mush have same dimension "
+                             f"({len(self.P_x_shape)}) as input tensor rank ({len(input[0].shape)}).")
         self.global_input_tensor_structure = backend.assemble_global_tensor_structure(
             self.input_tensor_structure, self.P_x, self.P_union)
         x_global_shape = np.asarray(self.global_input_tensor_structure.shape).astype(int)
