@@ -119,6 +119,11 @@ class HaloExchangeFunction(torch.autograd.Function):
                 ghost_plan.pack(grad_output, [lgb, rgb])
                 ghost_plan.zero(grad_output)
             _swap(P_x, ctx.neighbor_ranks[i], lgb, rgb, lbb, rbb)
-            if lbb is not None or rbb is not None:
+            if lbb is not None and rbb is not None and slices[i][0][i].stop > slices[i][2][i].start:
+                # Narrow shards: the left and right bulk strips share elements, so
+                # the two accumulations must not run in one launch.
+                bulk_plan.unpack(grad_output, [lbb, None], accumulate=True)
+                bulk_plan.unpack(grad_output, [None, rbb], accumulate=True)
+            elif lbb is not None or rbb is not None:
                 bulk_plan.unpack(grad_output, [lbb, rbb], accumulate=True)
         return grad_output, None, None, None, None
