@@ -6,10 +6,17 @@
 // Host side: every box is rewritten in BYTES, unit dimensions are dropped,
 // dimensions that are contiguous on both sides are merged, and the widest
 // power-of-two vector (<= 16 B) that divides the innermost run, both base
-// addresses and every remaining stride is chosen.  Device side: one workgroup
-// moves a tile of 256 x 4 vectors of one box; a vector's position is recovered
-// from its linear index with multiply-high divisions, so nothing but the box
-// table (passed by value as kernel arguments) is read besides the payload.
+// addresses and every remaining stride is chosen.  A box is then a matrix of
+// R rows (the flattened outer dimensions) by C vectors (the innermost one).
+//
+// Device side: a workgroup moves tiles of 1024 vectors shaped TR rows x TC
+// columns, TC the power of two covering C (at most 1024), so a vector's row and
+// column inside its tile are bit fields of its number; only the row needs
+// multiply-high divisions, and only when more than one outer dimension is left.
+// Workgroups are persistent (they stride over the tile sequence of the launch),
+// loads and stores are non-temporal, and nothing but the box table -- passed by
+// value as kernel arguments and read with scalar loads -- is read besides the
+// payload.
 #include "ddl_common.h"
 
 #include <algorithm>
@@ -18,34 +25,48 @@
 namespace ddl {
 namespace {
 
-constexpr int kMaxDevDims = 6;   // dimensions left after merging
+constexpr int kMaxDevDims = 5;   // outer dimensions left after merging (plus the innermost one)
 constexpr int kBatch = 16;       // boxes per launch (kernel-argument budget)
 constexpr int kThreads = 256;
 constexpr int kUnroll = 4;
 constexpr uint32_t kTileVecs = kThreads * kUnroll;
+constexpr uint32_t kTileLog = 10;  // log2(kTileVecs)
+static_assert((1u << kTileLog) == kTileVecs, "tile size must be 2^kTileLog");
+constexpr uint32_t kPersistentBlocks = 4096;  // 16 per CU
 constexpr uint64_t kMaxVecs = (1ull << 31) - kTileVecs;
 
 enum Op { OP_COPY = 0, OP_ADD = 1, OP_ZERO = 2 };
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
 struct DevDim {
     int64_t ss;  // source stride, bytes
     int64_t ds;  // destination stride, bytes
-    FastDiv fd;  // divide by the extent (in vectors for the innermost one)
+    FastDiv fd;  // divide by the extent
 };
 
 struct DevBox {
     const char* src;
     char* dst;
-    uint32_t total;       // vectors in the box
-    uint32_t nd;          // dimensions used
+    int64_t css, cds;     // column (innermost) strides, bytes
+    uint32_t cols;        // C: vectors per row
+    uint32_t rows;        // R: product of the outer extents
+    uint32_t tc_log;      // log2(TC)
+    uint32_t col_tiles;   // ceil(C / TC)
+    uint32_t nd;          // outer dimensions (0 = a single row)
     uint32_t vlog;        // log2(vector bytes)
-    uint32_t first_tile;  // first workgroup of this box in the launch
-    DevDim dim[kMaxDevDims];
+    uint32_t first_tile;  // first tile of this box in the launch
+    uint32_t ct_mul, ct_shr;  // multiply-high division by col_tiles
+    uint32_t pad;
+    DevDim dim[kMaxDevDims];  // outer dimensions, 0 = slowest
 };
 
 struct Batch {
     DevBox box[kBatch];
+    uint32_t first_tile[kBatch];  // copy of box[i].first_tile, contiguous for one wide scalar load
     uint32_t nbox;
+    uint32_t ntiles;
 };
 
 static_assert(sizeof(Batch) <= 4096, "box table must fit the kernel-argument segment");
@@ -117,69 +138,169 @@ __device__ inline V add_vectors(V d, V s) {
     return out;
 }
 
-template <int OP, typename T, typename V>
-__device__ inline void move_tile(const DevBox& bx, uint32_t tile) {
-    const uint32_t v0 = tile * kTileVecs + threadIdx.x;
+// The box table lives in the kernel-argument segment and is read with scalar
+// loads at compile-time offsets from the selected box; nothing of it is copied
+// into registers arrays, LDS or scratch.
+#if defined(__HIP_DEVICE_COMPILE__)
+typedef const Batch __attribute__((address_space(4))) * BatchPtr;
+typedef const DevBox __attribute__((address_space(4))) * DevBoxPtr;
+#else
+typedef const Batch* BatchPtr;
+typedef const DevBox* DevBoxPtr;
+#endif
+
+// ND = number of outer dimensions this instantiation decomposes (the table
+// entries beyond a box's own count hold extent 1 and stride 0).  Every table
+// field is fetched unconditionally at the top, so the scalar loads are issued
+// together and waited for once per tile.
+template <int OP, typename T, typename V, int ND>
+__device__ inline void move_tile(DevBoxPtr bx, uint32_t tile) {
+    const uint32_t col_tiles = bx->col_tiles;
+    const uint32_t tc_log = bx->tc_log;
+    const uint32_t ct_mul = bx->ct_mul, ct_shr = bx->ct_shr;
+    const uint32_t rows = bx->rows, cols = bx->cols;
+    const int64_t css = bx->css, cds = bx->cds;
+    int64_t dss[ND > 0 ? ND : 1], dds[ND > 0 ? ND : 1];
+    uint32_t ddiv[ND > 0 ? ND : 1], dmul[ND > 0 ? ND : 1], dshr[ND > 0 ? ND : 1];
+#pragma unroll
+    for (int d = 0; d < ND; ++d) {
+        dss[d] = bx->dim[d].ss;
+        dds[d] = bx->dim[d].ds;
+        ddiv[d] = bx->dim[d].fd.div;
+        dmul[d] = bx->dim[d].fd.mul;
+        dshr[d] = bx->dim[d].fd.shr;
+    }
+    const uint32_t row_tile = col_tiles == 1 ? tile : (__umulhi(tile, ct_mul) >> ct_shr);  // wave-uniform
+    const uint32_t col_tile = tile - row_tile * col_tiles;
+    const uint32_t row0 = row_tile << (kTileLog - tc_log);
+    const uint32_t col0 = col_tile << tc_log;
     int64_t soff[kUnroll], doff[kUnroll];
     bool live[kUnroll];
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-        uint32_t r = v0 + u * kThreads;
-        live[u] = r < bx.total;
-        int64_t so = 0, dof = 0;
-        for (int d = static_cast<int>(bx.nd) - 1; d > 0; --d) {
-            const uint32_t q = fd_div(r, bx.dim[d].fd);
-            const uint32_t idx = r - q * bx.dim[d].fd.div;
-            so += static_cast<int64_t>(idx) * bx.dim[d].ss;
-            dof += static_cast<int64_t>(idx) * bx.dim[d].ds;
-            r = q;
+    const uint32_t tc = 1u << tc_log;
+    const bool interior = col0 + tc <= cols && row0 + (kTileVecs >> tc_log) <= rows;   // wave-uniform
+    if (ND <= 1 && interior) {
+        // Whole tile inside the box and rows addressed by one stride: the four
+        // vectors of a lane differ by wave-uniform steps, so one position is
+        // computed and the others follow by addition.
+        const uint32_t j = threadIdx.x;
+        const uint32_t col = col0 + (j & (tc - 1u));
+        const uint32_t r = row0 + (j >> tc_log);
+        int64_t so = static_cast<int64_t>(col) * css, dof = static_cast<int64_t>(col) * cds;
+        if (ND > 0) {
+            so += static_cast<int64_t>(r) * dss[0];
+            dof += static_cast<int64_t>(r) * dds[0];
         }
-        so += static_cast<int64_t>(r) * bx.dim[0].ss;
-        dof += static_cast<int64_t>(r) * bx.dim[0].ds;
-        soff[u] = so;
-        doff[u] = dof;
+        // step of kThreads vectors: columns while they fit the tile row, rows after that
+        int64_t sstep[kUnroll], dstep[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const uint32_t jj = u * kThreads;                 // uniform
+            const uint32_t dc = jj & (tc - 1u), dr = jj >> tc_log;
+            sstep[u] = static_cast<int64_t>(dc) * css + (ND > 0 ? static_cast<int64_t>(dr) * dss[0] : 0);
+            dstep[u] = static_cast<int64_t>(dc) * cds + (ND > 0 ? static_cast<int64_t>(dr) * dds[0] : 0);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            soff[u] = so + sstep[u];
+            doff[u] = dof + dstep[u];
+            live[u] = true;
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const uint32_t j = threadIdx.x + u * kThreads;   // vector number inside the tile
+            uint32_t col = col0 + (j & (tc - 1u));
+            uint32_t r = row0 + (j >> tc_log);
+            live[u] = col < cols && r < rows;
+            // Vectors past the edge of the box are clamped onto its last column /
+            // row: they re-move an element another lane moves too, which keeps
+            // every load and store unconditional.
+            col = col < cols ? col : cols - 1;
+            r = r < rows ? r : rows - 1;
+            int64_t so = static_cast<int64_t>(col) * css, dof = static_cast<int64_t>(col) * cds;
+#pragma unroll
+            for (int d = ND - 1; d > 0; --d) {
+                const uint32_t q = ddiv[d] == 1 ? r : (__umulhi(r, dmul[d]) >> dshr[d]);
+                const uint32_t idx = r - q * ddiv[d];
+                so += static_cast<int64_t>(idx) * dss[d];
+                dof += static_cast<int64_t>(idx) * dds[d];
+                r = q;
+            }
+            if (ND > 0) {
+                so += static_cast<int64_t>(r) * dss[0];
+                dof += static_cast<int64_t>(r) * dds[0];
+            }
+            soff[u] = so;
+            doff[u] = dof;
+        }
     }
+    char* const dst = bx->dst;
     if constexpr (OP == OP_ZERO) {
         V z;
         __builtin_memset(&z, 0, sizeof(V));
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
-            if (live[u]) *reinterpret_cast<V*>(bx.dst + doff[u]) = z;
+        for (int u = 0; u < kUnroll; ++u) __builtin_nontemporal_store(z, reinterpret_cast<V*>(dst + doff[u]));
         return;
     }
+    const char* const src = bx->src;
     V val[kUnroll];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
-        if (live[u]) val[u] = *reinterpret_cast<const V*>(bx.src + soff[u]);
+    for (int u = 0; u < kUnroll; ++u) val[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(src + soff[u]));
     if constexpr (OP == OP_ADD) {
         if constexpr (sizeof(V) >= sizeof(T)) {
             V cur[kUnroll];
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u)
-                if (live[u]) cur[u] = *reinterpret_cast<const V*>(bx.dst + doff[u]);
+            for (int u = 0; u < kUnroll; ++u) cur[u] = *reinterpret_cast<const V*>(dst + doff[u]);
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u)
-                if (live[u]) val[u] = add_vectors<T, V>(cur[u], val[u]);
+            for (int u = 0; u < kUnroll; ++u) val[u] = add_vectors<T, V>(cur[u], val[u]);
         }
+        // An accumulation must happen exactly once per element.
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+            if (live[u]) *reinterpret_cast<V*>(dst + doff[u]) = val[u];
+        return;
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
-        if (live[u]) *reinterpret_cast<V*>(bx.dst + doff[u]) = val[u];
+    for (int u = 0; u < kUnroll; ++u) __builtin_nontemporal_store(val[u], reinterpret_cast<V*>(dst + doff[u]));
+}
+
+template <int OP, typename T, typename V>
+__device__ inline void move_tile_nd(DevBoxPtr bx, uint32_t tile, uint32_t nd) {
+    if (nd == 0)
+        move_tile<OP, T, V, 0>(bx, tile);
+    else if (nd == 1)
+        move_tile<OP, T, V, 1>(bx, tile);
+    else if (nd == 2)
+        move_tile<OP, T, V, 2>(bx, tile);
+    else
+        move_tile<OP, T, V, kMaxDevDims>(bx, tile);
 }
 
 template <int OP, typename T>
-__global__ __launch_bounds__(kThreads) void box_kernel(const Batch bt) {
-    const uint32_t b = blockIdx.x;
-    uint32_t bi = 0;
-    for (uint32_t i = 1; i < bt.nbox; ++i) bi = (b >= bt.box[i].first_tile) ? i : bi;
-    const DevBox& bx = bt.box[bi];
-    const uint32_t tile = b - bx.first_tile;
-    switch (bx.vlog) {
-        case 4: move_tile<OP, T, uint4>(bx, tile); break;
-        case 3: move_tile<OP, T, uint2>(bx, tile); break;
-        case 2: move_tile<OP, T, uint32_t>(bx, tile); break;
-        case 1: move_tile<OP, T, uint16_t>(bx, tile); break;
-        default: move_tile<OP, T, uint8_t>(bx, tile); break;
+__global__ __launch_bounds__(kThreads) void box_kernel(const Batch bt_by_value) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    BatchPtr bt = (BatchPtr)__builtin_amdgcn_kernarg_segment_ptr();
+#else
+    BatchPtr bt = &bt_by_value;
+#endif
+    // Persistent workgroups: each walks the launch's tile sequence with a
+    // stride of the grid, so a few thousand workgroups serve any volume.
+    const uint32_t nbox = bt->nbox;
+    const uint32_t ntiles = bt->ntiles;
+    for (uint32_t b = blockIdx.x; b < ntiles; b += gridDim.x) {
+        uint32_t bi = 0;
+#pragma unroll
+        for (uint32_t i = 1; i < kBatch; ++i) bi += (i < nbox && b >= bt->first_tile[i]) ? 1u : 0u;
+        DevBoxPtr bx = &bt->box[bi];
+        const uint32_t tile = b - bx->first_tile;
+        const uint32_t nd = bx->nd;
+        switch (bx->vlog) {
+            case 4: move_tile_nd<OP, T, u32x4>(bx, tile, nd); break;
+            case 3: move_tile_nd<OP, T, u32x2>(bx, tile, nd); break;
+            case 2: move_tile_nd<OP, T, uint32_t>(bx, tile, nd); break;
+            case 1: move_tile_nd<OP, T, uint16_t>(bx, tile, nd); break;
+            default: move_tile_nd<OP, T, uint8_t>(bx, tile, nd); break;
+        }
     }
 }
 
@@ -232,7 +353,7 @@ int lower_box(const ddl_box_t& in, int elem_size, bool has_src, std::vector<DevB
     m.back().n /= vbytes;
     m.back().ss = has_src ? vbytes : 0;
     m.back().ds = vbytes;
-    if (m.back().n == 1 && m.size() > 1) m.pop_back();
+    if (m.back().n == 1 && m.size() > 1) m.pop_back();  // element == vector: the next dimension becomes the columns
 
     // Split until the box fits 31-bit vector indices and kMaxDevDims dimensions.
     struct Piece {
@@ -249,11 +370,11 @@ int lower_box(const ddl_box_t& in, int elem_size, bool has_src, std::vector<DevB
             if (h.n > static_cast<int64_t>(kMaxVecs) || total * static_cast<uint64_t>(h.n) > kMaxVecs) too_big = true;
             if (!too_big) total *= static_cast<uint64_t>(h.n);
         }
-        if (too_big || static_cast<int>(p.d.size()) > kMaxDevDims) {
+        if (too_big || static_cast<int>(p.d.size()) > kMaxDevDims + 1) {
             // Cut the outermost dimension: in halves when it alone is large,
             // into single slices when there are too many dimensions.
             HostDim o = p.d.front();
-            if (static_cast<int>(p.d.size()) > kMaxDevDims || o.n == 1) {
+            if (static_cast<int>(p.d.size()) > kMaxDevDims + 1 || o.n == 1) {
                 for (int64_t i = 0; i < o.n; ++i) {
                     Piece q{std::vector<HostDim>(p.d.begin() + 1, p.d.end()), p.so + i * o.ss, p.dof + i * o.ds};
                     work.push_back(std::move(q));
@@ -270,16 +391,39 @@ int lower_box(const ddl_box_t& in, int elem_size, bool has_src, std::vector<DevB
             }
             continue;
         }
+        // Innermost dimension = columns, the rest = rows.
         DevBox db{};
         db.src = has_src ? static_cast<const char*>(in.src) + p.so : nullptr;
         db.dst = static_cast<char*>(in.dst) + p.dof;
-        db.total = static_cast<uint32_t>(total);
-        db.nd = static_cast<uint32_t>(p.d.size());
+        const HostDim inner = p.d.back();
+        db.cols = static_cast<uint32_t>(inner.n);
+        db.css = inner.ss;
+        db.cds = inner.ds;
+        db.rows = static_cast<uint32_t>(total / static_cast<uint64_t>(inner.n));
+        uint32_t tc_log = 0;
+        while (tc_log < kTileLog && (1u << tc_log) < db.cols) ++tc_log;
+        db.tc_log = tc_log;
+        db.col_tiles = (db.cols + (1u << tc_log) - 1) >> tc_log;
+        const FastDiv ct = make_fastdiv(db.col_tiles);
+        db.ct_mul = ct.mul;
+        db.ct_shr = ct.shr;
+        db.nd = static_cast<uint32_t>(p.d.size() - 1);
         db.vlog = vlog;
-        for (size_t d = 0; d < p.d.size(); ++d) {
-            db.dim[d].ss = p.d[d].ss;
-            db.dim[d].ds = p.d[d].ds;
-            db.dim[d].fd = make_fastdiv(static_cast<uint32_t>(p.d[d].n));
+        for (int d = 0; d < kMaxDevDims; ++d) {
+            // Unused entries (extent 1, stride 0) sit at the slow end so that the
+            // general instantiation may decompose all kMaxDevDims of them.
+            const int unused = kMaxDevDims - static_cast<int>(db.nd);
+            const bool general = db.nd > 2;
+            const int src_d = general ? d - unused : d;
+            if (src_d >= 0 && src_d < static_cast<int>(db.nd)) {
+                db.dim[d].ss = p.d[src_d].ss;
+                db.dim[d].ds = p.d[src_d].ds;
+                db.dim[d].fd = make_fastdiv(static_cast<uint32_t>(p.d[src_d].n));
+            } else {
+                db.dim[d].ss = 0;
+                db.dim[d].ds = 0;
+                db.dim[d].fd = make_fastdiv(1);
+            }
         }
         out->push_back(db);
     }
@@ -294,16 +438,20 @@ int launch_batches(const std::vector<DevBox>& boxes, hipStream_t stream) {
         uint64_t tiles = 0;
         uint32_t n = 0;
         while (i < boxes.size() && n < kBatch) {
-            const uint64_t t = (static_cast<uint64_t>(boxes[i].total) + kTileVecs - 1) / kTileVecs;
+            const uint64_t tr = kTileVecs >> boxes[i].tc_log;  // rows per tile
+            const uint64_t t = static_cast<uint64_t>(boxes[i].col_tiles) * ((boxes[i].rows + tr - 1) / tr);
             if (n > 0 && tiles + t > 0x7FFFFFFFull) break;
             bt.box[n] = boxes[i];
             bt.box[n].first_tile = static_cast<uint32_t>(tiles);
+            bt.first_tile[n] = static_cast<uint32_t>(tiles);
             tiles += t;
             ++n;
             ++i;
         }
         bt.nbox = n;
-        hipLaunchKernelGGL((box_kernel<OP, T>), dim3(static_cast<uint32_t>(tiles)), dim3(kThreads), 0, stream, bt);
+        bt.ntiles = static_cast<uint32_t>(tiles);
+        const uint32_t blocks = tiles < kPersistentBlocks ? static_cast<uint32_t>(tiles) : kPersistentBlocks;
+        hipLaunchKernelGGL((box_kernel<OP, T>), dim3(blocks), dim3(kThreads), 0, stream, bt);
         if (int rc = check_launch("box_kernel")) return rc;
     }
     return 0;
