@@ -16,227 +16,446 @@
 // source (a ghost slab, the shard, or zero) and is forwarded to the bulk slabs
 // that contain it.
 //
-// Mapping.  A wavefront owns kRows consecutive rows (all dimensions but the
-// last); row geometry is wave-uniform scalar work, the lanes walk the last
-// dimension, and the loads of all owned rows are issued before any store so
-// that enough bytes are in flight to cover HBM latency.  The innermost face
-// (a 1-element-wide slab at a 520-byte pitch in the 130^3 case) costs nothing
-// extra here because every row is streamed anyway.
+// Mapping.  Dimensions are named L (last, columns), M (second to last, rows)
+// and "outer" (the rest, a plane index).  A workgroup owns one plane and a
+// chunk of its rows: everything that depends on the outer coordinates only
+// (which slab or shard plane feeds the rows, which bulk slabs take them, all
+// base offsets) is wave-uniform scalar work done once per workgroup.  Each row
+// is then a run [wlo, whi) copied from one source with 16-byte vectors -- the
+// padded row starts are only 4-byte aligned, which gfx950 handles at nearly
+// full speed -- plus a few edge elements (padding zeros, last-dimension ghosts,
+// the run's remainder) handled one element per lane.  LPR lanes share a row, so
+// a wavefront covers 64/LPR rows per instruction and keeps kUnroll such row
+// groups in flight before the first store.
 #include "ddl_common.h"
+#include <cstdlib>
 
 namespace ddl {
 namespace {
 
-constexpr int HD = 6;       // tensor dimensions supported by the fused kernel
+constexpr int HD = 6;        // tensor dimensions supported by the fused kernel
 constexpr int kWave = 64;
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
-constexpr int kRows = 8;    // rows per wavefront
+constexpr int kUnroll = 4;   // row groups in flight per wavefront (lean path)
+constexpr int kGen = 1;      // row groups in flight in the general path
+
+struct Slab {
+    char* ptr;               // nullptr when the slab is absent
+    int64_t base;            // element offset of padded coordinate 0 (may be negative)
+    int64_t stride[HD - 1];  // element strides of dimensions 0..L-1 (dimension L has stride 1)
+};
 
 struct HaloArgs {
     const char* x;
     char* xpad;
-    const char* ghost[HD][2];
-    char* bulk[HD][2];
-    int64_t xstride[HD];        // elements
-    int64_t gstride[HD][2][HD]; // ghost slab strides of (dim, side), dims < L
-    int64_t bstride[HD][2][HD];
-    int64_t gbase[HD][2];       // offset correction, see slab_offset()
-    int64_t bbase[HD][2];
+    Slab ghost[HD][2];
+    Slab bulk[HD][2];
+    int64_t xstride[HD];
     uint32_t xs[HD], ps[HD], padl[HD];
     uint32_t recvl[HD], recvr[HD], sendl[HD], sendr[HD];
-    FastDiv fd[HD];             // division by ps[j]
-    int32_t nd;
-    uint32_t nrows;             // product of ps[0..nd-2]
+    FastDiv fd[HD];          // division by ps[j]
+    int32_t nd;              // >= 2
+    uint32_t nplanes;        // product of ps[0..nd-3]
+    uint32_t row_chunks;     // workgroups per plane
+    uint32_t rows_per_block;
+    uint32_t max_vecs;       // vectors of the longest run of any row
+    uint32_t max_edge;       // single-element tasks per row, upper bound
 };
-static_assert(sizeof(HaloArgs) <= 3800, "halo arguments must fit the kernel-argument segment");
+static_assert(sizeof(HaloArgs) <= 3900, "halo arguments must fit the kernel-argument segment");
 
-struct RowInfo {
-    const char* mid;   // element w of the row is mid[w] for wlo <= w < whi
-    uint32_t wlo, whi;
-    uint32_t special;  // row touches a ghost or bulk strip of a dimension < L
+#if defined(__HIP_DEVICE_COMPILE__)
+typedef const HaloArgs __attribute__((address_space(4))) * ArgsPtr;
+typedef const Slab __attribute__((address_space(4))) * SlabPtr;
+#else
+typedef const HaloArgs* ArgsPtr;
+typedef const Slab* SlabPtr;
+#endif
+
+template <typename T, int N>
+struct VecType {
+    typedef T type __attribute__((ext_vector_type(N), aligned(sizeof(T))));
 };
-
-// Coordinates of a padded row in dimensions 0..L-1 (loops are fully unrolled so
-// that the coordinate array stays in registers).
-__device__ inline void row_coords(const HaloArgs& a, uint32_t row, uint32_t (&c)[HD]) {
-    const int L = a.nd - 1;
-    uint32_t r = row;
-#pragma unroll
-    for (int j = HD - 2; j > 0; --j) {
-        c[j] = 0;
-        if (j < L) {
-            const uint32_t q = fd_div(r, a.fd[j]);
-            c[j] = r - q * a.ps[j];
-            r = q;
-        }
-    }
-    c[0] = r;
-    c[HD - 1] = 0;
-}
-
 template <typename T>
-__device__ inline RowInfo classify(const HaloArgs& a, uint32_t row) {
-    const int L = a.nd - 1;
-    uint32_t c[HD];
-    row_coords(a, row, c);
-    int gh = -1, gside = 0;
-    bool inx = true;
-    uint32_t special = 0;
-    int64_t xoff = 0;
+struct VecType<T, 1> {
+    typedef T type;
+};
+
+// Offset of padded coordinates (c[0..M-1], h, w) inside a slab.
+__device__ inline int64_t slab_offset(SlabPtr b, const uint32_t (&c)[HD], int M, uint32_t h, uint32_t w) {
+    int64_t off = b->base + static_cast<int64_t>(h) * b->stride[M] + w;
 #pragma unroll
-    for (int j = 0; j < HD - 1; ++j) {
-        if (j >= L) break;
-        const uint32_t lo = a.recvl[j], hi = a.ps[j] - a.recvr[j];
-        if (c[j] < lo) {
-            gh = j;
-            gside = 0;
-        } else if (c[j] >= hi) {
-            gh = j;
-            gside = 1;
-        } else if (c[j] < lo + a.sendl[j] || c[j] >= hi - a.sendr[j]) {
-            special = 1;
-        }
-        const uint32_t xc = c[j] - a.padl[j];  // wraps when left of the shard
-        inx = inx && xc < a.xs[j];
-        xoff += static_cast<int64_t>(xc) * a.xstride[j];
-    }
-    RowInfo ri;
-    ri.special = special | (gh >= 0 ? 1u : 0u);
-    if (gh >= 0) {
-        int64_t off = a.gbase[gh][gside];
-#pragma unroll
-        for (int j = 0; j < HD - 1; ++j)
-            if (j < L) off += static_cast<int64_t>(c[j]) * a.gstride[gh][gside][j];
-        ri.mid = a.ghost[gh][gside] + off * static_cast<int64_t>(sizeof(T));
-        ri.wlo = a.recvl[L];
-        ri.whi = a.ps[L] - a.recvr[L];
-    } else if (inx) {
-        ri.mid = a.x + (xoff - static_cast<int64_t>(a.padl[L])) * static_cast<int64_t>(sizeof(T));
-        ri.wlo = a.padl[L];
-        ri.whi = a.padl[L] + a.xs[L];
-    } else {
-        ri.mid = nullptr;
-        ri.wlo = 0;
-        ri.whi = 0;
-    }
-    return ri;
+    for (int j = 0; j < HD - 2; ++j)
+        if (j < M) off += static_cast<int64_t>(c[j]) * b->stride[j];
+    return off;
 }
 
-// Forwards the row's values to the bulk slabs of dimensions < L containing it.
-template <typename T, int KW>
-__device__ inline void forward_row(const HaloArgs& a, uint32_t row, uint32_t w0, const T (&v)[KW]) {
-    const int L = a.nd - 1;
-    const int lane = threadIdx.x & (kWave - 1);
-    uint32_t c[HD];
-    row_coords(a, row, c);
-    const uint32_t blo = a.recvl[L], bhi = a.ps[L] - a.recvr[L];
-    bool inner_bulk = true;  // dimensions j > i (below L) inside their bulk range
+// Stores `val` (a vector of the row's run, or one edge element) into every
+// bulk slab of a dimension below L that contains position (c, h, w).
+template <typename T, typename V>
+__device__ inline void forward_below_L(ArgsPtr a, const uint32_t (&c)[HD], int M, uint32_t h, uint32_t w, bool lane_on,
+                                       V val) {
+    const uint32_t hlo = a->recvl[M], hhi = a->ps[M] - a->recvr[M];
+    // dimension M: the row's own strips; outer dimensions are unrestricted
 #pragma unroll
-    for (int i = HD - 2; i >= 0; --i) {
-        if (i >= L) continue;
-        const uint32_t lo = a.recvl[i], hi = a.ps[i] - a.recvr[i];
+    for (int s = 0; s < 2; ++s) {
+        SlabPtr b = &a->bulk[M][s];
+        if (b->ptr == nullptr) continue;                                   // scalar test
+        const uint32_t s0 = s == 0 ? hlo : hhi - a->sendr[M], s1 = s == 0 ? hlo + a->sendl[M] : hhi;
+        if (lane_on && h >= s0 && h < s1) *reinterpret_cast<V*>(reinterpret_cast<T*>(b->ptr) + slab_offset(b, c, M, h, w)) = val;
+    }
+    // outer dimension i: decided by the plane, and the row must be in the bulk range of M
+    const bool h_bulk = h >= hlo && h < hhi;
+    bool inner_bulk = true;   // outer dimensions above i inside their bulk range
+#pragma unroll
+    for (int i = HD - 3; i >= 0; --i) {
+        if (i >= M) continue;
+        const uint32_t lo = a->recvl[i], hi = a->ps[i] - a->recvr[i];
         if (inner_bulk) {
+#pragma unroll
             for (int s = 0; s < 2; ++s) {
-                const uint32_t s0 = s == 0 ? lo : hi - a.sendr[i];
-                const uint32_t s1 = s == 0 ? lo + a.sendl[i] : hi;
-                if (a.bulk[i][s] == nullptr || c[i] < s0 || c[i] >= s1) continue;
-                int64_t off = a.bbase[i][s];
-#pragma unroll
-                for (int j = 0; j < HD - 1; ++j)
-                    if (j < L) off += static_cast<int64_t>(c[j]) * a.bstride[i][s][j];
-                T* dst = reinterpret_cast<T*>(a.bulk[i][s]) + off;
-#pragma unroll
-                for (int k = 0; k < KW; ++k) {
-                    const uint32_t w = w0 + lane + k * kWave;
-                    if (w >= blo && w < bhi) dst[w] = v[k];
-                }
+                SlabPtr b = &a->bulk[i][s];
+                const uint32_t s0 = s == 0 ? lo : hi - a->sendr[i], s1 = s == 0 ? lo + a->sendl[i] : hi;
+                if (b->ptr == nullptr || c[i] < s0 || c[i] >= s1) continue;   // scalar test
+                if (lane_on && h_bulk) *reinterpret_cast<V*>(reinterpret_cast<T*>(b->ptr) + slab_offset(b, c, M, h, w)) = val;
             }
         }
         inner_bulk = inner_bulk && c[i] >= lo && c[i] < hi;
     }
 }
 
-template <typename T, int KW>
-__global__ __launch_bounds__(kBlock) void halo_pad_kernel(const HaloArgs a) {
-    const int L = a.nd - 1;
-    const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * kWavesPerBlock + threadIdx.x / kWave);
-    const uint32_t row0 = wave * kRows;
-    if (row0 >= a.nrows) return;
-    const uint32_t W = a.ps[L];
-    const uint32_t glo = a.recvl[L], ghi = W - a.recvr[L];
-    const T* gl = reinterpret_cast<const T*>(a.ghost[L][0]);
-    const T* gr = reinterpret_cast<const T*>(a.ghost[L][1]);
-    T* bl = reinterpret_cast<T*>(a.bulk[L][0]);
-    T* br = reinterpret_cast<T*>(a.bulk[L][1]);
+template <typename T, int LPR>
+__global__ __launch_bounds__(kBlock) void halo_pad_kernel(const HaloArgs args_by_value) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    ArgsPtr a = (ArgsPtr)__builtin_amdgcn_kernarg_segment_ptr();
+#else
+    ArgsPtr a = &args_by_value;
+#endif
+    constexpr int EPV = sizeof(T) >= 4 ? 16 / sizeof(T) : 1;   // elements per vector
+    typedef typename VecType<T, EPV>::type V;
+    constexpr int RPI = kWave / LPR;                            // rows per wavefront instruction
+    constexpr int kRowsPerPass = RPI * kWavesPerBlock;
 
-    RowInfo ri[kRows];
+    const int nd = a->nd;
+    const int L = nd - 1, M = nd - 2;
+    const uint32_t plane = blockIdx.x / a->row_chunks;          // scalar
+    const uint32_t chunk = blockIdx.x - plane * a->row_chunks;
+    const uint32_t W = a->ps[L], H = a->ps[M];
+    const uint32_t glo = a->recvl[L], ghi = W - a->recvr[L];
+    const uint32_t sl = a->sendl[L], sr = a->sendr[L];
+    const uint32_t hlo = a->recvl[M], hhi = H - a->recvr[M];
+
+    // ---- outer coordinates and what they decide (scalar) ----
+    uint32_t c[HD];
+    {
+        uint32_t r = plane;
 #pragma unroll
-    for (int i = 0; i < kRows; ++i) {
-        if (row0 + i < a.nrows) {
-            ri[i] = classify<T>(a, row0 + i);
-        } else {
-            ri[i].mid = nullptr;
-            ri[i].wlo = ri[i].whi = 0;
-            ri[i].special = 0;
+        for (int j = HD - 3; j > 0; --j) {
+            c[j] = 0;
+            if (j < M) {
+                const uint32_t n = a->ps[j];
+                const uint32_t q = n == 1 ? r : (__umulhi(r, a->fd[j].mul) >> a->fd[j].shr);
+                c[j] = r - q * n;
+                r = q;
+            }
+        }
+        c[0] = M > 0 ? r : 0;
+        c[HD - 2] = c[HD - 1] = 0;
+    }
+    const int64_t plane_row0 = static_cast<int64_t>(plane) * H;
+    bool in_x = true;
+    int64_t x_off = 0;
+    int gh = -1, gside = 0;
+#pragma unroll
+    for (int j = 0; j < HD - 2; ++j) {
+        if (j < M) {
+            const uint32_t lo = a->recvl[j], hi = a->ps[j] - a->recvr[j];
+            if (c[j] < lo) {
+                gh = j;
+                gside = 0;
+            } else if (c[j] >= hi) {
+                gh = j;
+                gside = 1;
+            }
+            const uint32_t xc = c[j] - a->padl[j];               // wraps when left of the shard
+            in_x = in_x && xc < a->xs[j];
+            x_off += static_cast<int64_t>(xc) * a->xstride[j];
+        }
+    }
+    // Row sources decided by the plane: an outer ghost slab, or the two ghost slabs of M.
+    const char* gh_ptr = nullptr;
+    int64_t gh_off = 0, gh_mstride = 0;
+    if (gh >= 0) {
+        SlabPtr g = &a->ghost[gh][gside];
+        gh_ptr = g->ptr;
+        gh_off = slab_offset(g, c, M, 0, 0);
+        gh_mstride = g->stride[M];
+    }
+    const char* gm_ptr[2];
+    int64_t gm_off[2], gm_mstride[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+        SlabPtr g = &a->ghost[M][s];
+        gm_ptr[s] = g->ptr;
+        gm_off[s] = slab_offset(g, c, M, 0, 0);
+        gm_mstride[s] = g->stride[M];
+    }
+    const T* gl = reinterpret_cast<const T*>(a->ghost[L][0].ptr);
+    const T* gr = reinterpret_cast<const T*>(a->ghost[L][1].ptr);
+    T* bl = reinterpret_cast<T*>(a->bulk[L][0].ptr);
+    T* br = reinterpret_cast<T*>(a->bulk[L][1].ptr);
+    const uint32_t n_bl = bl ? sl : 0u, n_br = br ? sr : 0u;
+    const uint32_t rl = a->recvl[L], rr = a->recvr[L];
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const uint32_t lc = lane & (LPR - 1);                        // this lane's position inside its row
+    const uint32_t sub = lane / LPR;                             // which of the wavefront's RPI rows
+    const uint32_t h_begin = chunk * a->rows_per_block;
+    const uint32_t h_end = h_begin + a->rows_per_block < H ? h_begin + a->rows_per_block : H;
+    const uint32_t xsM = a->xs[M], padM = a->padl[M], padL = a->padl[L], xsL = a->xs[L];
+    const int64_t xstrM = a->xstride[M];
+    const T* xbase = reinterpret_cast<const T*>(a->x);
+    T* obase = reinterpret_cast<T*>(a->xpad);
+    const uint32_t max_vecs = a->max_vecs, max_edge = a->max_edge;
+
+    // Does any bulk slab of an outer dimension take rows of this plane?  (scalar)
+    bool outer_forward = false;
+    {
+        bool inner_bulk = true;
+#pragma unroll
+        for (int i = HD - 3; i >= 0; --i) {
+            if (i >= M) continue;
+            const uint32_t lo = a->recvl[i], hi = a->ps[i] - a->recvr[i];
+            if (inner_bulk) {
+                if (a->bulk[i][0].ptr != nullptr && c[i] >= lo && c[i] < lo + a->sendl[i]) outer_forward = true;
+                if (a->bulk[i][1].ptr != nullptr && c[i] >= hi - a->sendr[i] && c[i] < hi) outer_forward = true;
+            }
+            inner_bulk = inner_bulk && c[i] >= lo && c[i] < hi;
+        }
+    }
+    // Rows [plain_lo, plain_hi) of a plain plane are shard rows that feed no
+    // slab below L: their source and destination are affine in the row number.
+    const bool plane_plain = in_x && gh < 0 && !outer_forward;
+    const uint32_t left_m = a->bulk[M][0].ptr ? hlo + a->sendl[M] : hlo;
+    const uint32_t right_m = a->bulk[M][1].ptr ? hhi - a->sendr[M] : hhi;
+    const uint32_t plain_lo = padM > left_m ? padM : left_m;
+    const uint32_t plain_hi = padM + xsM < right_m ? padM + xsM : right_m;
+    const uint32_t wave_s = __builtin_amdgcn_readfirstlane(wave);
+    constexpr uint32_t kRowsPerWave = RPI * kUnroll;
+
+    // The chunk's rows split into [h_begin, lean_lo) and [lean_hi, h_end), which
+    // take the general path, and the plain rows [lean_lo, lean_hi) between them.
+    uint32_t lean_lo = h_end, lean_hi = h_end;
+    if (plane_plain) {
+        lean_lo = plain_lo < h_begin ? h_begin : (plain_lo < h_end ? plain_lo : h_end);
+        lean_hi = plain_hi < lean_lo ? lean_lo : (plain_hi < h_end ? plain_hi : h_end);
+    }
+
+    // ---- lean path: groups of kRowsPerWave plain rows, dealt round-robin to the wavefronts ----
+    for (uint32_t wh0 = lean_lo + wave_s * kRowsPerWave; wh0 < lean_hi; wh0 += kWavesPerBlock * kRowsPerWave) {
+        {
+            const T* sp[kUnroll];
+            T* op[kUnroll];
+            int64_t rowi[kUnroll];
+            bool rv[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                uint32_t h = wh0 + u * RPI + sub;
+                rv[u] = h < lean_hi;
+                h = rv[u] ? h : lean_hi - 1;                       // rows past the range: loads stay valid, stores are masked
+                sp[u] = xbase + (x_off + static_cast<int64_t>(h - padM) * xstrM - static_cast<int64_t>(padL));
+                rowi[u] = plane_row0 + h;
+                op[u] = obase + rowi[u] * static_cast<int64_t>(W);
+            }
+            const uint32_t x_hi = padL + xsL;
+            const uint32_t nvx = xsL / EPV;
+            const uint32_t run_end = padL + nvx * EPV;
+            const uint32_t n_edge = padL + (W - run_end);
+            const uint32_t n_task = n_edge + n_bl + n_br;
+            // All loads of a step -- the vectors of the run and the single
+            // elements -- are issued before its first store.
+            for (uint32_t it = 0; it * LPR < nvx || it * LPR < n_task; ++it) {
+                V val[kUnroll];
+                const uint32_t vi = it * LPR + lc;
+                const bool act = vi < nvx;
+                const uint32_t wv = padL + (act ? vi : 0u) * EPV;
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) val[u] = *reinterpret_cast<const V*>(sp[u] + wv);
+
+                const uint32_t e = it * LPR + lc;
+                uint32_t w = 0;
+                int k = 3;
+                if (e < n_edge) {
+                    w = e < padL ? e : run_end + (e - padL);
+                    k = 0;
+                } else if (e < n_edge + n_bl) {
+                    w = glo + (e - n_edge);
+                    k = 1;
+                } else if (e < n_task) {
+                    w = ghi - sr + (e - n_edge - n_bl);
+                    k = 2;
+                }
+                const bool in_l = w < glo, in_r = w >= ghi;
+                const bool in_m = !in_l && !in_r && w >= padL && w < x_hi;
+                T ev[kUnroll];
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) {
+                    const T* p = xbase;
+                    p = in_m ? sp[u] + w : p;
+                    p = in_l ? gl + rowi[u] * rl + w : p;
+                    p = in_r ? gr + rowi[u] * rr + (w - ghi) : p;
+                    const T t = *p;
+                    ev[u] = (in_l || in_r || in_m) ? t : T(0);
+                }
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u)
+                    if (act && rv[u]) *reinterpret_cast<V*>(op[u] + wv) = val[u];
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) {
+                    if (k == 0 && rv[u]) op[u][w] = ev[u];
+                    if (k == 1 && rv[u]) bl[rowi[u] * sl + (w - glo)] = ev[u];
+                    if (k == 2 && rv[u]) br[rowi[u] * sr + (w - (ghi - sr))] = ev[u];
+                }
+            }
         }
     }
 
-    for (uint32_t w0 = 0; w0 < W; w0 += kWave * KW) {
-        T v[kRows][KW];
+    // ---- general path: the rows before and after the plain range, RPI rows per wavefront step ----
+#pragma unroll 1
+    for (int part = 0; part < 2; ++part) {
+        const uint32_t r0 = part == 0 ? h_begin : lean_hi;
+        const uint32_t r1 = part == 0 ? lean_lo : h_end;
+#pragma unroll 1
+        for (uint32_t wh0 = r0 + wave_s * RPI; wh0 < r1; wh0 += kWavesPerBlock * RPI) {
+            const int g = 0;
+            {
+            // ---- per lane: the rows it serves and the single source of each ----
+            const T* src[kGen];      // element w of the run is src[w]; nullptr = zeros
+            uint32_t wlo[kGen], whi[kGen], hh[kGen];
+            T* out[kGen];
 #pragma unroll
-        for (int i = 0; i < kRows; ++i) {
-            const uint32_t row = row0 + i;
+            for (int u = 0; u < kGen; ++u) {
+                uint32_t h = wh0 + (g * kGen + u) * RPI + sub;
+                // Rows past the range are clamped onto its last row: they redo it
+                // with identical values, which keeps every load unconditional.
+                h = h < r1 ? h : r1 - 1;
+                hh[u] = h;
+                const uint32_t xh = h - padM;
+                const T* p = nullptr;
+                uint32_t lo = glo, hi = ghi;                          // zero rows and ghost rows span the bulk range of L
+                if (in_x && xh < xsM) {
+                    p = xbase + (x_off + static_cast<int64_t>(xh) * xstrM - static_cast<int64_t>(padL));
+                    lo = padL;
+                    hi = padL + xsL;
+                }
+                if (gh_ptr) {
+                    p = reinterpret_cast<const T*>(gh_ptr) + (gh_off + static_cast<int64_t>(h) * gh_mstride);
+                    lo = glo;
+                    hi = ghi;
+                }
+                if (h < hlo && gm_ptr[0]) {
+                    p = reinterpret_cast<const T*>(gm_ptr[0]) + (gm_off[0] + static_cast<int64_t>(h) * gm_mstride[0]);
+                    lo = glo;
+                    hi = ghi;
+                }
+                if (h >= hhi && gm_ptr[1]) {
+                    p = reinterpret_cast<const T*>(gm_ptr[1]) + (gm_off[1] + static_cast<int64_t>(h) * gm_mstride[1]);
+                    lo = glo;
+                    hi = ghi;
+                }
+                src[u] = p;
+                wlo[u] = lo;
+                whi[u] = hi;
+                out[u] = obase + (plane_row0 + h) * static_cast<int64_t>(W);
+            }
+
+            // ---- the runs, one vector per lane and step ----
+            for (uint32_t v0 = 0; v0 < max_vecs; v0 += LPR) {
+                V val[kGen];
+                bool act[kGen];
 #pragma unroll
-            for (int k = 0; k < KW; ++k) {
-                const uint32_t w = w0 + lane + k * kWave;
-                T t = T(0);
-                if (row < a.nrows && w < W) {
-                    if (w < glo) {
-                        t = gl[static_cast<int64_t>(row) * a.recvl[L] + w];
-                    } else if (w >= ghi) {
-                        t = gr[static_cast<int64_t>(row) * a.recvr[L] + (w - ghi)];
-                    } else if (w >= ri[i].wlo && w < ri[i].whi) {
-                        t = reinterpret_cast<const T*>(ri[i].mid)[w];
+                for (int u = 0; u < kGen; ++u) {
+                    const uint32_t w = wlo[u] + (v0 + lc) * EPV;
+                    act[u] = w + EPV <= whi[u];
+                    const bool has = act[u] && src[u] != nullptr;
+                    const T* p = has ? src[u] + w : xbase;            // idle lanes read a valid dummy address
+                    const V t = *reinterpret_cast<const V*>(p);
+                    V z;
+                    __builtin_memset(&z, 0, sizeof(V));
+                    val[u] = has ? t : z;
+                }
+#pragma unroll
+                for (int u = 0; u < kGen; ++u) {
+                    const uint32_t w = wlo[u] + (v0 + lc) * EPV;
+                    if (act[u]) *reinterpret_cast<V*>(out[u] + w) = val[u];
+                }
+#pragma unroll
+                for (int u = 0; u < kGen; ++u) {
+                    const uint32_t w = wlo[u] + (v0 + lc) * EPV;
+                    forward_below_L<T, V>(a, c, M, hh[u], w, act[u], val[u]);
+                }
+            }
+
+            // ---- edge elements and the bulk strips of L, one element per lane ----
+            for (uint32_t e0 = 0; e0 < max_edge; e0 += LPR) {
+                T ev[kGen];
+                uint32_t ew[kGen];
+                int kind[kGen];                                    // 0 edge, 1 left strip, 2 right strip, 3 nothing
+#pragma unroll
+                for (int u = 0; u < kGen; ++u) {
+                    const int64_t row = plane_row0 + hh[u];
+                    const uint32_t run_end = wlo[u] + ((whi[u] - wlo[u]) / EPV) * EPV;   // first element after the vectors
+                    const uint32_t n_edge = wlo[u] + (W - run_end);                      // [0,wlo) and [run_end,W)
+                    const uint32_t e = e0 + lc;
+                    uint32_t w = 0;
+                    int k = 3;
+                    if (e < n_edge) {
+                        w = e < wlo[u] ? e : run_end + (e - wlo[u]);
+                        k = 0;
+                    } else if (e < n_edge + n_bl) {
+                        w = glo + (e - n_edge);
+                        k = 1;
+                    } else if (e < n_edge + n_bl + n_br) {
+                        w = ghi - sr + (e - n_edge - n_bl);
+                        k = 2;
                     }
+                    const bool in_l = w < glo, in_r = w >= ghi;
+                    const bool in_m = !in_l && !in_r && src[u] != nullptr && w >= wlo[u] && w < whi[u];
+                    const T* p = xbase;
+                    p = in_m ? src[u] + w : p;
+                    p = in_l ? gl + row * rl + w : p;
+                    p = in_r ? gr + row * rr + (w - ghi) : p;
+                    const T t = *p;
+                    ev[u] = (in_l || in_r || in_m) ? t : T(0);
+                    ew[u] = w;
+                    kind[u] = k;
                 }
-                v[i][k] = t;
-            }
-        }
 #pragma unroll
-        for (int i = 0; i < kRows; ++i) {
-            const uint32_t row = row0 + i;
-            if (row >= a.nrows) continue;
-            T* out = reinterpret_cast<T*>(a.xpad) + static_cast<int64_t>(row) * W;
-#pragma unroll
-            for (int k = 0; k < KW; ++k) {
-                const uint32_t w = w0 + lane + k * kWave;
-                if (w < W) {
-                    out[w] = v[i][k];
-                    if (bl && w >= glo && w < glo + a.sendl[L]) bl[static_cast<int64_t>(row) * a.sendl[L] + (w - glo)] = v[i][k];
-                    if (br && w >= ghi - a.sendr[L] && w < ghi)
-                        br[static_cast<int64_t>(row) * a.sendr[L] + (w - (ghi - a.sendr[L]))] = v[i][k];
+                for (int u = 0; u < kGen; ++u) {
+                    const int64_t row = plane_row0 + hh[u];
+                    const uint32_t w = ew[u];
+                    if (kind[u] == 0) out[u][w] = ev[u];
+                    if (kind[u] == 1) bl[row * sl + (w - glo)] = ev[u];
+                    if (kind[u] == 2) br[row * sr + (w - (ghi - sr))] = ev[u];
+                    // an edge element inside the bulk range of L also belongs to the slabs below L
+                    forward_below_L<T, T>(a, c, M, hh[u], w, kind[u] == 0 && w >= glo && w < ghi, ev[u]);
                 }
             }
-            if (ri[i].special) forward_row<T, KW>(a, row, w0, v[i]);
+            }
         }
     }
 }
 
 template <typename T>
-int launch_halo(const HaloArgs& a, hipStream_t s) {
-    const uint32_t waves = (a.nrows + kRows - 1) / kRows;
-    const uint32_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
-    const uint32_t W = a.ps[a.nd - 1];
-    if (W <= 64)
-        hipLaunchKernelGGL((halo_pad_kernel<T, 1>), dim3(blocks), dim3(kBlock), 0, s, a);
-    else if (W <= 128)
-        hipLaunchKernelGGL((halo_pad_kernel<T, 2>), dim3(blocks), dim3(kBlock), 0, s, a);
-    else if (W <= 192)
-        hipLaunchKernelGGL((halo_pad_kernel<T, 3>), dim3(blocks), dim3(kBlock), 0, s, a);
+int launch_halo(const HaloArgs& a, uint32_t lpr, hipStream_t s) {
+    const uint32_t blocks = a.nplanes * a.row_chunks;
+    if (lpr <= 16)
+        hipLaunchKernelGGL((halo_pad_kernel<T, 16>), dim3(blocks), dim3(kBlock), 0, s, a);
+    else if (lpr <= 32)
+        hipLaunchKernelGGL((halo_pad_kernel<T, 32>), dim3(blocks), dim3(kBlock), 0, s, a);
     else
-        hipLaunchKernelGGL((halo_pad_kernel<T, 4>), dim3(blocks), dim3(kBlock), 0, s, a);
+        hipLaunchKernelGGL((halo_pad_kernel<T, 64>), dim3(blocks), dim3(kBlock), 0, s, a);
     return check_launch("halo_pad_kernel");
 }
 
@@ -253,19 +472,26 @@ extern "C" int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x
         return fail(DDL_E_ARG, "halo: element size %d not in {1,2,4,8}", elem_size);
 
     // Leading dimensions that carry no padding and no exchange are folded into
-    // one (batch x channel in the convolution case).
-    int64_t xs[DDL_MAX_DIMS], pl[DDL_MAX_DIMS], pr[DDL_MAX_DIMS], rl[DDL_MAX_DIMS], rr[DDL_MAX_DIMS], sl[DDL_MAX_DIMS],
-        sr[DDL_MAX_DIMS];
-    int src_dim[DDL_MAX_DIMS];
+    // one (batch x channel in the convolution case); a 1-D tensor gets a unit
+    // row dimension in front.
+    int64_t xs[DDL_MAX_DIMS + 1], pl[DDL_MAX_DIMS + 1], pr[DDL_MAX_DIMS + 1], rl[DDL_MAX_DIMS + 1], rr[DDL_MAX_DIMS + 1],
+        sl[DDL_MAX_DIMS + 1], sr[DDL_MAX_DIMS + 1];
+    int src_dim[DDL_MAX_DIMS + 1];
     int nd = 0;
+    if (ndim == 1) {
+        xs[0] = 1;
+        pl[0] = pr[0] = rl[0] = rr[0] = sl[0] = sr[0] = 0;
+        src_dim[0] = -1;
+        nd = 1;
+    }
     for (int d = 0; d < ndim; ++d) {
         const int64_t v[7] = {x_shape[d], pad[2 * d], pad[2 * d + 1], recv[2 * d], recv[2 * d + 1], send[2 * d], send[2 * d + 1]};
         for (int q = 0; q < 7; ++q)
             if (v[q] < 0) return fail(DDL_E_ARG, "halo: negative geometry value in dim %d", d);
         const bool plain = v[1] == 0 && v[2] == 0 && v[3] == 0 && v[4] == 0 && v[5] == 0 && v[6] == 0;
-        const bool prev_plain = nd > 0 && pl[nd - 1] == 0 && pr[nd - 1] == 0 && rl[nd - 1] == 0 && rr[nd - 1] == 0 &&
-                                sl[nd - 1] == 0 && sr[nd - 1] == 0;
-        if (plain && prev_plain && d != ndim - 1) {
+        const bool prev_plain = nd > 0 && src_dim[nd - 1] >= 0 && pl[nd - 1] == 0 && pr[nd - 1] == 0 && rl[nd - 1] == 0 &&
+                                rr[nd - 1] == 0 && sl[nd - 1] == 0 && sr[nd - 1] == 0;
+        if (plain && prev_plain && d < ndim - 2) {
             xs[nd - 1] *= v[0];
             continue;
         }
@@ -279,24 +505,26 @@ extern "C" int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x
     a.nd = nd;
     a.x = static_cast<const char*>(x);
     a.xpad = static_cast<char*>(xpad);
+    const int L = nd - 1, M = nd - 2;
     int64_t ps[HD];
-    int64_t total = 1, nrows = 1;
+    int64_t total = 1, nplanes = 1;
     for (int j = 0; j < nd; ++j) {
         ps[j] = xs[j] + pl[j] + pr[j];
         if (rl[j] + sl[j] > ps[j] - rr[j] || rr[j] + sr[j] > ps[j] - rl[j])
             return fail(DDL_E_SHAPE, "halo: ghost+bulk widths exceed the padded extent %lld in dim %d", (long long)ps[j], src_dim[j]);
+        if (rl[j] > pl[j] || rr[j] > pr[j])
+            return fail(DDL_E_SHAPE, "halo: ghost width larger than the padding in dim %d", src_dim[j]);
         if (ps[j] >= (1ll << 31)) return fail(DDL_E_UNSUPP, "halo: padded extent too large");
         total *= ps[j];
-        if (j < nd - 1) nrows *= ps[j];
+        if (j < M) nplanes *= ps[j];
     }
     if (total == 0) return 0;
-    if (nrows >= (1ll << 31) - 4096) return fail(DDL_E_UNSUPP, "halo: more than 2^31 rows");
     if (!xpad) return fail(DDL_E_ARG, "halo: null output");
     int64_t xvol = 1;
     for (int j = 0; j < nd; ++j) xvol *= xs[j];
     if (xvol > 0 && !x) return fail(DDL_E_ARG, "halo: null input");
     if (!aligned_to(xpad, elem_size) || !aligned_to(x, elem_size)) return fail(DDL_E_ALIGN, "halo: tensor misaligned");
-    a.nrows = static_cast<uint32_t>(nrows);
+    if (xvol == 0) a.x = a.xpad;   // only ever used as a readable dummy address
     int64_t st = 1;
     for (int j = nd - 1; j >= 0; --j) {
         a.xstride[j] = st;
@@ -310,21 +538,21 @@ extern "C" int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x
         a.sendr[j] = static_cast<uint32_t>(sr[j]);
         a.fd[j] = make_fastdiv(static_cast<uint32_t>(ps[j] > 0 ? ps[j] : 1));
     }
-    const int L = nd - 1;
     for (int i = 0; i < nd; ++i) {
         for (int s = 0; s < 2; ++s) {
             const int d = src_dim[i];
-            const void* gb = ghost_bufs ? ghost_bufs[2 * d + s] : nullptr;
-            void* bb = bulk_bufs ? bulk_bufs[2 * d + s] : nullptr;
+            const void* gb = (ghost_bufs && d >= 0) ? ghost_bufs[2 * d + s] : nullptr;
+            void* bb = (bulk_bufs && d >= 0) ? bulk_bufs[2 * d + s] : nullptr;
             const int64_t gw = s == 0 ? rl[i] : rr[i];
             const int64_t bw = s == 0 ? sl[i] : sr[i];
             if (gw > 0 && !gb) return fail(DDL_E_ARG, "halo: ghost width %lld in dim %d side %d but no slab given", (long long)gw, d, s);
             if (!aligned_to(gb, elem_size) || !aligned_to(bb, elem_size)) return fail(DDL_E_ALIGN, "halo: slab misaligned");
-            a.ghost[i][s] = gw > 0 ? static_cast<const char*>(gb) : nullptr;
-            a.bulk[i][s] = bw > 0 ? static_cast<char*>(bb) : nullptr;
             // Slab extents: j < i full, j == i the strip, j > i the bulk range.
             for (int kind = 0; kind < 2; ++kind) {
+                Slab& sb = kind == 0 ? a.ghost[i][s] : a.bulk[i][s];
                 const int64_t width = kind == 0 ? gw : bw;
+                sb.ptr = nullptr;
+                if (width > 0) sb.ptr = kind == 0 ? const_cast<char*>(static_cast<const char*>(gb)) : static_cast<char*>(bb);
                 const int64_t strip0 = kind == 0 ? (s == 0 ? 0 : ps[i] - rr[i]) : (s == 0 ? rl[i] : ps[i] - rr[i] - sr[i]);
                 int64_t ext[HD], str[HD];
                 for (int j = 0; j < nd; ++j) ext[j] = j < i ? ps[j] : (j == i ? width : ps[j] - rl[j] - rr[j]);
@@ -335,16 +563,39 @@ extern "C" int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x
                 }
                 int64_t base = -strip0 * str[i];
                 for (int j = i + 1; j < nd; ++j) base -= rl[j] * str[j];
-                for (int j = 0; j < L; ++j) (kind == 0 ? a.gstride : a.bstride)[i][s][j] = str[j];
-                (kind == 0 ? a.gbase : a.bbase)[i][s] = base;
+                for (int j = 0; j < L; ++j) sb.stride[j] = str[j];
+                sb.base = base;
             }
         }
     }
+    // Work split: LPR lanes per row (a power of two covering the longest run in
+    // vectors, at most a wavefront); the rows of a plane are cut into about
+    // 64-row chunks, one workgroup each.
+    const int epv = elem_size >= 4 ? 16 / elem_size : 1;
+    const int64_t bulk_l = ps[L] - rl[L] - rr[L];
+    const int64_t longest = bulk_l > xs[L] ? bulk_l : xs[L];
+    const int64_t shortest = bulk_l < xs[L] ? bulk_l : xs[L];
+    a.max_vecs = static_cast<uint32_t>(longest / epv);
+    // edge tasks: what whole vectors of the shortest run leave uncovered, plus the bulk strips of L
+    a.max_edge = static_cast<uint32_t>(ps[L] - (shortest / epv) * epv + sl[L] + sr[L]);
+    uint32_t lpr = 16;
+    while (lpr < 64 && lpr < a.max_vecs) lpr *= 2;
+    const int64_t rows_per_pass = (64 / lpr) * kWavesPerBlock;
+    int64_t target_rows = 64;
+    if (const char* e = getenv("DDL_TUNE_HALO_ROWS")) target_rows = atoi(e);
+    int64_t chunks = (ps[M] + target_rows / 2) / target_rows;
+    if (chunks < 1) chunks = 1;
+    int64_t rpb = (ps[M] + chunks - 1) / chunks;
+    rpb = ((rpb + rows_per_pass - 1) / rows_per_pass) * rows_per_pass;
+    a.rows_per_block = static_cast<uint32_t>(rpb);
+    a.row_chunks = static_cast<uint32_t>((ps[M] + rpb - 1) / rpb);
+    if (nplanes * static_cast<int64_t>(a.row_chunks) >= (1ll << 31)) return fail(DDL_E_UNSUPP, "halo: too many workgroups");
+    a.nplanes = static_cast<uint32_t>(nplanes);
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (elem_size) {
-        case 1: return launch_halo<uint8_t>(a, s);
-        case 2: return launch_halo<uint16_t>(a, s);
-        case 4: return launch_halo<uint32_t>(a, s);
-        default: return launch_halo<uint64_t>(a, s);
+        case 1: return launch_halo<uint8_t>(a, lpr, s);
+        case 2: return launch_halo<uint16_t>(a, lpr, s);
+        case 4: return launch_halo<uint32_t>(a, lpr, s);
+        default: return launch_halo<uint64_t>(a, lpr, s);
     }
 }
