@@ -28,7 +28,6 @@
 // a wavefront covers 64/LPR rows per instruction and keeps kUnroll such row
 // groups in flight before the first store.
 #include "ddl_common.h"
-#include <cstdlib>
 
 namespace ddl {
 namespace {
@@ -581,8 +580,7 @@ extern "C" int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x
     uint32_t lpr = 16;
     while (lpr < 64 && lpr < a.max_vecs) lpr *= 2;
     const int64_t rows_per_pass = (64 / lpr) * kWavesPerBlock;
-    int64_t target_rows = 64;
-    if (const char* e = getenv("DDL_TUNE_HALO_ROWS")) target_rows = atoi(e);
+    const int64_t target_rows = 64;
     int64_t chunks = (ps[M] + target_rows / 2) / target_rows;
     if (chunks < 1) chunks = 1;
     int64_t rpb = (ps[M] + chunks - 1) / chunks;
