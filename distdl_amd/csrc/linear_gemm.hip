@@ -8,12 +8,15 @@
 // that each lane ends up with four consecutive n of one output row and can
 // store them as one 8-byte word.
 //
-//   workgroup  256 threads = 4 wavefronts (2 x 2), tile 256(m) x 256(n) x 64(k)
-//   wavefront  128 x 128 = 4 x 4 tiles of v_mfma_f32_32x32x16_bf16, 256 fp32
-//              accumulators per lane, one wavefront per SIMD
+//   workgroup  512 threads = 8 wavefronts (2 along m x 4 along n), tile
+//              256(m) x 256(n) x 64(k); two wavefronts share a SIMD so that one
+//              can issue MFMAs while the other waits for LDS
+//   wavefront  128(m) x 64(n) = 4 x 2 tiles of v_mfma_f32_32x32x16_bf16, 128 fp32
+//              accumulators per lane
 //   LDS        two stages of {w tile, x tile} = 2 x 64 KiB; rows are 128 B with
-//              the 16-byte chunk index XOR-ed by (row & 7) so that the 32 rows
-//              an operand fetch touches spread over all banks
+//              the 16-byte chunk index XOR-ed by ((row >> 1) & 7): the 16 lanes
+//              served per LDS cycle read 16 consecutive rows, and (row & 1,
+//              (row >> 1) & 7) is distinct for each, so they cover all 64 banks
 //   schedule   global loads of k-tile t+1 are issued before the MFMAs of tile
 //              t and written to the other LDS stage after them; one barrier
 //              per k-tile
@@ -29,13 +32,13 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 
 constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;
 constexpr int kTileBytes = BM * BK * 2;          // one operand tile, 32 KiB
 constexpr int kStageBytes = 2 * kTileBytes;      // w tile + x tile
 constexpr int kLdsBytes = 2 * kStageBytes;       // two stages
 constexpr int kXcds = 8;
 
-__device__ inline uint32_t lds_offset(int row, int chunk) { return row * (BK * 2) + ((chunk ^ (row & 7)) << 4); }
+__device__ inline uint32_t lds_offset(int row, int chunk) { return row * (BK * 2) + ((chunk ^ ((row >> 1) & 7)) << 4); }
 
 __device__ inline uint16_t f32_to_bf16_bits(float f) {
     uint32_t u = __float_as_uint(f);
@@ -46,17 +49,17 @@ __device__ inline uint16_t f32_to_bf16_bits(float f) {
 
 __device__ inline float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(static_cast<uint32_t>(b) << 16); }
 
-// Loads this thread's eight 16-byte chunks of one operand tile (rows row0..+255
+// Loads this thread's four 16-byte chunks of one operand tile (rows row0..+255
 // of a [rows_total, K] matrix, columns k0..k0+63).  Rows past the end repeat the
 // last valid row (their products are never stored); chunks past K read as zero.
 __device__ inline void load_tile(const uint16_t* __restrict__ g, int64_t ld, int64_t rows_total, int64_t row0, int64_t K,
-                                 int64_t k0, uint4 (&r)[8]) {
+                                 int64_t k0, uint4 (&r)[4]) {
     const int c = threadIdx.x & 7;
     const int rr = threadIdx.x >> 3;
     const int64_t k = k0 + c * 8;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        int64_t row = row0 + rr + 32 * i;
+    for (int i = 0; i < 4; ++i) {
+        int64_t row = row0 + rr + 64 * i;
         row = row < rows_total ? row : rows_total - 1;
         if (k < K)
             r[i] = *reinterpret_cast<const uint4*>(g + row * ld + k);
@@ -65,11 +68,11 @@ __device__ inline void load_tile(const uint16_t* __restrict__ g, int64_t ld, int
     }
 }
 
-__device__ inline void store_tile(char* lds, const uint4 (&r)[8]) {
+__device__ inline void store_tile(char* lds, const uint4 (&r)[4]) {
     const int c = threadIdx.x & 7;
     const int rr = threadIdx.x >> 3;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4*>(lds + lds_offset(rr + 32 * i, c)) = r[i];
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(lds + lds_offset(rr + 64 * i, c)) = r[i];
 }
 
 __global__ __launch_bounds__(kThreads) void linear_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
@@ -97,18 +100,19 @@ __global__ __launch_bounds__(kThreads) void linear_bf16_kernel(const uint16_t* _
 
     const int64_t m0 = static_cast<int64_t>(tm) * BM, n0 = static_cast<int64_t>(tn) * BN;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int wm = (wave & 1) * 128, wn = (wave >> 1) * 128;  // wavefront origin inside the tile
+    const int wm = (wave & 1) * 128, wn = (wave >> 1) * 64;   // wavefront origin inside the tile
     const int l32 = lane & 31, kg = lane >> 5;
 
-    floatx16 acc[4][4];  // [n sub-tile][m sub-tile]
+    constexpr int TN = 2, TM = 4;   // 32x32 sub-tiles of a wavefront along n and m
+    floatx16 acc[TN][TM];  // [n sub-tile][m sub-tile]
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+    for (int a = 0; a < TN; ++a)
 #pragma unroll
         for (int b = 0; b < 4; ++b)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
-    uint4 rw[8], rx[8];
+    uint4 rw[4], rx[4];
     const int64_t ktiles = (K + BK - 1) / BK;
     load_tile(w, ldw, N, n0, K, 0, rw);
     load_tile(x, ldx, M, m0, K, 0, rx);
@@ -126,17 +130,31 @@ __global__ __launch_bounds__(kThreads) void linear_bf16_kernel(const uint16_t* _
         }
         const char* sw = cur;
         const char* sx = cur + kTileBytes;
+        // Operand fragments are double-buffered: the LDS reads of k-step ks+1
+        // are issued before the MFMAs of k-step ks, so a wavefront does not
+        // stall on LDS latency between k-steps.
+        bf16x8 fa[2][TN], fb[2][TM];
+#pragma unroll
+        for (int a = 0; a < TN; ++a) fa[0][a] = *reinterpret_cast<const bf16x8*>(sw + lds_offset(wn + a * 32 + l32, kg));
+#pragma unroll
+        for (int b = 0; b < TM; ++b) fb[0][b] = *reinterpret_cast<const bf16x8*>(sx + lds_offset(wm + b * 32 + l32, kg));
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
-            bf16x8 fa[4], fb[4];
+            const int cb = ks & 1, nb = cb ^ 1;
+            const bool pre = ks + 1 < BK / 16;
+            // One LDS read of the next k-step is issued behind each MFMA of this
+            // one, so that LDS traffic is spread evenly instead of arriving in
+            // bursts that fill the LDS queues of all wavefronts at once.
 #pragma unroll
-            for (int a = 0; a < 4; ++a) fa[a] = *reinterpret_cast<const bf16x8*>(sw + lds_offset(wn + a * 32 + l32, ks * 2 + kg));
-#pragma unroll
-            for (int b = 0; b < 4; ++b) fb[b] = *reinterpret_cast<const bf16x8*>(sx + lds_offset(wm + b * 32 + l32, ks * 2 + kg));
-#pragma unroll
-            for (int a = 0; a < 4; ++a)
-#pragma unroll
-                for (int b = 0; b < 4; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[a], fb[b], acc[a][b], 0, 0, 0);
+            for (int i = 0; i < TN * TM; ++i) {
+                const int a = i / TM, b = i % TM;
+                acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cb][a], fb[cb][b], acc[a][b], 0, 0, 0);
+                if (pre && i < TN)
+                    fa[nb][i] = *reinterpret_cast<const bf16x8*>(sw + lds_offset(wn + i * 32 + l32, (ks + 1) * 2 + kg));
+                else if (pre && i < TN + TM)
+                    fb[nb][i - TN] = *reinterpret_cast<const bf16x8*>(sx + lds_offset(wm + (i - TN) * 32 + l32, (ks + 1) * 2 + kg));
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         if (more) {
             store_tile(nxt, rw);
@@ -148,7 +166,7 @@ __global__ __launch_bounds__(kThreads) void linear_bf16_kernel(const uint16_t* _
     // Epilogue.  Lane holds, per 32x32 tile, output row m = l32 and the columns
     // n = 8*g + 4*kg + {0,1,2,3} for g = 0..3 in acc[...][4*g + {0..3}].
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
+    for (int a = 0; a < TN; ++a) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const int64_t n = n0 + wn + a * 32 + 8 * g + 4 * kg;
