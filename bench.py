@@ -33,9 +33,18 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
-# HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (see profiles/); None until measured for a kernel.
-MEASURED_TRAFFIC_BYTES = {}
+# HBM bytes per launch (read + write) from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of these same workloads, each counter scaled by what it reads
+# for a plain 64 MiB device copy (FETCH_SIZE x1.9993, WRITE_SIZE x1.0000); the
+# summaries are profiles/*_hbm_traffic_pmc.txt.  layernorm is the mean of its two
+# kernels (stats 8 498 546 B, normalize 17 132 572 B), like its launch time.
+MEASURED_TRAFFIC_BYTES = {
+    "repartition": 134419452,
+    "layernorm": 12815559,
+    "embedding": 1210713945,
+    "linear": 1009567583,
+    "halo": 579156303,
+}
 
 
 def parse_args():
@@ -44,7 +53,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default=None, help="run a single workload (repartition, layernorm, embedding, linear, halo)")
+    ap.add_argument("--only", default=None, help="run a single workload (repartition, layernorm, embedding, linear, halo, calib)")
     ap.add_argument("--no-graph", action="store_true", help="launch on the stream instead of replaying a HIP graph")
     return ap.parse_args()
 
@@ -94,13 +103,15 @@ class Timed:
             torch.cuda.synchronize()
 
     def run(self, steps):
-        """Runs `steps` steps (rounded up to whole passes over the buffer sets);
-        returns (steps actually run, wall seconds, event seconds)."""
+        """Runs exactly `steps` steps: whole passes over the buffer sets (graph
+        replays when a graph was captured) and the remaining steps launched on
+        the stream.  Returns (steps, wall seconds, event seconds)."""
         torch = self.torch
         nsets = len(self.step_fns)
-        passes = (steps + nsets - 1) // nsets
+        passes, rest = divmod(steps, nsets)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
+        bind_stream(torch)
         t0 = time.perf_counter()
         e0.record()
         for _ in range(passes):
@@ -108,10 +119,13 @@ class Timed:
                 self.graph.replay()
             else:
                 self._run_sets()
+        for fns in self.step_fns[:rest]:
+            for fn in fns:
+                fn()
         e1.record()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
-        return passes * nsets, t1 - t0, e0.elapsed_time(e1) * 1e-3
+        return steps, t1 - t0, e0.elapsed_time(e1) * 1e-3
 
 
 def measure(torch, name, step_fns, launches_per_step, steps, warmup, use_graph):
@@ -276,6 +290,23 @@ def build_halo(torch, lib, _lib, nsets):
     return steps, keep, 562531072
 
 
+def build_calib(torch, lib, _lib, nsets):
+    """Counter calibration: a plain contiguous device-to-device copy of 64 MiB
+    (torch's own copy kernel), so that FETCH_SIZE / WRITE_SIZE readings of the
+    kernels above can be scaled by what the same counters read for a known
+    amount of traffic."""
+    keep, steps = [], []
+    for s in range(nsets):
+        a = torch.empty(64 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        b = torch.empty_like(a)
+        keep.append((a, b))
+
+        def copy(a=a, b=b):
+            b.copy_(a)      # torch's current stream is the one STREAM[0] is bound to
+        steps.append([copy])
+    return steps, keep, 2 * (64 << 20)
+
+
 # ----------------------------------------------------------------------------
 # CPU baseline (the oracle, i.e. a port of the reference's mpi_numpy path)
 # ----------------------------------------------------------------------------
@@ -332,8 +363,9 @@ def main():
         "embedding": (build_embedding, 4, 1, "hbm"),
         "linear": (build_linear, 4, 1, "mfma"),
         "halo": (build_halo, 4, 1, "hbm"),
+        "calib": (build_calib, 4, 1, "hbm"),     # only with --only calib
     }
-    names = [args.only] if args.only else list(builders)
+    names = [args.only] if args.only else [n for n in builders if n != "calib"]
     results = {}
     for name in names:
         build, nsets, launches, bound = builders[name]
