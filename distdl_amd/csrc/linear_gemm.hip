@@ -9,21 +9,33 @@
 // store them as one 8-byte word.
 //
 //   workgroup  512 threads = 8 wavefronts (2 along m x 4 along n), tile
-//              256(m) x 256(n) x 64(k); two wavefronts share a SIMD so that one
-//              can issue MFMAs while the other waits for LDS
+//              256(m) x 256(n); two wavefronts share a SIMD so that one can
+//              issue MFMAs while the other waits
 //   wavefront  128(m) x 64(n) = 4 x 2 tiles of v_mfma_f32_32x32x16_bf16, 128 fp32
 //              accumulators per lane
-//   LDS        two stages of {w tile, x tile} = 2 x 64 KiB; rows are 128 B with
-//              the 16-byte chunk index XOR-ed by ((row >> 1) & 7): the 16 lanes
-//              served per LDS cycle read 16 consecutive rows, and (row & 1,
-//              (row >> 1) & 7) is distinct for each, so they cover all 64 banks
-//   schedule   global loads of k-tile t+1 are issued before the MFMAs of tile
-//              t and written to the other LDS stage after them; one barrier
-//              per k-tile
+//   LDS        five stages of {w tile, x tile}, each tile 256 rows x 32 k =
+//              16 KiB (160 KiB in all).  Rows are 64 B; the 16-byte chunk index
+//              is XOR-ed with ((row >> 2) & 3): the 16 lanes served per LDS
+//              cycle read 16 consecutive rows, and (row & 3, (row >> 2) & 3) is
+//              distinct for each, so they cover all 64 banks
+//   global     tiles go from global memory straight into LDS
+//              (global_load_lds_dwordx4: each wavefront instruction fills 1 KiB
+//              = 16 rows); no staging registers, no LDS stores.  Tile t+4 is
+//              requested while tile t is multiplied and has to be complete one
+//              tile before its turn, so a request has three k-tiles of MFMA
+//              time to arrive
+//   schedule   per k-tile: wait for own requests of tile t+1, barrier, then
+//              2 x 8 MFMAs with one LDS fragment read issued behind each (the
+//              fragments of the next k-step, crossing into tile t+1) and the
+//              request instructions of tile t+4 spread between them
+//   epilogue   bias add and bf16 rounding in registers, then each wavefront
+//              transposes its block through LDS so that rows of y are written
+//              in 16-byte pieces, whole 128-byte lines per instruction
 //   launch     workgroup ids are regrouped so that the 32 workgroups resident
 //              on one XCD cover a compact patch of the tile grid and share
 //              their operand panels in that XCD's L2
 #include "ddl_common.h"
+#include <type_traits>
 
 namespace ddl {
 namespace {
@@ -31,14 +43,13 @@ namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 
-constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int kThreads = 512;
-constexpr int kTileBytes = BM * BK * 2;          // one operand tile, 32 KiB
-constexpr int kStageBytes = 2 * kTileBytes;      // w tile + x tile
-constexpr int kLdsBytes = 2 * kStageBytes;       // two stages
+constexpr int BM = 256, BN = 256, BK = 32;
+constexpr int kStages = 5;
+constexpr int kTileBytes = BM * BK * 2;              // one operand tile, 16 KiB
+constexpr int kStageBytes = 2 * kTileBytes;          // w tile + x tile
+constexpr int kLdsBytes = kStages * kStageBytes;     // 160 KiB: all of a CU's LDS
+constexpr int kAhead = kStages - 1;                  // tile t + kAhead is requested while tile t is multiplied
 constexpr int kXcds = 8;
-
-__device__ inline uint32_t lds_offset(int row, int chunk) { return row * (BK * 2) + ((chunk ^ ((row >> 1) & 7)) << 4); }
 
 __device__ inline uint16_t f32_to_bf16_bits(float f) {
     uint32_t u = __float_as_uint(f);
@@ -49,33 +60,24 @@ __device__ inline uint16_t f32_to_bf16_bits(float f) {
 
 __device__ inline float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(static_cast<uint32_t>(b) << 16); }
 
-// Loads this thread's four 16-byte chunks of one operand tile (rows row0..+255
-// of a [rows_total, K] matrix, columns k0..k0+63).  Rows past the end repeat the
-// last valid row (their products are never stored); chunks past K read as zero.
-__device__ inline void load_tile(const uint16_t* __restrict__ g, int64_t ld, int64_t rows_total, int64_t row0, int64_t K,
-                                 int64_t k0, uint4 (&r)[4]) {
-    const int c = threadIdx.x & 7;
-    const int rr = threadIdx.x >> 3;
-    const int64_t k = k0 + c * 8;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        int64_t row = row0 + rr + 64 * i;
-        row = row < rows_total ? row : rows_total - 1;
-        if (k < K)
-            r[i] = *reinterpret_cast<const uint4*>(g + row * ld + k);
-        else
-            r[i] = make_uint4(0, 0, 0, 0);
-    }
+typedef const __attribute__((address_space(1))) void* global_ptr;
+typedef __attribute__((address_space(3))) void* lds_ptr;
+
+// One wavefront instruction: lane l copies 16 bytes from its own global address
+// to LDS byte (dst + 16 l); dst is the same for all lanes.
+__device__ inline void dma16(const char* src, char* dst) {
+    __builtin_amdgcn_global_load_lds((global_ptr)src, (lds_ptr)dst, 16, 0, 0);
 }
 
-__device__ inline void store_tile(char* lds, const uint4 (&r)[4]) {
-    const int c = threadIdx.x & 7;
-    const int rr = threadIdx.x >> 3;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(lds + lds_offset(rr + 64 * i, c)) = r[i];
-}
+// s_waitcnt immediates (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4,
+// lgkmcnt 11:8): wait until at most N vector-memory requests are outstanding
+// and all LDS reads have returned.
+constexpr int kWaitVm4Lgkm0 = 0x0074;
+constexpr int kWaitVm8Lgkm0 = 0x0078;
+constexpr int kWaitVm0Lgkm0 = 0x0070;
 
-__global__ __launch_bounds__(kThreads) void linear_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+template <int NWM, int NWN>   // wavefronts along m and n; each owns (256/NWM) x (256/NWN)
+__global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
                                                                const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
                                                                int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw,
                                                                int64_t ldy, int tiles_m, int tiles_n, int vec_store) {
@@ -100,99 +102,255 @@ __global__ __launch_bounds__(kThreads) void linear_bf16_kernel(const uint16_t* _
 
     const int64_t m0 = static_cast<int64_t>(tm) * BM, n0 = static_cast<int64_t>(tn) * BN;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int wm = (wave & 1) * 128, wn = (wave >> 1) * 64;   // wavefront origin inside the tile
+    constexpr int TM = BM / NWM / 32, TN = BN / NWN / 32;   // 32x32 sub-tiles of a wavefront along m and n
+    constexpr int NW = NWM * NWN;
+    constexpr int JW = 16 / NW;      // request instructions per wavefront and operand tile
+    const int wm = (wave % NWM) * (TM * 32), wn = (wave / NWM) * (TN * 32);   // wavefront origin inside the tile
     const int l32 = lane & 31, kg = lane >> 5;
 
-    constexpr int TN = 2, TM = 4;   // 32x32 sub-tiles of a wavefront along n and m
-    floatx16 acc[TN][TM];  // [n sub-tile][m sub-tile]
+    floatx16 acc[TN][TM];           // [n sub-tile][m sub-tile]
 #pragma unroll
     for (int a = 0; a < TN; ++a)
 #pragma unroll
-        for (int b = 0; b < 4; ++b)
+        for (int b = 0; b < TM; ++b)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
-    uint4 rw[4], rx[4];
-    const int64_t ktiles = (K + BK - 1) / BK;
-    load_tile(w, ldw, N, n0, K, 0, rw);
-    load_tile(x, ldx, M, m0, K, 0, rx);
-    store_tile(lds, rw);
-    store_tile(lds + kTileBytes, rx);
-    __syncthreads();
-
-    for (int64_t kt = 0; kt < ktiles; ++kt) {
-        char* cur = lds + (kt & 1) * kStageBytes;
-        char* nxt = lds + ((kt + 1) & 1) * kStageBytes;
-        const bool more = kt + 1 < ktiles;
-        if (more) {
-            load_tile(w, ldw, N, n0, K, (kt + 1) * BK, rw);
-            load_tile(x, ldx, M, m0, K, (kt + 1) * BK, rx);
+    // Global -> LDS requests of this lane.  Instruction j of this wavefront
+    // fills rows (2 wave + j) 16 .. +15 of a tile; lane l lands on row l / 4,
+    // physical chunk l % 4 of that row, i.e. logical chunk (l % 4) ^ ((row >> 2) & 3).
+    // Rows past the end of the matrix repeat its last row (their products are
+    // never stored).
+    const char* src_w[JW];
+    const char* src_x[JW];
+    int chunk_k;   // first k (in elements) of this lane's chunk inside a k-tile
+    {
+        const int r = lane >> 2;
+        chunk_k = ((lane & 3) ^ ((r >> 2) & 3)) * 8;
+#pragma unroll
+        for (int j = 0; j < JW; ++j) {
+            const int row = (JW * wave + j) * 16 + r;
+            int64_t rn = n0 + row, rm = m0 + row;
+            rn = rn < N ? rn : N - 1;
+            rm = rm < M ? rm : M - 1;
+            src_w[j] = reinterpret_cast<const char*>(w + rn * ldw + chunk_k);
+            src_x[j] = reinterpret_cast<const char*>(x + rm * ldx + chunk_k);
         }
-        const char* sw = cur;
-        const char* sx = cur + kTileBytes;
-        // Operand fragments are double-buffered: the LDS reads of k-step ks+1
-        // are issued before the MFMAs of k-step ks, so a wavefront does not
-        // stall on LDS latency between k-steps.
-        bf16x8 fa[2][TN], fb[2][TM];
+    }
+    char* const dma_dst = lds + (JW * wave) * 1024;   // + stage, + operand, + j KiB
+
+    const int ktiles = static_cast<int>((K + BK - 1) / BK);
+    const int full_tiles = static_cast<int>(K / BK);   // tiles [full_tiles, ktiles) straddle K
+
+    // One request instruction of a full tile: i = 0 .. 2 JW - 1.
+    auto request_part = [&](int t, int stage_off, int i) {
+        char* st = dma_dst + stage_off;
+        const int64_t kb = static_cast<int64_t>(t) * (BK * 2);
+        const int j = i >> 1;
+        if (i & 1)
+            dma16(src_x[j] + kb, st + kTileBytes + j * 1024);
+        else
+            dma16(src_w[j] + kb, st + j * 1024);
+    };
+
+    // Requests k-tile t into its stage in one go.  A tile that straddles K goes
+    // through registers so that the chunks past K can be written as zeros.
+    auto request = [&](int t, int stage_off) {
+        if (t < full_tiles) {
 #pragma unroll
-        for (int a = 0; a < TN; ++a) fa[0][a] = *reinterpret_cast<const bf16x8*>(sw + lds_offset(wn + a * 32 + l32, kg));
+            for (int i = 0; i < 2 * JW; ++i) request_part(t, stage_off, i);
+        } else {
+            char* st = dma_dst + stage_off;
+            const int64_t kb = static_cast<int64_t>(t) * (BK * 2);
+            const bool in = static_cast<int64_t>(t) * BK + chunk_k < K;
 #pragma unroll
-        for (int b = 0; b < TM; ++b) fb[0][b] = *reinterpret_cast<const bf16x8*>(sx + lds_offset(wm + b * 32 + l32, kg));
-#pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            const int cb = ks & 1, nb = cb ^ 1;
-            const bool pre = ks + 1 < BK / 16;
-            // One LDS read of the next k-step is issued behind each MFMA of this
-            // one, so that LDS traffic is spread evenly instead of arriving in
-            // bursts that fill the LDS queues of all wavefronts at once.
-#pragma unroll
-            for (int i = 0; i < TN * TM; ++i) {
-                const int a = i / TM, b = i % TM;
-                acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cb][a], fb[cb][b], acc[a][b], 0, 0, 0);
-                if (pre && i < TN)
-                    fa[nb][i] = *reinterpret_cast<const bf16x8*>(sw + lds_offset(wn + i * 32 + l32, (ks + 1) * 2 + kg));
-                else if (pre && i < TN + TM)
-                    fb[nb][i - TN] = *reinterpret_cast<const bf16x8*>(sx + lds_offset(wm + (i - TN) * 32 + l32, (ks + 1) * 2 + kg));
-                __builtin_amdgcn_sched_barrier(0);
+            for (int j = 0; j < JW; ++j) {
+                uint4 vw = make_uint4(0, 0, 0, 0), vx = make_uint4(0, 0, 0, 0);
+                if (in) {
+                    vw = *reinterpret_cast<const uint4*>(src_w[j] + kb);
+                    vx = *reinterpret_cast<const uint4*>(src_x[j] + kb);
+                }
+                *reinterpret_cast<uint4*>(st + j * 1024 + lane * 16) = vw;
+                *reinterpret_cast<uint4*>(st + kTileBytes + j * 1024 + lane * 16) = vx;
             }
         }
-        if (more) {
-            store_tile(nxt, rw);
-            store_tile(nxt + kTileBytes, rx);
+    };
+
+    // Fragment addresses: row (sub-tile origin + l32), logical chunk 2 ks + kg.
+    // Sub-tile origins are multiples of 32, so the swizzle term is (l32 >> 2) & 3.
+    const int frag_row = l32 * (BK * 2);
+    const int sw_k0 = ((kg ^ ((l32 >> 2) & 3)) << 4);        // k-step 0
+    const int sw_k1 = (((2 + kg) ^ ((l32 >> 2) & 3)) << 4);  // k-step 1
+    const int off_w = wn * (BK * 2) + frag_row;
+    const int off_x = kTileBytes + wm * (BK * 2) + frag_row;
+
+    auto read_frags = [&](const char* stage, int sw, bf16x8 (&fa)[TN], bf16x8 (&fb)[TM], int i) {
+        if (i < TN)
+            fa[i] = *reinterpret_cast<const bf16x8*>(stage + off_w + i * (32 * BK * 2) + sw);
+        else
+            fb[i - TN] = *reinterpret_cast<const bf16x8*>(stage + off_x + (i - TN) * (32 * BK * 2) + sw);
+    };
+
+    constexpr int kReqGap = (TN * TM) / (2 * JW);   // MFMAs between two request instructions
+    // vmcnt(n) lgkmcnt(0) with n = the requests of tiles t+2 .. t+kAhead-1, which may stay in flight
+    constexpr int kInFlight = (kAhead - 2) * 2 * JW;
+    static_assert(kInFlight < 64, "vmcnt counts to 63");
+    constexpr int kWaitSteady = 0x0070 | (kInFlight & 15) | ((kInFlight >> 4) << 14);
+    int cur_off = 0, nxt_off = kStageBytes, req_off = kAhead * kStageBytes;   // stages of tiles t, t+1, t+kAhead
+    auto next_stage = [](int off) { return off + kStageBytes == kLdsBytes ? 0 : off + kStageBytes; };
+    bf16x8 fa[2][TN], fb[2][TM];
+
+    // One k-tile.  On entry the fragments of (tile t, k-step 0) are in fa[0] /
+    // fb[0] or on their way.  STEADY: tile t+kAhead exists and is a full tile; its
+    // request instructions are spread between the MFMAs.
+    auto k_tile = [&](int t, auto steady) {
+        constexpr bool STEADY = decltype(steady)::value;
+        // Own requests of tile t+1 (and older) have landed; only tile t+2's may
+        // still be in flight.  The LDS reads issued so far have returned, so
+        // the stage that tile t+3 overwrites is no longer being read by this
+        // wavefront; the barrier extends both facts to the workgroup.
+        if (STEADY)
+            __builtin_amdgcn_s_waitcnt(kWaitSteady);
+        else
+            __builtin_amdgcn_s_waitcnt(kWaitVm0Lgkm0);
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (!STEADY && t + kAhead < ktiles) request(t + kAhead, req_off);
+
+        const char* cur = lds + cur_off;
+        const char* nxt = lds + nxt_off;
+        // k-step 0 of tile t; behind each MFMA one fragment read of k-step 1.
+#pragma unroll
+        for (int i = 0; i < TN * TM; ++i) {
+            const int a = i / TM, b = i % TM;
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0][a], fb[0][b], acc[a][b], 0, 0, 0);
+            if (i < TN + TM) read_frags(cur, sw_k1, fa[1], fb[1], i);
+            if (STEADY && (i % kReqGap == kReqGap - 1)) request_part(t + kAhead, req_off, i / kReqGap);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __syncthreads();
-    }
+        // k-step 1 of tile t; behind each MFMA one fragment read of tile t+1,
+        // k-step 0 (that stage is complete: every wavefront waited for its
+        // share before the barrier above).  Past the last tile the reads fetch
+        // stale LDS contents that are never used.
+#pragma unroll
+        for (int i = 0; i < TN * TM; ++i) {
+            const int a = i / TM, b = i % TM;
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][a], fb[1][b], acc[a][b], 0, 0, 0);
+            if (i < TN + TM) read_frags(nxt, sw_k0, fa[0], fb[0], i);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        cur_off = nxt_off;
+        nxt_off = next_stage(nxt_off);
+        req_off = next_stage(req_off);
+    };
+
+#pragma unroll 1
+    for (int t = 0; t < kAhead; ++t)
+        if (t < ktiles) request(t, t * kStageBytes);
+    // Tile 0 complete and visible, then its first fragments.
+    __builtin_amdgcn_s_waitcnt(kWaitVm0Lgkm0);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < TN + TM; ++i) read_frags(lds, sw_k0, fa[0], fb[0], i);
+
+    const int steady_end = full_tiles - kAhead > 0 ? full_tiles - kAhead : 0;
+    int t = 0;
+#pragma unroll 1
+    for (; t < steady_end; ++t) k_tile(t, std::true_type{});
+#pragma unroll 1
+    for (; t < ktiles; ++t) k_tile(t, std::false_type{});
 
     // Epilogue.  Lane holds, per 32x32 tile, output row m = l32 and the columns
     // n = 8*g + 4*kg + {0,1,2,3} for g = 0..3 in acc[...][4*g + {0..3}].
+    if (vec_store == 2) {
+        // Through LDS, so that global stores are 16 bytes per lane and whole
+        // 128-byte (or longer) row segments per instruction.  Each wavefront
+        // transposes its own (32 TM) x (32 TN) block in a private LDS region:
+        // row pitch 64 TN bytes, the 16-byte chunk index XOR-ed with a function
+        // of the row so that neither the 8-byte writes (32 rows, one column
+        // group) nor the 16-byte reads (whole rows) pile up on banks.
+        constexpr int kPitch = TN * 64;              // bytes of one row of the block
+        constexpr int kChunks = TN * 4;              // 16-byte chunks per row
+        constexpr int kRowsPerPass = 64 / kChunks;   // rows one read instruction covers
+        auto swz = [](int row) { return TN == 2 ? ((row >> 1) & 7) : (row & (kChunks - 1)); };
+        __syncthreads();   // every wavefront is done with the operand stages (and every request has landed)
+        char* region = lds + wave * (TM * 32 * kPitch);
 #pragma unroll
-    for (int a = 0; a < TN; ++a) {
+        for (int a = 0; a < TN; ++a) {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int64_t n = n0 + wn + a * 32 + 8 * g + 4 * kg;
-            float bv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (bias) {
+            for (int g = 0; g < 4; ++g) {
+                const int64_t n = n0 + wn + a * 32 + 8 * g + 4 * kg;
+                float bv[4] = {0.f, 0.f, 0.f, 0.f};
+                if (bias) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (n + e < N) bv[e] = bf16_bits_to_f32(bias[n + e]);
-            }
+                    for (int e = 0; e < 4; ++e)
+                        if (n + e < N) bv[e] = bf16_bits_to_f32(bias[n + e]);
+                }
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                const int64_t m = m0 + wm + b * 32 + l32;
-                if (m >= M) continue;
-                uint16_t o[4];
+                for (int b = 0; b < TM; ++b) {
+                    const int row = b * 32 + l32;
+                    uint16_t o[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16_bits(acc[a][b][4 * g + e] + bv[e]);
-                uint16_t* dst = y + m * ldy + n;
-                if (vec_store && n + 3 < N) {
+                    for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16_bits(acc[a][b][4 * g + e] + bv[e]);
                     uint2 pk;
                     pk.x = static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16);
                     pk.y = static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16);
-                    *reinterpret_cast<uint2*>(dst) = pk;
-                } else {
+                    *reinterpret_cast<uint2*>(region + row * kPitch + (((a * 4 + g) ^ swz(row)) << 4) + kg * 8) = pk;
+                }
+            }
+        }
+        // LDS operations of one wavefront complete in order, so its reads below
+        // see its writes above; no other wavefront touches this region.
+        asm volatile("" ::: "memory");
+        const int chunk = lane % kChunks;
+        const int64_t n = n0 + wn + chunk * 8;
+#pragma unroll 4
+        for (int r0 = 0; r0 < TM * 32; r0 += kRowsPerPass) {
+            const int row = r0 + lane / kChunks;
+            const int64_t m = m0 + wm + row;
+            const uint4 v = *reinterpret_cast<const uint4*>(region + row * kPitch + ((chunk ^ swz(row)) << 4));
+            if (m >= M || n >= N) continue;
+            uint16_t* dst = y + m * ldy + n;
+            if (n + 8 <= N) {
+                *reinterpret_cast<uint4*>(dst) = v;
+            } else {
+                const uint32_t words[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (n + e < N) dst[e] = static_cast<uint16_t>(words[e >> 1] >> (16 * (e & 1)));
+            }
+        }
+    } else {
+    #pragma unroll
+        for (int a = 0; a < TN; ++a) {
+    #pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int64_t n = n0 + wn + a * 32 + 8 * g + 4 * kg;
+                float bv[4] = {0.f, 0.f, 0.f, 0.f};
+                if (bias) {
+    #pragma unroll
                     for (int e = 0; e < 4; ++e)
-                        if (n + e < N) dst[e] = o[e];
+                        if (n + e < N) bv[e] = bf16_bits_to_f32(bias[n + e]);
+                }
+    #pragma unroll
+                for (int b = 0; b < TM; ++b) {
+                    const int64_t m = m0 + wm + b * 32 + l32;
+                    if (m >= M) continue;
+                    uint16_t o[4];
+    #pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16_bits(acc[a][b][4 * g + e] + bv[e]);
+                    uint16_t* dst = y + m * ldy + n;
+                    if (vec_store && n + 3 < N) {
+                        uint2 pk;
+                        pk.x = static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16);
+                        pk.y = static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16);
+                        *reinterpret_cast<uint2*>(dst) = pk;
+                    } else {
+    #pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (n + e < N) dst[e] = o[e];
+                    }
                 }
             }
         }
@@ -217,17 +375,22 @@ extern "C" int ddl_linear_bf16(const void* x, const void* w, const void* bias, v
     const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     if (tiles_m * tiles_n > 0x7FFFFFFFll || tiles_m > 0x7FFFFFll || tiles_n > 0x7FFFFFll)
         return fail(DDL_E_UNSUPP, "linear: too many output tiles");
-    static bool attr_done = false;
-    if (!attr_done) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(linear_bf16_kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-        if (e != hipSuccess) return fail(static_cast<int>(e), "linear: cannot reserve %d bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
-        attr_done = true;
-    }
-    const int vec_store = (ldy % 4 == 0) && aligned_to(y, 8);
-    hipLaunchKernelGGL(linear_bf16_kernel, dim3(static_cast<uint32_t>(tiles_m * tiles_n)), dim3(kThreads), kLdsBytes,
-                       static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w),
-                       static_cast<const uint16_t*>(bias), static_cast<uint16_t*>(y), M, N, K, ldx, ldw, ldy,
-                       static_cast<int>(tiles_m), static_cast<int>(tiles_n), vec_store);
+    // 2: rows of y can be stored 16 bytes at a time, 1: 8 bytes, 0: element by element
+    const int vec_store = (ldy % 8 == 0 && aligned_to(y, 16)) ? 2 : (ldy % 4 == 0 && aligned_to(y, 8)) ? 1 : 0;
+    auto launch = [&](auto kernel, int threads) -> int {
+        static bool attr_done = false;   // the attribute sticks to the function; set it on first use
+        if (!attr_done) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+            if (e != hipSuccess) return fail(static_cast<int>(e), "linear: cannot reserve %d bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
+            attr_done = true;
+        }
+        hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(tiles_m * tiles_n)), dim3(threads), kLdsBytes,
+                           static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w),
+                           static_cast<const uint16_t*>(bias), static_cast<uint16_t*>(y), M, N, K, ldx, ldw, ldy,
+                           static_cast<int>(tiles_m), static_cast<int>(tiles_n), vec_store);
+        return 0;
+    };
+    const int rc = launch(linear_bf16_kernel<2, 4>, 512);
+    if (rc) return rc;
     return check_launch("linear_bf16_kernel");
 }

@@ -257,6 +257,27 @@ def test_linear_small_integer_cases_are_exact(ops, M, N, K, use_bias):
     assert torch.equal(y.cpu().double(), want)
 
 
+@pytest.mark.parametrize("M,N,K,ldy", [(300, 259, 72, 264), (513, 100, 136, 104), (70, 255, 64, 512), (257, 36, 32, 36)])
+def test_linear_strided_output_through_the_c_abi(ops, M, N, K, ldy):
+    """Output rows with a pitch larger than N (and N not a multiple of the
+    16-byte store width): results exact, the gap between rows untouched."""
+    from distdl_amd import _lib
+    gen = torch.Generator().manual_seed(M + 3 * N + K)
+    x = torch.randint(-1, 2, (M, K), generator=gen).to(torch.bfloat16)
+    w = torch.randint(-1, 2, (N, K), generator=gen).to(torch.bfloat16)
+    b = torch.randint(-3, 4, (N,), generator=gen).to(torch.bfloat16)
+    xg, wg, bg = x.cuda(), w.cuda(), b.cuda()
+    out = torch.full((M, ldy), 77.0, dtype=torch.bfloat16, device="cuda")
+    rc = _lib.load().ddl_linear_bf16(xg.data_ptr(), wg.data_ptr(), bg.data_ptr(), out.data_ptr(), M, N, K, K, K, ldy,
+                                     torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "ddl_linear_bf16")
+    want = x.double() @ w.double().T + b.double()
+    assert want.abs().max() <= 256
+    got = out.cpu().double()
+    assert torch.equal(got[:, :N], want)
+    assert (got[:, N:] == 77.0).all()
+
+
 @pytest.mark.parametrize("M,N,K", [(128, 96, 256), (777, 333, 1024), (2048, 1024, 512)])
 def test_linear_random_within_tolerance(ops, M, N, K):
     gen = torch.Generator().manual_seed(M + N + K)
