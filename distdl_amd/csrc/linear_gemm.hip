@@ -13,21 +13,25 @@
 //              issue MFMAs while the other waits
 //   wavefront  128(m) x 64(n) = 4 x 2 tiles of v_mfma_f32_32x32x16_bf16, 128 fp32
 //              accumulators per lane
-//   LDS        five stages of {w tile, x tile}, each tile 256 rows x 32 k =
-//              16 KiB (160 KiB in all).  Rows are 64 B; the 16-byte chunk index
-//              is XOR-ed with ((row >> 2) & 3): the 16 lanes served per LDS
-//              cycle read 16 consecutive rows, and (row & 3, (row >> 2) & 3) is
-//              distinct for each, so they cover all 64 banks
+//   LDS        ring of five operand tiles (W0 X0 W1 X1 W2 | X2 W3 ...), each
+//              256 rows x 64 k = 32 KiB, 160 KiB in all.  Rows are 128 B; the
+//              16-byte chunk index is XOR-ed with ((row >> 1) & 7): the 16
+//              lanes served per LDS cycle read 16 consecutive rows, and
+//              (row & 1, (row >> 1) & 7) is distinct for each, so they cover all
+//              64 banks
 //   global     tiles go from global memory straight into LDS
-//              (global_load_lds_dwordx4: each wavefront instruction fills 1 KiB
-//              = 16 rows); no staging registers, no LDS stores.  Tile t+4 is
-//              requested while tile t is multiplied and has to be complete one
-//              tile before its turn, so a request has three k-tiles of MFMA
-//              time to arrive
-//   schedule   per k-tile: wait for own requests of tile t+1, barrier, then
-//              2 x 8 MFMAs with one LDS fragment read issued behind each (the
-//              fragments of the next k-step, crossing into tile t+1) and the
-//              request instructions of tile t+4 spread between them
+//              (buffer_load_dwordx4 ... lds: each wavefront instruction fills
+//              1 KiB = 8 rows, the eight lanes of a row fetching one whole
+//              128-byte line; half-line requests run at little more than half
+//              the rate).  No staging registers, no LDS stores, one 32-bit
+//              offset per lane and the k offset in a scalar
+//   schedule   per k-tile of 64: four k-steps of 8 MFMAs, one LDS fragment
+//              read issued behind each MFMA (the fragments of the next k-step,
+//              crossing into tile t+1 at the end).  W(t+2) is requested during
+//              k-step 0 into the slot X(t-1) left, X(t+2) during k-step 3 into
+//              the slot of W(t); before k-step 3 each wavefront waits for its
+//              own requests of tile t+1 and all its LDS reads, then one
+//              barrier: tile t+1 is readable, tile t's slots are free
 //   epilogue   bias add and bf16 rounding in registers, then each wavefront
 //              transposes its block through LDS so that rows of y are written
 //              in 16-byte pieces, whole 128-byte lines per instruction
@@ -43,12 +47,10 @@ namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 
-constexpr int BM = 256, BN = 256, BK = 32;
-constexpr int kStages = 5;
-constexpr int kTileBytes = BM * BK * 2;              // one operand tile, 16 KiB
-constexpr int kStageBytes = 2 * kTileBytes;          // w tile + x tile
-constexpr int kLdsBytes = kStages * kStageBytes;     // 160 KiB: all of a CU's LDS
-constexpr int kAhead = kStages - 1;                  // tile t + kAhead is requested while tile t is multiplied
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int kUnitBytes = BM * BK * 2;              // one operand tile (256 rows x 128 B), 32 KiB
+constexpr int kUnits = 5;                            // ring of operand tiles: W0 X0 W1 X1 W2 | X2 W3 ...
+constexpr int kLdsBytes = kUnits * kUnitBytes;       // 160 KiB: all of a CU's LDS
 constexpr int kXcds = 8;
 
 __device__ inline uint16_t f32_to_bf16_bits(float f) {
@@ -60,21 +62,19 @@ __device__ inline uint16_t f32_to_bf16_bits(float f) {
 
 __device__ inline float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(static_cast<uint32_t>(b) << 16); }
 
-typedef const __attribute__((address_space(1))) void* global_ptr;
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
-// One wavefront instruction: lane l copies 16 bytes from its own global address
-// to LDS byte (dst + 16 l); dst is the same for all lanes.
-__device__ inline void dma16(const char* src, char* dst) {
-    __builtin_amdgcn_global_load_lds((global_ptr)src, (lds_ptr)dst, 16, 0, 0);
+// One wavefront instruction: lane l copies the 16 bytes at byte (voffset +
+// soffset) of the buffer to LDS byte (dst + 16 l); dst and soffset are the same
+// for all lanes.
+__device__ inline void dma16(__amdgpu_buffer_rsrc_t buffer, int voffset, int soffset, char* dst) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(buffer, (lds_ptr)dst, 16, voffset, soffset, 0, 0);
 }
 
-// s_waitcnt immediates (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4,
-// lgkmcnt 11:8): wait until at most N vector-memory requests are outstanding
+// s_waitcnt immediate (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4,
+// lgkmcnt 11:8): wait until at most n vector-memory requests are outstanding
 // and all LDS reads have returned.
-constexpr int kWaitVm4Lgkm0 = 0x0074;
-constexpr int kWaitVm8Lgkm0 = 0x0078;
-constexpr int kWaitVm0Lgkm0 = 0x0070;
+constexpr int wait_vm_lgkm0(int n) { return 0x0070 | (n & 15) | ((n >> 4) << 14); }
 
 template <int NWM, int NWN>   // wavefronts along m and n; each owns (256/NWM) x (256/NWN)
 __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
@@ -104,7 +104,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     constexpr int TM = BM / NWM / 32, TN = BN / NWN / 32;   // 32x32 sub-tiles of a wavefront along m and n
     constexpr int NW = NWM * NWN;
-    constexpr int JW = 16 / NW;      // request instructions per wavefront and operand tile
+    constexpr int JW = 32 / NW;      // request instructions per wavefront and operand tile
     const int wm = (wave % NWM) * (TM * 32), wn = (wave / NWM) * (TN * 32);   // wavefront origin inside the tile
     const int l32 = lane & 31, kg = lane >> 5;
 
@@ -117,144 +117,138 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
     // Global -> LDS requests of this lane.  Instruction j of this wavefront
-    // fills rows (2 wave + j) 16 .. +15 of a tile; lane l lands on row l / 4,
-    // physical chunk l % 4 of that row, i.e. logical chunk (l % 4) ^ ((row >> 2) & 3).
-    // Rows past the end of the matrix repeat its last row (their products are
-    // never stored).
-    const char* src_w[JW];
-    const char* src_x[JW];
-    int chunk_k;   // first k (in elements) of this lane's chunk inside a k-tile
+    // fills rows (JW wave + j) 8 .. +7 of an operand tile; lane l lands on row
+    // l / 8, physical chunk l % 8 of that row, i.e. logical chunk
+    // (l % 8) ^ ((row >> 1) & 7): the eight lanes of a row fetch one whole
+    // 128-byte line.  Rows past the end of the matrix repeat its last row
+    // (their products are never stored).
+    // The operands are addressed as raw buffers that start at the tile's first
+    // row: a 32-bit byte offset per lane, the k-tile offset in a scalar.
+    const char* const base_w = reinterpret_cast<const char*>(w + n0 * ldw);
+    const char* const base_x = reinterpret_cast<const char*>(x + m0 * ldx);
+    const __amdgpu_buffer_rsrc_t buf_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base_w), 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t buf_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base_x), 0, -1, 0x00020000);
+    int off_gw[JW], off_gx[JW];
     {
-        const int r = lane >> 2;
-        chunk_k = ((lane & 3) ^ ((r >> 2) & 3)) * 8;
+        const int r = lane >> 3;
 #pragma unroll
         for (int j = 0; j < JW; ++j) {
-            const int row = (JW * wave + j) * 16 + r;
-            int64_t rn = n0 + row, rm = m0 + row;
-            rn = rn < N ? rn : N - 1;
-            rm = rm < M ? rm : M - 1;
-            src_w[j] = reinterpret_cast<const char*>(w + rn * ldw + chunk_k);
-            src_x[j] = reinterpret_cast<const char*>(x + rm * ldx + chunk_k);
+            const int row = (JW * wave + j) * 8 + r;
+            const int ck = ((lane & 7) ^ ((row >> 1) & 7)) * 8;   // first k of this lane's chunk inside a k-tile
+            const int64_t rn = n0 + row < N ? row : N - 1 - n0;
+            const int64_t rm = m0 + row < M ? row : M - 1 - m0;
+            off_gw[j] = static_cast<int>((rn * ldw + ck) * 2);
+            off_gx[j] = static_cast<int>((rm * ldx + ck) * 2);
         }
     }
-    char* const dma_dst = lds + (JW * wave) * 1024;   // + stage, + operand, + j KiB
+    char* const dma_dst = lds + (JW * wave) * 1024;   // + unit, + j KiB
 
     const int ktiles = static_cast<int>((K + BK - 1) / BK);
     const int full_tiles = static_cast<int>(K / BK);   // tiles [full_tiles, ktiles) straddle K
 
-    // One request instruction of a full tile: i = 0 .. 2 JW - 1.
-    auto request_part = [&](int t, int stage_off, int i) {
-        char* st = dma_dst + stage_off;
-        const int64_t kb = static_cast<int64_t>(t) * (BK * 2);
-        const int j = i >> 1;
-        if (i & 1)
-            dma16(src_x[j] + kb, st + kTileBytes + j * 1024);
-        else
-            dma16(src_w[j] + kb, st + j * 1024);
+    // One request instruction (j = 0 .. JW-1) of operand tile t, a full tile.
+    auto request_part = [&](__amdgpu_buffer_rsrc_t buf, const int (&off)[JW], int t, int unit_off, int j) {
+        dma16(buf, off[j], t * (BK * 2), dma_dst + unit_off + j * 1024);
     };
-
-    // Requests k-tile t into its stage in one go.  A tile that straddles K goes
-    // through registers so that the chunks past K can be written as zeros.
-    auto request = [&](int t, int stage_off) {
+    // A whole operand tile.  One that straddles K goes through registers so
+    // that the chunks past K can be written as zeros.
+    auto request_unit = [&](__amdgpu_buffer_rsrc_t buf, const char* base, const int (&off)[JW], int t, int unit_off) {
         if (t < full_tiles) {
 #pragma unroll
-            for (int i = 0; i < 2 * JW; ++i) request_part(t, stage_off, i);
+            for (int j = 0; j < JW; ++j) request_part(buf, off, t, unit_off, j);
         } else {
-            char* st = dma_dst + stage_off;
-            const int64_t kb = static_cast<int64_t>(t) * (BK * 2);
-            const bool in = static_cast<int64_t>(t) * BK + chunk_k < K;
 #pragma unroll
             for (int j = 0; j < JW; ++j) {
-                uint4 vw = make_uint4(0, 0, 0, 0), vx = make_uint4(0, 0, 0, 0);
-                if (in) {
-                    vw = *reinterpret_cast<const uint4*>(src_w[j] + kb);
-                    vx = *reinterpret_cast<const uint4*>(src_x[j] + kb);
-                }
-                *reinterpret_cast<uint4*>(st + j * 1024 + lane * 16) = vw;
-                *reinterpret_cast<uint4*>(st + kTileBytes + j * 1024 + lane * 16) = vx;
+                const int row = (JW * wave + j) * 8 + (lane >> 3);
+                const int ck = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (static_cast<int64_t>(t) * BK + ck < K)
+                    v = *reinterpret_cast<const uint4*>(base + off[j] + static_cast<int64_t>(t) * (BK * 2));
+                *reinterpret_cast<uint4*>(dma_dst + unit_off + j * 1024 + lane * 16) = v;
             }
         }
     };
 
     // Fragment addresses: row (sub-tile origin + l32), logical chunk 2 ks + kg.
-    // Sub-tile origins are multiples of 32, so the swizzle term is (l32 >> 2) & 3.
+    // Sub-tile origins are multiples of 32, so the swizzle term is (l32 >> 1) & 7.
     const int frag_row = l32 * (BK * 2);
-    const int sw_k0 = ((kg ^ ((l32 >> 2) & 3)) << 4);        // k-step 0
-    const int sw_k1 = (((2 + kg) ^ ((l32 >> 2) & 3)) << 4);  // k-step 1
+    int sw_off[4];   // byte offset of this lane's chunk in its row, per k-step
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) sw_off[ks] = ((2 * ks + kg) ^ ((l32 >> 1) & 7)) << 4;
     const int off_w = wn * (BK * 2) + frag_row;
-    const int off_x = kTileBytes + wm * (BK * 2) + frag_row;
+    const int off_x = wm * (BK * 2) + frag_row;
 
-    auto read_frags = [&](const char* stage, int sw, bf16x8 (&fa)[TN], bf16x8 (&fb)[TM], int i) {
+    auto read_frag = [&](const char* wt, const char* xt, int ks, bf16x8 (&fa)[TN], bf16x8 (&fb)[TM], int i) {
+        const int sw = sw_off[ks];
         if (i < TN)
-            fa[i] = *reinterpret_cast<const bf16x8*>(stage + off_w + i * (32 * BK * 2) + sw);
+            fa[i] = *reinterpret_cast<const bf16x8*>(wt + off_w + i * (32 * BK * 2) + sw);
         else
-            fb[i - TN] = *reinterpret_cast<const bf16x8*>(stage + off_x + (i - TN) * (32 * BK * 2) + sw);
+            fb[i - TN] = *reinterpret_cast<const bf16x8*>(xt + off_x + (i - TN) * (32 * BK * 2) + sw);
     };
 
-    constexpr int kReqGap = (TN * TM) / (2 * JW);   // MFMAs between two request instructions
-    // vmcnt(n) lgkmcnt(0) with n = the requests of tiles t+2 .. t+kAhead-1, which may stay in flight
-    constexpr int kInFlight = (kAhead - 2) * 2 * JW;
-    static_assert(kInFlight < 64, "vmcnt counts to 63");
-    constexpr int kWaitSteady = 0x0070 | (kInFlight & 15) | ((kInFlight >> 4) << 14);
-    int cur_off = 0, nxt_off = kStageBytes, req_off = kAhead * kStageBytes;   // stages of tiles t, t+1, t+kAhead
-    auto next_stage = [](int off) { return off + kStageBytes == kLdsBytes ? 0 : off + kStageBytes; };
+    auto unit_off = [](int slot) { return (slot >= kUnits ? slot - kUnits : slot) * kUnitBytes; };
+    int s0 = 0;   // ring slot of W(t); X(t), W(t+1), X(t+1), W(t+2) follow
     bf16x8 fa[2][TN], fb[2][TM];
 
-    // One k-tile.  On entry the fragments of (tile t, k-step 0) are in fa[0] /
-    // fb[0] or on their way.  STEADY: tile t+kAhead exists and is a full tile; its
-    // request instructions are spread between the MFMAs.
+    // One k-tile = four k-steps of 16.  On entry the fragments of (t, k-step 0)
+    // are in fa[0] / fb[0] or on their way, W(t+1) and X(t+1) have been
+    // requested.  STEADY: tile t+2 exists and is a full tile; its request
+    // instructions are spread between the MFMAs.
     auto k_tile = [&](int t, auto steady) {
         constexpr bool STEADY = decltype(steady)::value;
-        // Own requests of tile t+1 (and older) have landed; only tile t+2's may
-        // still be in flight.  The LDS reads issued so far have returned, so
-        // the stage that tile t+3 overwrites is no longer being read by this
-        // wavefront; the barrier extends both facts to the workgroup.
-        if (STEADY)
-            __builtin_amdgcn_s_waitcnt(kWaitSteady);
-        else
-            __builtin_amdgcn_s_waitcnt(kWaitVm0Lgkm0);
+        const char* wt = lds + unit_off(s0);
+        const char* xt = lds + unit_off(s0 + 1);
+        const char* wn1 = lds + unit_off(s0 + 2);
+        const char* xn1 = lds + unit_off(s0 + 3);
+        const int w2_off = unit_off(s0 + 4);   // slot of X(t-1), free since the barrier of tile t-1
+        const int x2_off = unit_off(s0);       // slot of W(t), free after this tile's barrier
+        if (!STEADY && t + 2 < ktiles) request_unit(buf_w, base_w, off_gw, t + 2, w2_off);
+#pragma unroll
+        for (int ks = 0; ks < 3; ++ks) {
+#pragma unroll
+            for (int i = 0; i < TN * TM; ++i) {
+                const int a = i / TM, b = i % TM;
+                acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][a], fb[ks & 1][b], acc[a][b], 0, 0, 0);
+                if (i < TN + TM) read_frag(wt, xt, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1], i);
+                if (STEADY && ks == 0 && (i & 1) && (i >> 1) < JW) request_part(buf_w, off_gw, t + 2, w2_off, i >> 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // Own requests of W(t+1), X(t+1) have landed (W(t+2)'s may still be in
+        // flight) and every LDS read issued so far -- all of tile t's -- has
+        // returned; the barrier extends both to the workgroup, so tile t+1 may
+        // be read and tile t's slots may be overwritten.
+        __builtin_amdgcn_s_waitcnt(STEADY ? wait_vm_lgkm0(JW) : wait_vm_lgkm0(0));
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        if (!STEADY && t + kAhead < ktiles) request(t + kAhead, req_off);
-
-        const char* cur = lds + cur_off;
-        const char* nxt = lds + nxt_off;
-        // k-step 0 of tile t; behind each MFMA one fragment read of k-step 1.
-#pragma unroll
-        for (int i = 0; i < TN * TM; ++i) {
-            const int a = i / TM, b = i % TM;
-            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0][a], fb[0][b], acc[a][b], 0, 0, 0);
-            if (i < TN + TM) read_frags(cur, sw_k1, fa[1], fb[1], i);
-            if (STEADY && (i % kReqGap == kReqGap - 1)) request_part(t + kAhead, req_off, i / kReqGap);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        // k-step 1 of tile t; behind each MFMA one fragment read of tile t+1,
-        // k-step 0 (that stage is complete: every wavefront waited for its
-        // share before the barrier above).  Past the last tile the reads fetch
-        // stale LDS contents that are never used.
+        if (!STEADY && t + 2 < ktiles) request_unit(buf_x, base_x, off_gx, t + 2, x2_off);
 #pragma unroll
         for (int i = 0; i < TN * TM; ++i) {
             const int a = i / TM, b = i % TM;
             acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][a], fb[1][b], acc[a][b], 0, 0, 0);
-            if (i < TN + TM) read_frags(nxt, sw_k0, fa[0], fb[0], i);
+            // Past the last tile these reads fetch stale LDS contents that are never used.
+            if (i < TN + TM) read_frag(wn1, xn1, 0, fa[0], fb[0], i);
+            if (STEADY && (i & 1) && (i >> 1) < JW) request_part(buf_x, off_gx, t + 2, x2_off, i >> 1);
             __builtin_amdgcn_sched_barrier(0);
         }
-        cur_off = nxt_off;
-        nxt_off = next_stage(nxt_off);
-        req_off = next_stage(req_off);
+        s0 = s0 + 2 >= kUnits ? s0 + 2 - kUnits : s0 + 2;
     };
 
-#pragma unroll 1
-    for (int t = 0; t < kAhead; ++t)
-        if (t < ktiles) request(t, t * kStageBytes);
+    static_assert(TN * TM >= 2 * JW, "not enough MFMAs in a k-step to spread the requests");
+    request_unit(buf_w, base_w, off_gw, 0, 0);
+    request_unit(buf_x, base_x, off_gx, 0, kUnitBytes);
+    if (ktiles > 1) {
+        request_unit(buf_w, base_w, off_gw, 1, 2 * kUnitBytes);
+        request_unit(buf_x, base_x, off_gx, 1, 3 * kUnitBytes);
+    }
     // Tile 0 complete and visible, then its first fragments.
-    __builtin_amdgcn_s_waitcnt(kWaitVm0Lgkm0);
+    __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 #pragma unroll
-    for (int i = 0; i < TN + TM; ++i) read_frags(lds, sw_k0, fa[0], fb[0], i);
+    for (int i = 0; i < TN + TM; ++i) read_frag(lds, lds + kUnitBytes, 0, fa[0], fb[0], i);
 
-    const int steady_end = full_tiles - kAhead > 0 ? full_tiles - kAhead : 0;
+    const int steady_end = full_tiles - 2 > 0 ? full_tiles - 2 : 0;
     int t = 0;
 #pragma unroll 1
     for (; t < steady_end; ++t) k_tile(t, std::true_type{});
@@ -372,6 +366,8 @@ extern "C" int ddl_linear_bf16(const void* x, const void* w, const void* bias, v
     if (K % 8 != 0 || ldx % 8 != 0 || ldw % 8 != 0 || !aligned_to(x, 16) || !aligned_to(w, 16))
         return fail(DDL_E_ALIGN, "linear: K, ldx, ldw must be multiples of 8 and x, w 16-byte aligned");
     if (!aligned_to(y, 2) || (bias && !aligned_to(bias, 2))) return fail(DDL_E_ALIGN, "linear: y / bias misaligned");
+    if (ldx > 0x3FFFFF || ldw > 0x3FFFFF || K > 0x3FFFFFFF)
+        return fail(DDL_E_UNSUPP, "linear: row pitch above 2^22 elements or K above 2^30");   // 32-bit byte offsets inside a tile
     const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     if (tiles_m * tiles_n > 0x7FFFFFFFll || tiles_m > 0x7FFFFFll || tiles_n > 0x7FFFFFll)
         return fail(DDL_E_UNSUPP, "linear: too many output tiles");
