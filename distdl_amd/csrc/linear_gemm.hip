@@ -47,8 +47,9 @@ namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 
-constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int kUnitBytes = BM * BK * 2;              // one operand tile (256 rows x 128 B), 32 KiB
+constexpr int BK = 64;
+constexpr int kMaxTileRows = 256;                    // rows of an operand tile: 256 of x; 256 or 192 of w
+constexpr int kUnitBytes = kMaxTileRows * BK * 2;    // ring slot for one operand tile (rows x 128 B), 32 KiB
 constexpr int kUnits = 5;                            // ring of operand tiles: W0 X0 W1 X1 W2 | X2 W3 ...
 constexpr int kLdsBytes = kUnits * kUnitBytes;       // 160 KiB: all of a CU's LDS
 constexpr int kXcds = 8;
@@ -76,7 +77,9 @@ __device__ inline void dma16(__amdgpu_buffer_rsrc_t buffer, int voffset, int sof
 // and all LDS reads have returned.
 constexpr int wait_vm_lgkm0(int n) { return 0x0070 | (n & 15) | ((n >> 4) << 14); }
 
-template <int NWM, int NWN>   // wavefronts along m and n; each owns (256/NWM) x (256/NWN)
+// NWM x NWN wavefronts, each owning TM x TN sub-tiles of 32 x 32: the workgroup
+// tile is (32 NWM TM) x (32 NWN TN).
+template <int NWM, int NWN, int TM, int TN>
 __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
                                                                const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
                                                                int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw,
@@ -100,11 +103,14 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
     const int tm = band_m0 + in_band % band_h;
     const int tn = in_band / band_h;
 
+    constexpr int BM = 32 * NWM * TM, BN = 32 * NWN * TN;
+    static_assert(BM <= kMaxTileRows && BN <= kMaxTileRows, "operand tile larger than a ring slot");
     const int64_t m0 = static_cast<int64_t>(tm) * BM, n0 = static_cast<int64_t>(tn) * BN;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    constexpr int TM = BM / NWM / 32, TN = BN / NWN / 32;   // 32x32 sub-tiles of a wavefront along m and n
     constexpr int NW = NWM * NWN;
-    constexpr int JW = 32 / NW;      // request instructions per wavefront and operand tile
+    // request instructions (8 rows each) per wavefront for a w tile and an x tile
+    constexpr int JW_W = BN / 8 / NW, JW_X = BM / 8 / NW;
+    static_assert(JW_W * 8 * NW == BN && JW_X * 8 * NW == BM, "tile rows do not divide among the wavefronts");
     const int wm = (wave % NWM) * (TM * 32), wn = (wave / NWM) * (TN * 32);   // wavefront origin inside the tile
     const int l32 = lane & 31, kg = lane >> 5;
 
@@ -117,7 +123,8 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
     // Global -> LDS requests of this lane.  Instruction j of this wavefront
-    // fills rows (JW wave + j) 8 .. +7 of an operand tile; lane l lands on row
+    // fills rows (J wave + j) 8 .. +7 of an operand tile (J instructions per
+    // wavefront); lane l lands on row
     // l / 8, physical chunk l % 8 of that row, i.e. logical chunk
     // (l % 8) ^ ((row >> 1) & 7): the eight lanes of a row fetch one whole
     // 128-byte line.  Rows past the end of the matrix repeat its last row
@@ -128,43 +135,49 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
     const char* const base_x = reinterpret_cast<const char*>(x + m0 * ldx);
     const __amdgpu_buffer_rsrc_t buf_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base_w), 0, -1, 0x00020000);
     const __amdgpu_buffer_rsrc_t buf_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base_x), 0, -1, 0x00020000);
-    int off_gw[JW], off_gx[JW];
+    int off_gw[JW_W], off_gx[JW_X];
     {
         const int r = lane >> 3;
 #pragma unroll
-        for (int j = 0; j < JW; ++j) {
-            const int row = (JW * wave + j) * 8 + r;
+        for (int j = 0; j < JW_W; ++j) {
+            const int row = (JW_W * wave + j) * 8 + r;
             const int ck = ((lane & 7) ^ ((row >> 1) & 7)) * 8;   // first k of this lane's chunk inside a k-tile
             const int64_t rn = n0 + row < N ? row : N - 1 - n0;
-            const int64_t rm = m0 + row < M ? row : M - 1 - m0;
             off_gw[j] = static_cast<int>((rn * ldw + ck) * 2);
+        }
+#pragma unroll
+        for (int j = 0; j < JW_X; ++j) {
+            const int row = (JW_X * wave + j) * 8 + r;
+            const int ck = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
+            const int64_t rm = m0 + row < M ? row : M - 1 - m0;
             off_gx[j] = static_cast<int>((rm * ldx + ck) * 2);
         }
     }
-    char* const dma_dst = lds + (JW * wave) * 1024;   // + unit, + j KiB
 
     const int ktiles = static_cast<int>((K + BK - 1) / BK);
     const int full_tiles = static_cast<int>(K / BK);   // tiles [full_tiles, ktiles) straddle K
 
-    // One request instruction (j = 0 .. JW-1) of operand tile t, a full tile.
-    auto request_part = [&](__amdgpu_buffer_rsrc_t buf, const int (&off)[JW], int t, int unit_off, int j) {
-        dma16(buf, off[j], t * (BK * 2), dma_dst + unit_off + j * 1024);
+    // One request instruction (j = 0 .. J-1) of operand tile t, a full tile.
+    auto request_part = [&](__amdgpu_buffer_rsrc_t buf, const auto& off, int t, int unit_off, int j) {
+        constexpr int J = sizeof(off) / sizeof(int);
+        dma16(buf, off[j], t * (BK * 2), lds + unit_off + (J * wave + j) * 1024);
     };
     // A whole operand tile.  One that straddles K goes through registers so
     // that the chunks past K can be written as zeros.
-    auto request_unit = [&](__amdgpu_buffer_rsrc_t buf, const char* base, const int (&off)[JW], int t, int unit_off) {
+    auto request_unit = [&](__amdgpu_buffer_rsrc_t buf, const char* base, const auto& off, int t, int unit_off) {
+        constexpr int J = sizeof(off) / sizeof(int);
         if (t < full_tiles) {
 #pragma unroll
-            for (int j = 0; j < JW; ++j) request_part(buf, off, t, unit_off, j);
+            for (int j = 0; j < J; ++j) request_part(buf, off, t, unit_off, j);
         } else {
 #pragma unroll
-            for (int j = 0; j < JW; ++j) {
-                const int row = (JW * wave + j) * 8 + (lane >> 3);
+            for (int j = 0; j < J; ++j) {
+                const int row = (J * wave + j) * 8 + (lane >> 3);
                 const int ck = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
                 uint4 v = make_uint4(0, 0, 0, 0);
                 if (static_cast<int64_t>(t) * BK + ck < K)
                     v = *reinterpret_cast<const uint4*>(base + off[j] + static_cast<int64_t>(t) * (BK * 2));
-                *reinterpret_cast<uint4*>(dma_dst + unit_off + j * 1024 + lane * 16) = v;
+                *reinterpret_cast<uint4*>(lds + unit_off + (J * wave + j) * 1024 + lane * 16) = v;
             }
         }
     };
@@ -186,6 +199,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
             fb[i - TN] = *reinterpret_cast<const bf16x8*>(xt + off_x + (i - TN) * (32 * BK * 2) + sw);
     };
 
+    constexpr int kGapW = (TN * TM) / JW_W, kGapX = (TN * TM) / JW_X;   // MFMAs from one request instruction to the next
     auto unit_off = [](int slot) { return (slot >= kUnits ? slot - kUnits : slot) * kUnitBytes; };
     int s0 = 0;   // ring slot of W(t); X(t), W(t+1), X(t+1), W(t+2) follow
     bf16x8 fa[2][TN], fb[2][TM];
@@ -210,7 +224,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
                 const int a = i / TM, b = i % TM;
                 acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][a], fb[ks & 1][b], acc[a][b], 0, 0, 0);
                 if (i < TN + TM) read_frag(wt, xt, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1], i);
-                if (STEADY && ks == 0 && (i & 1) && (i >> 1) < JW) request_part(buf_w, off_gw, t + 2, w2_off, i >> 1);
+                if (STEADY && ks == 0 && i % kGapW == kGapW - 1 && i / kGapW < JW_W) request_part(buf_w, off_gw, t + 2, w2_off, i / kGapW);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -218,7 +232,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
         // flight) and every LDS read issued so far -- all of tile t's -- has
         // returned; the barrier extends both to the workgroup, so tile t+1 may
         // be read and tile t's slots may be overwritten.
-        __builtin_amdgcn_s_waitcnt(STEADY ? wait_vm_lgkm0(JW) : wait_vm_lgkm0(0));
+        __builtin_amdgcn_s_waitcnt(STEADY ? wait_vm_lgkm0(JW_W) : wait_vm_lgkm0(0));
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         if (!STEADY && t + 2 < ktiles) request_unit(buf_x, base_x, off_gx, t + 2, x2_off);
@@ -228,13 +242,13 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
             acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][a], fb[1][b], acc[a][b], 0, 0, 0);
             // Past the last tile these reads fetch stale LDS contents that are never used.
             if (i < TN + TM) read_frag(wn1, xn1, 0, fa[0], fb[0], i);
-            if (STEADY && (i & 1) && (i >> 1) < JW) request_part(buf_x, off_gx, t + 2, x2_off, i >> 1);
+            if (STEADY && i % kGapX == kGapX - 1 && i / kGapX < JW_X) request_part(buf_x, off_gx, t + 2, x2_off, i / kGapX);
             __builtin_amdgcn_sched_barrier(0);
         }
         s0 = s0 + 2 >= kUnits ? s0 + 2 - kUnits : s0 + 2;
     };
 
-    static_assert(TN * TM >= 2 * JW, "not enough MFMAs in a k-step to spread the requests");
+    static_assert(TN * TM >= JW_W && TN * TM >= JW_X, "not enough MFMAs in a k-step to spread the requests");
     request_unit(buf_w, base_w, off_gw, 0, 0);
     request_unit(buf_x, base_x, off_gx, 0, kUnitBytes);
     if (ktiles > 1) {
@@ -264,10 +278,12 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
         // row pitch 64 TN bytes, the 16-byte chunk index XOR-ed with a function
         // of the row so that neither the 8-byte writes (32 rows, one column
         // group) nor the 16-byte reads (whole rows) pile up on banks.
-        constexpr int kPitch = TN * 64;              // bytes of one row of the block
-        constexpr int kChunks = TN * 4;              // 16-byte chunks per row
-        constexpr int kRowsPerPass = 64 / kChunks;   // rows one read instruction covers
-        auto swz = [](int row) { return TN == 2 ? ((row >> 1) & 7) : (row & (kChunks - 1)); };
+        constexpr int kChunks = TN * 4;              // 16-byte chunks per row of the block
+        constexpr bool kPow2 = (kChunks & (kChunks - 1)) == 0;
+        // A power-of-two row is swizzled; any other row length is padded by one
+        // chunk instead, which staggers consecutive rows over the banks.
+        constexpr int kPitch = kPow2 ? TN * 64 : TN * 64 + 16;
+        auto swz = [](int row) { return !kPow2 ? 0 : kChunks == 8 ? ((row >> 1) & 7) : (row & (kChunks - 1)); };
         __syncthreads();   // every wavefront is done with the operand stages (and every request has landed)
         char* region = lds + wave * (TM * 32 * kPitch);
 #pragma unroll
@@ -297,12 +313,13 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
         // LDS operations of one wavefront complete in order, so its reads below
         // see its writes above; no other wavefront touches this region.
         asm volatile("" ::: "memory");
-        const int chunk = lane % kChunks;
-        const int64_t n = n0 + wn + chunk * 8;
+        static_assert((TM * 32 * kChunks) % 64 == 0, "block does not split into whole wavefront passes");
 #pragma unroll 4
-        for (int r0 = 0; r0 < TM * 32; r0 += kRowsPerPass) {
-            const int row = r0 + lane / kChunks;
+        for (int p = 0; p < TM * 32 * kChunks / 64; ++p) {
+            const int idx = p * 64 + lane;
+            const int row = idx / kChunks, chunk = idx % kChunks;
             const int64_t m = m0 + wm + row;
+            const int64_t n = n0 + wn + chunk * 8;
             const uint4 v = *reinterpret_cast<const uint4*>(region + row * kPitch + ((chunk ^ swz(row)) << 4));
             if (m >= M || n >= N) continue;
             uint16_t* dst = y + m * ldy + n;
@@ -368,25 +385,59 @@ extern "C" int ddl_linear_bf16(const void* x, const void* w, const void* bias, v
     if (!aligned_to(y, 2) || (bias && !aligned_to(bias, 2))) return fail(DDL_E_ALIGN, "linear: y / bias misaligned");
     if (ldx > 0x3FFFFF || ldw > 0x3FFFFF || K > 0x3FFFFFFF)
         return fail(DDL_E_UNSUPP, "linear: row pitch above 2^22 elements or K above 2^30");   // 32-bit byte offsets inside a tile
-    const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-    if (tiles_m * tiles_n > 0x7FFFFFFFll || tiles_m > 0x7FFFFFll || tiles_n > 0x7FFFFFll)
-        return fail(DDL_E_UNSUPP, "linear: too many output tiles");
     // 2: rows of y can be stored 16 bytes at a time, 1: 8 bytes, 0: element by element
     const int vec_store = (ldy % 8 == 0 && aligned_to(y, 16)) ? 2 : (ldy % 4 == 0 && aligned_to(y, 8)) ? 1 : 0;
-    auto launch = [&](auto kernel, int threads) -> int {
-        static bool attr_done = false;   // the attribute sticks to the function; set it on first use
-        if (!attr_done) {
+    const uint16_t* const xp = static_cast<const uint16_t*>(x);
+    const uint16_t* const wp = static_cast<const uint16_t*>(w);
+    const uint16_t* const bp = static_cast<const uint16_t*>(bias);
+    uint16_t* const yp = static_cast<uint16_t*>(y);
+
+    // Columns [n_begin, n_begin + n_count) of the output with tiles of 256 x bn.
+    auto launch = [&](auto kernel, bool& attr_done, int threads, int bn, int64_t n_begin, int64_t n_count) -> int {
+        const int64_t tiles_m = (M + 255) / 256, tiles_n = (n_count + bn - 1) / bn;
+        if (tiles_m * tiles_n > 0x7FFFFFFFll || tiles_m > 0x7FFFFFll || tiles_n > 0x7FFFFFll)
+            return fail(DDL_E_UNSUPP, "linear: too many output tiles");
+        if (!attr_done) {   // the attribute sticks to the function; set it on first use
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
             if (e != hipSuccess) return fail(static_cast<int>(e), "linear: cannot reserve %d bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
             attr_done = true;
         }
         hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(tiles_m * tiles_n)), dim3(threads), kLdsBytes,
-                           static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w),
-                           static_cast<const uint16_t*>(bias), static_cast<uint16_t*>(y), M, N, K, ldx, ldw, ldy,
-                           static_cast<int>(tiles_m), static_cast<int>(tiles_n), vec_store);
-        return 0;
+                           static_cast<hipStream_t>(stream), xp, wp + n_begin * ldw, bp ? bp + n_begin : nullptr, yp + n_begin, M,
+                           n_count, K, ldx, ldw, ldy, static_cast<int>(tiles_m), static_cast<int>(tiles_n), vec_store);
+        return check_launch("linear_bf16_kernel");
     };
-    const int rc = launch(linear_bf16_kernel<2, 4>, 512);
-    if (rc) return rc;
-    return check_launch("linear_bf16_kernel");
+    static bool wide_ready = false, narrow_ready = false;
+    auto wide = [&](int64_t n_begin, int64_t n_count) { return launch(linear_bf16_kernel<2, 4, 4, 2>, wide_ready, 512, 256, n_begin, n_count); };
+    auto narrow = [&](int64_t n_begin, int64_t n_count) { return launch(linear_bf16_kernel<4, 2, 2, 3>, narrow_ready, 512, 192, n_begin, n_count); };
+
+    // One workgroup per CU is resident, so the tiles run in rounds of one per
+    // CU and a last round that is only partly filled costs as much as a full
+    // one.  When it pays, the columns are split: whole rounds of 256-wide
+    // tiles first, the rest with 192-wide tiles, whose rounds are shorter.
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1)
+            n = 256;
+        cus = n;
+    }
+    const int64_t tiles_m = (M + 255) / 256, cols = (N + 255) / 256;
+    auto rounds = [&](int64_t tiles) { return (tiles + cus - 1) / cus; };
+    const int64_t cost_wide = rounds(tiles_m * cols) * 256;
+    int64_t best_cost = cost_wide, best_split = cols;   // columns of 256 given to the wide kernel
+    for (int64_t c = cols - 1; c >= 0 && c >= cols - 16; --c) {
+        const int64_t rest = N - c * 256;
+        const int64_t cost = rounds(tiles_m * c) * 256 + rounds(tiles_m * ((rest + 191) / 192)) * 192;
+        if (cost < best_cost) {
+            best_cost = cost;
+            best_split = c;
+        }
+    }
+    if (best_split == cols) return wide(0, N);
+    if (best_split > 0) {
+        const int rc = wide(0, best_split * 256);
+        if (rc) return rc;
+    }
+    return narrow(best_split * 256, N - best_split * 256);
 }
