@@ -45,18 +45,30 @@ __device__ inline float block_sum(float v, float* scratch) {
 // Mean-of-local-means / mean-of-local-variances of nn/layernorm.py:230-247,
 // written on the gathered {mean_p, M2_p}:
 //   mean((x-mean)^2 over worker p) = (M2_p + n_p (mean_p-mean)^2) / n_p.
+// A whole wavefront works on one row: lane p holds worker p's pair (`first`,
+// loaded by the caller so that it travels together with the row itself; zeros
+// for lanes >= nparts) and 1/n_p; workers beyond the 64th are fetched here.
+__device__ inline float2 load_part(const float* __restrict__ part_stats, int64_t rows, int64_t r, int p) {
+    return reinterpret_cast<const float2*>(part_stats)[static_cast<int64_t>(p) * rows + r];
+}
+
 __device__ inline void combine_parts(const float* __restrict__ part_stats, int64_t rows, int64_t r, int nparts,
-                                     const PartCounts& pc, float eps, float* mean_out, float* rstd_out) {
-    float msum = 0.f;
-    for (int p = 0; p < nparts; ++p) msum += part_stats[(static_cast<int64_t>(p) * rows + r) * 2];
-    const float mean = msum / static_cast<float>(nparts);
+                                     const PartCounts& pc, float eps, int lane, float2 first, float first_inv_n,
+                                     float* mean_out, float* rstd_out) {
+    float msum = lane < nparts ? first.x : 0.f;
+    for (int p = lane + kWave; p < nparts; p += kWave) msum += load_part(part_stats, rows, r, p).x;
+    const float mean = wave_sum(msum) / static_cast<float>(nparts);
     float vsum = 0.f;
-    for (int p = 0; p < nparts; ++p) {
-        const float* s = part_stats + (static_cast<int64_t>(p) * rows + r) * 2;
-        const float d = s[0] - mean;
-        vsum += s[1] * pc.inv_n[p] + d * d;
+    if (lane < nparts) {
+        const float d = first.x - mean;
+        vsum = first.y * first_inv_n + d * d;
     }
-    const float var = vsum / static_cast<float>(nparts);
+    for (int p = lane + kWave; p < nparts; p += kWave) {
+        const float2 s = load_part(part_stats, rows, r, p);
+        const float d = s.x - mean;
+        vsum += s.y * pc.inv_n[p] + d * d;
+    }
+    const float var = wave_sum(vsum) / static_cast<float>(nparts);
     *mean_out = mean;
     *rstd_out = 1.0f / sqrtf(var + eps);
 }
@@ -125,6 +137,16 @@ __global__ __launch_bounds__(kBlock) void ln_norm_rows(const float* __restrict__
             }
         }
     }
+    // Everything this wavefront reads is requested before anything is used:
+    // the gathered statistics of its rows (lane p fetches worker p's pair) and
+    // the rows themselves.
+    float2 ps[RPW];
+    const float inv_n = lane < nparts ? pc.inv_n[lane] : 0.f;
+#pragma unroll
+    for (int i = 0; i < RPW; ++i) {
+        const int64_t r = r0 + i;
+        ps[i] = (r < rows && lane < nparts) ? load_part(part_stats, rows, r, lane) : make_float2(0.f, 0.f);
+    }
     float4 v[RPW][NV];
 #pragma unroll
     for (int i = 0; i < RPW; ++i) {
@@ -140,7 +162,7 @@ __global__ __launch_bounds__(kBlock) void ln_norm_rows(const float* __restrict__
         const int64_t r = r0 + i;
         if (r >= rows) continue;
         float mean, rstd;
-        combine_parts(part_stats, rows, r, nparts, pc, eps, &mean, &rstd);
+        combine_parts(part_stats, rows, r, nparts, pc, eps, lane, ps[i], inv_n, &mean, &rstd);
         if (lane == 0) {
             if (mean_out) mean_out[r] = mean;
             if (rstd_out) rstd_out[r] = rstd;
@@ -202,7 +224,10 @@ __global__ __launch_bounds__(kBlock) void ln_norm_stream(const float* __restrict
                                                          float* __restrict__ rstd_out) {
     for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
         float mean, rstd;
-        combine_parts(part_stats, rows, r, nparts, pc, eps, &mean, &rstd);
+        const int lane = threadIdx.x & (kWave - 1);
+        combine_parts(part_stats, rows, r, nparts, pc, eps, lane,
+                      lane < nparts ? load_part(part_stats, rows, r, lane) : make_float2(0.f, 0.f),
+                      lane < nparts ? pc.inv_n[lane] : 0.f, &mean, &rstd);
         if (threadIdx.x == 0) {
             if (mean_out) mean_out[r] = mean;
             if (rstd_out) rstd_out[r] = rstd;
@@ -281,6 +306,8 @@ int ddl_ln_normalize_affine_f32(const float* x, int64_t rows, int64_t cols, int6
     if (rows == 0) return 0;
     if (!x || !y || !part_stats || !part_cols) return fail(DDL_E_ARG, "ln normalize: null pointer");
     if (rows > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "ln normalize: more than 2^31 rows");
+    if (!aligned_to(x, 4) || !aligned_to(y, 4) || !aligned_to(part_stats, 8))
+        return fail(DDL_E_ALIGN, "ln normalize: x, y must be 4-byte and the statistics 8-byte aligned");
     PartCounts pc{};
     for (int p = 0; p < nparts; ++p) {
         if (part_cols[p] < 1) return fail(DDL_E_ARG, "ln normalize: worker %d holds %lld columns", p, (long long)part_cols[p]);

@@ -84,11 +84,12 @@ def test_layernorm_config1_rank0(ops):
 
 
 @pytest.mark.parametrize("cols", [[4, 4], [64, 64, 64], [300, 212], [1000, 24], [2048], [7, 9], [4100, 4100],
-                                  [20000, 100]])
+                                  [20000, 100], [8] * 70, [4] * 200])
 @pytest.mark.parametrize("affine", [True, False])
 def test_layernorm_shapes_and_paths(ops, cols, affine):
     """Register path (aligned, <= 2048 columns), LDS-staged path (unaligned or
-    long rows), streaming path (rows longer than the LDS stage), unequal widths."""
+    long rows), streaming path (rows longer than the LDS stage), unequal widths,
+    more workers per row than a wavefront has lanes."""
     rng = np.random.default_rng(sum(cols))
     rows = 37
     shards = [(rng.standard_normal((rows, c)) * 3 + 1.5).astype(np.float32) for c in cols]
