@@ -6,8 +6,8 @@
 //                -> combined mean / var -> y = (x-mean)*rstd*gamma+beta
 //
 // Rows of up to 2048 columns live in registers: one wavefront owns a row, each
-// lane holds float4 pieces, sums go through DPP/shuffle butterflies, and several
-// rows per wavefront are in flight to cover HBM latency.  Longer (or unaligned)
+// lane holds float4 pieces, sums go through DPP/shuffle butterflies; a long
+// input keeps two rows per wavefront in flight.  Longer (or unaligned)
 // rows are staged once in LDS by a 256-thread workgroup and reduced from there.
 #include "ddl_common.h"
 
@@ -246,9 +246,13 @@ bool rows_vectorizable(const void* p, int64_t cols, int64_t ld) {
     return cols % 4 == 0 && ld % 4 == 0 && cols <= 2048 && aligned_to(p, 16);
 }
 
-template <int NV>
-int launch_stats(const float* x, int64_t rows, int cols, int64_t ld, float* stats, hipStream_t s) {
-    constexpr int RPW = NV <= 2 ? 4 : (NV <= 4 ? 2 : 1);
+// Rows a wavefront keeps in flight.  Few rows per wavefront mean more
+// wavefronts, which is what a small input needs to occupy the whole chip; two
+// rows per wavefront stream a long input a little faster.
+constexpr int64_t kSmallRows = 65536;
+
+template <int NV, int RPW>
+int launch_stats_rpw(const float* x, int64_t rows, int cols, int64_t ld, float* stats, hipStream_t s) {
     const int64_t waves = (rows + RPW - 1) / RPW;
     const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     hipLaunchKernelGGL((ln_stats_rows<NV, RPW>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, s, x, rows, cols, ld, stats);
@@ -256,10 +260,15 @@ int launch_stats(const float* x, int64_t rows, int cols, int64_t ld, float* stat
 }
 
 template <int NV>
-int launch_norm(const float* x, int64_t rows, int cols, int64_t ld, const float* ps, int nparts, const PartCounts& pc,
-                const float* gamma, const float* beta, float eps, float* y, int64_t ldy, float* mo, float* ro,
-                hipStream_t s) {
-    constexpr int RPW = NV <= 2 ? 4 : (NV <= 4 ? 2 : 1);
+int launch_stats(const float* x, int64_t rows, int cols, int64_t ld, float* stats, hipStream_t s) {
+    if (NV <= 2 && rows > kSmallRows) return launch_stats_rpw<NV, 2>(x, rows, cols, ld, stats, s);
+    return launch_stats_rpw<NV, 1>(x, rows, cols, ld, stats, s);
+}
+
+template <int NV, int RPW>
+int launch_norm_rpw(const float* x, int64_t rows, int cols, int64_t ld, const float* ps, int nparts, const PartCounts& pc,
+                    const float* gamma, const float* beta, float eps, float* y, int64_t ldy, float* mo, float* ro,
+                    hipStream_t s) {
     const int64_t waves = (rows + RPW - 1) / RPW;
     const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (gamma)
@@ -269,6 +278,14 @@ int launch_norm(const float* x, int64_t rows, int cols, int64_t ld, const float*
         hipLaunchKernelGGL((ln_norm_rows<NV, RPW, false>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, s, x, rows,
                            cols, ld, ps, nparts, pc, gamma, beta, eps, y, ldy, mo, ro);
     return check_launch("ln_norm_rows");
+}
+
+template <int NV>
+int launch_norm(const float* x, int64_t rows, int cols, int64_t ld, const float* ps, int nparts, const PartCounts& pc,
+                const float* gamma, const float* beta, float eps, float* y, int64_t ldy, float* mo, float* ro,
+                hipStream_t s) {
+    if (NV <= 2 && rows > kSmallRows) return launch_norm_rpw<NV, 2>(x, rows, cols, ld, ps, nparts, pc, gamma, beta, eps, y, ldy, mo, ro, s);
+    return launch_norm_rpw<NV, 1>(x, rows, cols, ld, ps, nparts, pc, gamma, beta, eps, y, ldy, mo, ro, s);
 }
 
 }  // namespace
