@@ -65,6 +65,8 @@ SIGNATURES = {
                                      c_void_p, c_void_p]),
     "ddl_linear_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                 c_int64, c_void_p]),
+    "ddl_transpose_2d": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),
+    "ddl_colsum_bf16": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_void_p]),
 }
 
 _lib = None

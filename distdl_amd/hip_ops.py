@@ -317,3 +317,86 @@ def linear_bf16(x, weight, bias=None, out=None):
                                      x2.stride(0) if m > 1 else k, weight.stride(0) if n > 1 else k, n, _stream())
     _lib.check(rc, "ddl_linear_bf16")
     return out
+
+
+def _round_up(n, m):
+    return (n + m - 1) // m * m
+
+
+def transpose_2d(src, ld_dst=None):
+    """``src[rows, cols]`` (16-bit elements, row stride arbitrary) -> a new
+    ``[cols, ld_dst]`` tensor whose first ``rows`` columns hold the transpose;
+    any further columns are zero."""
+    _require_gpu(src)
+    if src.dim() != 2 or src.element_size() != 2:
+        raise ValueError("transpose_2d: a 2-D tensor of 16-bit elements is required")
+    if src.stride(1) != 1 and src.shape[1] > 1:
+        src = src.contiguous()
+    rows, cols = src.shape
+    ld_dst = rows if ld_dst is None else ld_dst
+    alloc = torch.empty if ld_dst == rows else torch.zeros
+    dst = alloc((cols, ld_dst), dtype=src.dtype, device=src.device)
+    rc = _lib.load().ddl_transpose_2d(src.data_ptr(), dst.data_ptr(), rows, cols, src.stride(0) if rows > 1 else cols,
+                                      ld_dst, 2, _stream())
+    _lib.check(rc, "ddl_transpose_2d")
+    return dst
+
+
+def colsum_bf16(a):
+    """Column sums of a 2-D bf16 tensor, fp32 accumulation, bf16 result."""
+    _require_gpu(a)
+    if a.dim() != 2 or a.dtype != torch.bfloat16:
+        raise ValueError("colsum_bf16: a 2-D bfloat16 tensor is required")
+    if a.stride(1) != 1 and a.shape[1] > 1:
+        a = a.contiguous()
+    rows, cols = a.shape
+    out = torch.empty(cols, dtype=torch.bfloat16, device=a.device)
+    splits = max(1, min(64, (rows + 127) // 128))
+    work = torch.empty(splits * max(cols, 1), dtype=torch.float32, device=a.device)
+    rc = _lib.load().ddl_colsum_bf16(a.data_ptr(), rows, cols, a.stride(0) if rows > 1 else cols, out.data_ptr(),
+                                     work.data_ptr(), work.numel(), _stream())
+    _lib.check(rc, "ddl_colsum_bf16")
+    return out
+
+
+def linear_bf16_backward(x, weight, grad_output, need_input=True, need_weight=True, need_bias=True):
+    """Adjoint of :func:`linear_bf16`: ``(dx, dw, db)`` for ``y = x @ weight.T + bias``
+    (entries not asked for are None).  The operands that are not contiguous
+    along the reduction dimension are transposed into temporaries whose row
+    pitch is padded to a multiple of 8 with zeros, then the same GEMM runs."""
+    _require_gpu(x, weight, grad_output)
+    n, k = weight.shape
+    x2 = x.reshape(-1, k)
+    dy = grad_output.reshape(-1, n)
+    if dy.stride(1) != 1 and n > 1:
+        dy = dy.contiguous()
+    m = x2.shape[0]
+    dx = dw = db = None
+    if need_input:
+        # dx[m, k] = sum_n dy[m, n] w[n, k]: operands dy[M, N] and wT[K, N]
+        np8 = _round_up(n, 8)
+        w_t = transpose_2d(weight, np8)                       # [K, np8], padding columns zero
+        dy_p = dy
+        if np8 != n or (m > 1 and dy.stride(0) % 8 != 0) or dy.data_ptr() % 16 != 0:
+            dy_p = torch.zeros((m, np8), dtype=dy.dtype, device=dy.device)
+            full = [slice(0, m), slice(0, n)]
+            copy_box(dy, full, dy_p, full)
+        dx = _linear_padded(dy_p, w_t, m, k, np8).reshape(x.shape)
+    if need_weight:
+        # dw[n, k] = sum_m dy[m, n] x[m, k]: operands dyT[N, M] and xT[K, M]
+        mp8 = _round_up(m, 8)
+        dy_t = transpose_2d(dy, mp8)                          # [N, mp8]
+        x_t = transpose_2d(x2, mp8)                           # [K, mp8]
+        dw = _linear_padded(dy_t, x_t, n, k, mp8)
+    if need_bias:
+        db = colsum_bf16(dy)
+    return dx, dw, db
+
+
+def _linear_padded(a, b, m, n, k_padded):
+    """``a[m, k_padded] @ b[n, k_padded].T`` where the padding columns are zero."""
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    rc = _lib.load().ddl_linear_bf16(a.data_ptr(), b.data_ptr(), None, out.data_ptr(), m, n, k_padded,
+                                     a.stride(0) if m > 1 else k_padded, b.stride(0) if n > 1 else k_padded, n, _stream())
+    _lib.check(rc, "ddl_linear_bf16")
+    return out

@@ -15,14 +15,22 @@ from .sum_reduce import SumReduce
 
 
 class _LinearShard(torch.autograd.Function):
+    """``F.linear`` and its adjoint (dx = dy w, dw = dy^T x, db = column sums of
+    dy) on the HIP kernels."""
 
     @staticmethod
     def forward(ctx, x, weight, bias):
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias = bias is not None
         return hip_ops.linear_bf16(x.detach(), weight.detach(), None if bias is None else bias.detach())
 
     @staticmethod
     def backward(ctx, grad_output):
-        raise NotImplementedError("the backward pass of the linear shard is not part of this build")
+        x, weight = ctx.saved_tensors
+        need_x, need_w, need_b = ctx.needs_input_grad
+        dx, dw, db = hip_ops.linear_bf16_backward(x.detach(), weight.detach(), grad_output.detach().to(torch.bfloat16),
+                                                  need_x, need_w, need_b and ctx.has_bias)
+        return dx, dw, db
 
 
 def linear_shard(x, weight, bias):

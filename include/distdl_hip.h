@@ -211,6 +211,26 @@ int ddl_linear_bf16(const void* x, const void* w, const void* bias, void* y,
                     int64_t M, int64_t N, int64_t K,
                     int64_t ldx, int64_t ldw, int64_t ldy, void* stream);
 
+/* Adjoint of the shard GEMM (what autograd runs for the two calls above):
+ *   dx = dy . w,   dw = dy^T . x,   db = column sums of dy.
+ * ddl_linear_bf16 multiplies operands that are contiguous along the reduction
+ * dimension, so the host transposes w (for dx), dy and x (for dw) with
+ * ddl_transpose_2d into caller-provided buffers and calls ddl_linear_bf16 again:
+ *   dx[M,K] = linear(dy[M,N],   wT[K,N])      dw[N,K] = linear(dyT[N,M], xT[K,M]).
+ *
+ * ddl_transpose_2d:  dst[c, r] = src[r, c] for r < rows, c < cols; 2-byte
+ * elements only (elem_size = 2); ld_src >= cols, ld_dst >= rows. */
+int ddl_transpose_2d(const void* src, void* dst, int64_t rows, int64_t cols,
+                     int64_t ld_src, int64_t ld_dst, int elem_size, void* stream);
+
+/* out[c] = bf16( sum over r < rows of a[r, c] ), fp32 accumulation, for the
+ * bias gradient.  `workspace` is device memory for at least `cols` floats
+ * (up to 64 * cols are used: one row of partial sums per row split); its
+ * contents on entry do not matter. */
+int ddl_colsum_bf16(const void* a, int64_t rows, int64_t cols, int64_t ld,
+                    void* out, float* workspace, int64_t workspace_elems,
+                    void* stream);
+
 #ifdef __cplusplus
 }
 #endif

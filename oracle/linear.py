@@ -32,3 +32,16 @@ def linear(x_bits, w_bits, bias_bits=None, dtype=np.float32):
     if bias_bits is not None:
         y = y + bf16_bits_to_f32(bias_bits).astype(dtype)
     return y.reshape(x.shape[:-1] + (w.shape[0],))
+
+
+def linear_backward(x_bits, w_bits, dy_bits, dtype=np.float64):
+    """Adjoint of ``linear`` on bf16 bit patterns: returns ``(dx, dw, db)`` in
+    ``dtype`` (exact sums, not rounded to bf16):
+        dx = dy @ w        dw = dy.T @ x        db = dy.sum(0)
+    which is what autograd derives for torch.nn.functional.linear
+    (reference call sites nn/linear.py:103, nn/linear_ag.py:486).  Pinned by
+    torch autograd on the same operands in tests/test_oracle_golden.py."""
+    x = bf16_bits_to_f32(x_bits).astype(dtype)
+    w = bf16_bits_to_f32(w_bits).astype(dtype)
+    dy = bf16_bits_to_f32(dy_bits).astype(dtype)
+    return dy @ w, dy.T @ x, dy.sum(axis=0)

@@ -315,6 +315,80 @@ def test_linear_config4_rank0(ops):
     assert float(rel.max()) <= LIN_RTOL
 
 
+@pytest.mark.parametrize("rows,cols", [(1, 1), (64, 64), (65, 63), (300, 130), (1000, 8), (7, 513)])
+def test_transpose_2d_is_bit_exact(ops, rows, cols):
+    gen = torch.Generator().manual_seed(rows * 1000 + cols)
+    src = torch.randint(-32768, 32767, (rows, cols), generator=gen, dtype=torch.int16)
+    got = ops.transpose_2d(src.cuda())
+    assert torch.equal(got.cpu(), src.t().contiguous())
+    # padded pitch: the extra columns are zero
+    ld = (rows + 7) // 8 * 8 + 8
+    got = ops.transpose_2d(src.cuda(), ld)
+    assert torch.equal(got[:, :rows].cpu(), src.t().contiguous()) and (got[:, rows:] == 0).all()
+    # a strided source view
+    wide = torch.randint(-32768, 32767, (rows, cols + 5), generator=gen, dtype=torch.int16).cuda()
+    assert torch.equal(ops.transpose_2d(wide[:, 2:2 + cols]).cpu(), wide[:, 2:2 + cols].cpu().t().contiguous())
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (5, 3), (128, 64), (129, 65), (8192, 200), (3000, 1000)])
+def test_colsum_bf16(ops, rows, cols):
+    gen = torch.Generator().manual_seed(rows + cols)
+    a = torch.randn(rows, cols, generator=gen).to(torch.bfloat16)
+    got = ops.colsum_bf16(a.cuda()).cpu().double()
+    exact = a.double().sum(0)
+    # fp32 accumulation of bf16 values, one bf16 rounding of the result
+    tol = 2.0 ** -8 * exact.abs() + 1e-5 * a.double().abs().sum(0)
+    assert ((got - exact).abs() <= tol).all()
+    # small integers: exact
+    ai = torch.randint(-2, 3, (rows, cols), generator=gen).to(torch.bfloat16)
+    want = ai.double().sum(0)
+    if want.abs().max() <= 256:
+        assert torch.equal(ops.colsum_bf16(ai.cuda()).cpu().double(), want)
+
+
+@pytest.mark.parametrize("M,N,K", [(8, 8, 8), (96, 80, 128), (300, 200, 72), (257, 36, 40), (5, 3, 16), (64, 1000, 256)])
+def test_linear_backward_small_integer_cases_are_exact(ops, M, N, K):
+    """dx = dy w, dw = dy^T x, db = sum dy with small integers: every sum is
+    exact in fp32 and representable in bf16, so the results must be the exact
+    integers -- a wrong transpose or pitch shows at once."""
+    gen = torch.Generator().manual_seed(M * 5 + N * 3 + K)
+    x = torch.randint(-1, 2, (M, K), generator=gen).to(torch.bfloat16)
+    w = torch.randint(-1, 2, (N, K), generator=gen).to(torch.bfloat16)
+    dy = torch.randint(-1, 2, (M, N), generator=gen).to(torch.bfloat16)
+    # keep the sums below 2^8: thin out dy and w
+    dy = dy * (torch.rand(M, N, generator=gen) < min(1.0, 40.0 / max(M, N))).to(torch.bfloat16)
+    w = w * (torch.rand(N, K, generator=gen) < min(1.0, 40.0 / N)).to(torch.bfloat16)
+    dx, dw, db = ops.linear_bf16_backward(x.cuda(), w.cuda(), dy.cuda())
+    want_dx, want_dw, want_db = o_lin.linear_backward(bits16(x), bits16(w), bits16(dy))
+    assert max(np.abs(want_dx).max(), np.abs(want_dw).max(), np.abs(want_db).max()) <= 256
+    assert np.array_equal(dx.cpu().double().numpy(), want_dx)
+    assert np.array_equal(dw.cpu().double().numpy(), want_dw)
+    assert np.array_equal(db.cpu().double().numpy(), want_db)
+
+
+def test_linear_shard_autograd_matches_torch(ops):
+    """The reference's layer runs torch autograd through F.linear; the same
+    gradients must come out of the HIP path (bf16 tolerance), including through
+    a batch-shaped input and with no bias."""
+    from distdl_amd.nn.linear import linear_shard
+    gen = torch.Generator().manual_seed(9)
+    x = torch.randn(3, 50, 96, generator=gen).to(torch.bfloat16)
+    w = (0.05 * torch.randn(72, 96, generator=gen)).to(torch.bfloat16)
+    b = (0.05 * torch.randn(72, generator=gen)).to(torch.bfloat16)
+    dy = torch.randn(3, 50, 72, generator=gen).to(torch.bfloat16)
+    for use_bias in (True, False):
+        xg, wg = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+        bg = b.cuda().requires_grad_(True) if use_bias else None
+        linear_shard(xg, wg, bg).backward(dy.cuda())
+        xr, wr = x.double().requires_grad_(True), w.double().requires_grad_(True)
+        br = b.double().requires_grad_(True) if use_bias else None
+        F.linear(xr, wr, br).backward(dy.double())
+        for got, ref in ((xg.grad, xr.grad), (wg.grad, wr.grad)) + (((bg.grad, br.grad),) if use_bias else ()):
+            assert got.dtype == torch.bfloat16 and got.shape == ref.shape
+            err = (got.cpu().double() - ref).abs()
+            assert (err <= LIN_RTOL * (ref.abs() + ref.abs().mean())).all()
+
+
 def test_linear_layers_forward(ops):
     """DistributedLinear and DistributedLinearAllGather (solo rank 0 of 8,
     weights split on out_features) call the same kernel."""

@@ -345,3 +345,24 @@ def test_linear_oracle_matches_torch_and_exact_cases():
     wi = torch.randint(-4, 5, (9, 16)).float()
     exact = (xi.double() @ wi.double().T).numpy()
     assert np.array_equal(o_lin.linear(bits(xi.to(torch.bfloat16)), bits(wi.to(torch.bfloat16))), exact)
+
+
+def test_linear_backward_oracle_matches_torch_autograd():
+    """The adjoint restatement against what autograd derives for F.linear, on
+    float64 copies of the same bf16 values (sums exact enough to compare at 1e-12)."""
+    torch.manual_seed(4)
+    x = torch.randn(11, 24).to(torch.bfloat16)
+    w = (0.1 * torch.randn(7, 24)).to(torch.bfloat16)
+    b = torch.randn(7).to(torch.bfloat16)
+    dy = torch.randn(11, 7).to(torch.bfloat16)
+
+    def bits(t):
+        return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+    xd, wd, bd = (t.double().requires_grad_(True) for t in (x, w, b))
+    F.linear(xd, wd, bd).backward(dy.double())
+    dx, dw, db = o_lin.linear_backward(bits(x), bits(w), bits(dy))
+    assert np.allclose(dx, xd.grad.numpy(), rtol=1e-12, atol=1e-12)
+    assert np.allclose(dw, wd.grad.numpy(), rtol=1e-12, atol=1e-12)
+    assert np.allclose(db, bd.grad.numpy(), rtol=1e-12, atol=1e-12)
+    # a transposed operand or a swapped product would break these shapes / values
+    assert dx.shape == (11, 24) and dw.shape == (7, 24) and db.shape == (7,)
