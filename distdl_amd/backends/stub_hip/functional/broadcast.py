@@ -1,8 +1,9 @@
-"""Broadcast stand-in.  The reference's broadcast (and its sum-reduce adjoint,
-backends/mpi_numpy/functional/broadcast.py:116-128, :213-221) is a collective
-and therefore outside this build; the forward is delegated to the transport
-(identity for a solo rank that owns the data, a copy from the owning rank thread
-under loopback) so that layers storing weights on a sub-grid work end to end."""
+"""Broadcast stand-in.  The reference's broadcast and its sum-reduce adjoint
+(backends/mpi_numpy/functional/broadcast.py:116-128, :213-221) are collectives
+and therefore outside this build; both directions are delegated to the
+transport (identity for a solo rank that owns the data; copies between rank
+threads, summed with the box kernel, under loopback) so that layers storing
+weights on a sub-grid work end to end, gradients included."""
 
 __all__ = ["BroadcastFunction"]
 
@@ -15,9 +16,17 @@ class BroadcastFunction(torch.autograd.Function):
     def forward(ctx, input, P_send, P_recv, preserve_batch=False, tag=None):
         if not (P_send.active or P_recv.active):
             return input
+        ctx.P_send, ctx.P_recv, ctx.tag = P_send, P_recv, tag
+        ctx.input_like = (tuple(input.shape), input.dtype, input.device)
         world = P_send._world if P_send._world is not None else P_recv._world
         return world.transport.broadcast(P_send, P_recv, input.detach(), tag=tag)
 
     @staticmethod
     def backward(ctx, grad_output):
-        raise NotImplementedError("the adjoint of Broadcast is a sum-reduce collective, not part of this build")
+        P_send, P_recv = ctx.P_send, ctx.P_recv
+        world = P_send._world if P_send._world is not None else P_recv._world
+        grad = world.transport.broadcast_adjoint(P_send, P_recv, grad_output.detach(), tag=ctx.tag)
+        if grad is None:
+            shape, dtype, device = ctx.input_like
+            grad = torch.zeros(shape, dtype=dtype, device=device)
+        return grad, None, None, None, None

@@ -105,6 +105,11 @@ class SoloTransport:
             return tensor
         raise TransportError("solo transport: the live rank is not a source of this broadcast")
 
+    def broadcast_adjoint(self, P_src, P_dst, grad, tag=None):
+        """The live rank owns the data; the gradients of the absent workers are
+        absent too."""
+        return grad if P_src.active else None
+
 
 # ---------------------------------------------------------------------------
 # Loopback
@@ -295,4 +300,31 @@ class LoopbackTransport:
                 raise TransportError("broadcast: no source worker matches this destination index")
             out = match.clone()
         self._allgather_obj(union, None, ("tbcast-done", tag))
+        return out
+
+    def broadcast_adjoint(self, P_src, P_dst, grad, tag=None):
+        """Sum-reduce: every worker of ``P_src`` receives the sum of the
+        gradients held by the workers of ``P_dst`` it was broadcast to; the
+        other workers receive None."""
+        from ... import hip_ops
+        union = P_src.create_partition_union(P_dst)
+        payload = (tuple(int(i) for i in P_dst.index), grad) if P_dst.active else None
+        everyone = self._allgather_obj(union, payload, ("tbcast-adj", tag))
+        out = None
+        if P_src.active:
+            mine = [int(i) for i in P_src.index]
+            src_shape = [int(s) for s in P_src.shape]
+            for item in everyone:
+                if item is None:
+                    continue
+                index, g = item
+                if not all(src_shape[d] == 1 or index[d] == mine[d] for d in range(len(src_shape))):
+                    continue
+                if out is None:
+                    out = g.clone()
+                else:
+                    full = [slice(0, int(n)) for n in g.shape]
+                    hip_ops.copy_box(g, full, out, full, accumulate=True)
+        # Nobody may reuse its gradient buffer before every source has summed it.
+        self._allgather_obj(union, None, ("tbcast-adj-done", tag))
         return out

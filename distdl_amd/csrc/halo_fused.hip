@@ -133,7 +133,6 @@ __global__ __launch_bounds__(kBlock) void halo_pad_kernel(const HaloArgs args_by
     constexpr int EPV = sizeof(T) >= 4 ? 16 / sizeof(T) : 1;   // elements per vector
     typedef typename VecType<T, EPV>::type V;
     constexpr int RPI = kWave / LPR;                            // rows per wavefront instruction
-    constexpr int kRowsPerPass = RPI * kWavesPerBlock;
 
     const int nd = a->nd;
     const int L = nd - 1, M = nd - 2;

@@ -1,0 +1,245 @@
+// Backward of the DistributedLayerNorm shard, fp32: what autograd derives from
+// the reference's forward (nn/layernorm.py:230-247, 295-309)
+//
+//   mean = allreduce(local mean) / P        var = allreduce(local mean((x-mean)^2)) / P
+//   xhat = (x - mean) rstd                  y = gamma xhat + beta
+//
+// Every element of worker p enters mean and var with weight a_p = 1 / (P n_p)
+// (n_p = columns held by p; the weights of a row add up to 1), which gives
+//
+//   g    = dy gamma
+//   S1   = sum over the whole row of g           S2 = sum over the whole row of g xhat
+//   dx   = rstd (g - a_p (S1 + xhat S2))
+//   dgamma[c] = sum over rows of dy xhat         dbeta[c] = sum over rows of dy
+//
+// S1 and S2 span all workers of the row, so the work is split like the forward:
+//   ln_bwd_partial   local {sum g, sum g xhat} per row      (one read of dy, x)
+//   -- the caller gathers the pairs of the P workers --
+//   ln_bwd_input     sums the gathered pairs, writes dx      (one read of dy, x)
+//   ln_bwd_params    column sums over the local rows, in row splits through a
+//                    workspace, for dgamma and dbeta
+// One wavefront owns a row and strides over its columns (float4 when the row is
+// aligned); nothing is kept between passes, so rows of any length work.
+#include "ddl_common.h"
+
+namespace ddl {
+namespace {
+
+constexpr int kWave = 64;
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / kWave;
+constexpr int kStrip = 64;     // columns per workgroup of the parameter kernel
+
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void ln_bwd_partial(const float* __restrict__ dy, const float* __restrict__ x, int64_t rows,
+                                                         int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                                         const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                         const float* __restrict__ gamma, float* __restrict__ sums) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + threadIdx.x / kWave;
+    if (r >= rows) return;
+    const float m = mean[r], rs = rstd[r];
+    const float* dyr = dy + r * ld_dy;
+    const float* xr = x + r * ld_x;
+    float s1 = 0.f, s2 = 0.f;
+    if (VEC) {
+        for (int64_t c = lane * 4; c < cols; c += kWave * 4) {
+            const float4 d = *reinterpret_cast<const float4*>(dyr + c);
+            const float4 v = *reinterpret_cast<const float4*>(xr + c);
+            float4 g = make_float4(1.f, 1.f, 1.f, 1.f);
+            if (gamma) g = *reinterpret_cast<const float4*>(gamma + c);
+            const float g0 = d.x * g.x, g1 = d.y * g.y, g2 = d.z * g.z, g3 = d.w * g.w;
+            s1 += (g0 + g1) + (g2 + g3);
+            s2 += (g0 * ((v.x - m) * rs) + g1 * ((v.y - m) * rs)) + (g2 * ((v.z - m) * rs) + g3 * ((v.w - m) * rs));
+        }
+    } else {
+        for (int64_t c = lane; c < cols; c += kWave) {
+            const float g = dyr[c] * (gamma ? gamma[c] : 1.f);
+            s1 += g;
+            s2 += g * ((xr[c] - m) * rs);
+        }
+    }
+    s1 = wave_sum(s1);
+    s2 = wave_sum(s2);
+    if (lane == 0) reinterpret_cast<float2*>(sums)[r] = make_float2(s1, s2);
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void ln_bwd_input(const float* __restrict__ dy, const float* __restrict__ x, int64_t rows,
+                                                       int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                                       const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                       const float* __restrict__ gamma, const float* __restrict__ part_sums,
+                                                       int nparts, float weight, float* __restrict__ dx, int64_t ld_dx) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + threadIdx.x / kWave;
+    if (r >= rows) return;
+    // the pairs of all workers of this row, one worker per lane (and round)
+    float p1 = 0.f, p2 = 0.f;
+    for (int p = lane; p < nparts; p += kWave) {
+        const float2 s = reinterpret_cast<const float2*>(part_sums)[static_cast<int64_t>(p) * rows + r];
+        p1 += s.x;
+        p2 += s.y;
+    }
+    const float m = mean[r], rs = rstd[r];
+    const float S1 = wave_sum(p1) * weight, S2 = wave_sum(p2) * weight;   // already times a_p
+    const float* dyr = dy + r * ld_dy;
+    const float* xr = x + r * ld_x;
+    float* dxr = dx + r * ld_dx;
+    if (VEC) {
+        for (int64_t c = lane * 4; c < cols; c += kWave * 4) {
+            const float4 d = *reinterpret_cast<const float4*>(dyr + c);
+            const float4 v = *reinterpret_cast<const float4*>(xr + c);
+            float4 g = make_float4(1.f, 1.f, 1.f, 1.f);
+            if (gamma) g = *reinterpret_cast<const float4*>(gamma + c);
+            float4 o;
+            o.x = rs * (d.x * g.x - (S1 + ((v.x - m) * rs) * S2));
+            o.y = rs * (d.y * g.y - (S1 + ((v.y - m) * rs) * S2));
+            o.z = rs * (d.z * g.z - (S1 + ((v.z - m) * rs) * S2));
+            o.w = rs * (d.w * g.w - (S1 + ((v.w - m) * rs) * S2));
+            *reinterpret_cast<float4*>(dxr + c) = o;
+        }
+    } else {
+        for (int64_t c = lane; c < cols; c += kWave) {
+            const float g = dyr[c] * (gamma ? gamma[c] : 1.f);
+            dxr[c] = rs * (g - (S1 + ((xr[c] - m) * rs) * S2));
+        }
+    }
+}
+
+// Workgroup (strip, split): rows [split * rows_per_split, ...) of a 64-column
+// strip; lane group t / 64 takes every fourth row, thread t % 64 one column.
+// partial[split, 0, c] = sum dy xhat, partial[split, 1, c] = sum dy.
+__global__ __launch_bounds__(kBlock) void ln_bwd_params_partial(const float* __restrict__ dy, const float* __restrict__ x,
+                                                                int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                                                const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                                int64_t rows_per_split, float* __restrict__ partial, int strips) {
+    __shared__ float fold[2][kWavesPerBlock][kStrip];
+    const int split = blockIdx.x / strips, strip = blockIdx.x - split * strips;
+    const int g = threadIdx.x / kStrip, t = threadIdx.x % kStrip;
+    const int64_t c = static_cast<int64_t>(strip) * kStrip + t;
+    const int64_t r_begin = split * rows_per_split;
+    const int64_t r_end = r_begin + rows_per_split < rows ? r_begin + rows_per_split : rows;
+    float a = 0.f, b = 0.f;
+    if (c < cols) {
+        for (int64_t r = r_begin + g; r < r_end; r += kWavesPerBlock) {
+            const float d = dy[r * ld_dy + c];
+            a += d * ((x[r * ld_x + c] - mean[r]) * rstd[r]);
+            b += d;
+        }
+    }
+    fold[0][g][t] = a;
+    fold[1][g][t] = b;
+    __syncthreads();
+    if (threadIdx.x < 2 * kStrip) {
+        const int which = threadIdx.x / kStrip;
+        float s = 0.f;
+#pragma unroll
+        for (int k = 0; k < kWavesPerBlock; ++k) s += fold[which][k][t];
+        if (c < cols) partial[(static_cast<int64_t>(split) * 2 + which) * cols + c] = s;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void ln_bwd_params_final(const float* __restrict__ partial, int64_t cols, int splits,
+                                                              float* __restrict__ dgamma, float* __restrict__ dbeta) {
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (c >= cols) return;
+    float a = 0.f, b = 0.f;
+    for (int k = 0; k < splits; ++k) {
+        a += partial[(static_cast<int64_t>(k) * 2) * cols + c];
+        b += partial[(static_cast<int64_t>(k) * 2 + 1) * cols + c];
+    }
+    if (dgamma) dgamma[c] = a;
+    if (dbeta) dbeta[c] = b;
+}
+
+bool vectorizable(int64_t cols, std::initializer_list<int64_t> lds, std::initializer_list<const void*> ptrs) {
+    if (cols % 4 != 0) return false;
+    for (int64_t ld : lds)
+        if (ld % 4 != 0) return false;
+    for (const void* p : ptrs)
+        if (p && !aligned_to(p, 16)) return false;
+    return true;
+}
+
+int check_rows(const char* what, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x) {
+    if (rows < 0 || cols < 1 || ld_dy < cols || ld_x < cols)
+        return fail(DDL_E_ARG, "%s: rows=%lld cols=%lld ld_dy=%lld ld_x=%lld", what, (long long)rows, (long long)cols,
+                    (long long)ld_dy, (long long)ld_x);
+    if (rows > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "%s: more than 2^31 rows", what);
+    return 0;
+}
+
+}  // namespace
+}  // namespace ddl
+
+extern "C" int ddl_ln_bwd_partial_f32(const float* dy, const float* x, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                      const float* mean, const float* rstd, const float* gamma, float* sums, void* stream) {
+    using namespace ddl;
+    if (int rc = check_rows("ln backward sums", rows, cols, ld_dy, ld_x)) return rc;
+    if (rows == 0) return 0;
+    if (!dy || !x || !mean || !rstd || !sums) return fail(DDL_E_ARG, "ln backward sums: null pointer");
+    if (!aligned_to(dy, 4) || !aligned_to(x, 4) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) || !aligned_to(gamma, 4) || !aligned_to(sums, 8))
+        return fail(DDL_E_ALIGN, "ln backward sums: pointers must be 4-byte aligned, the sums 8-byte");
+    const uint32_t blocks = static_cast<uint32_t>((rows + kWavesPerBlock - 1) / kWavesPerBlock);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (vectorizable(cols, {ld_dy, ld_x}, {dy, x, gamma}))
+        hipLaunchKernelGGL(ln_bwd_partial<true>, dim3(blocks), dim3(kBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, sums);
+    else
+        hipLaunchKernelGGL(ln_bwd_partial<false>, dim3(blocks), dim3(kBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, sums);
+    return check_launch("ln_bwd_partial");
+}
+
+extern "C" int ddl_ln_bwd_input_f32(const float* dy, const float* x, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                    const float* mean, const float* rstd, const float* gamma, const float* part_sums,
+                                    int nparts, float weight, float* dx, int64_t ld_dx, void* stream) {
+    using namespace ddl;
+    if (int rc = check_rows("ln backward input", rows, cols, ld_dy, ld_x)) return rc;
+    if (ld_dx < cols || nparts < 1) return fail(DDL_E_ARG, "ln backward input: ld_dx=%lld nparts=%d", (long long)ld_dx, nparts);
+    if (rows == 0) return 0;
+    if (!dy || !x || !mean || !rstd || !part_sums || !dx) return fail(DDL_E_ARG, "ln backward input: null pointer");
+    if (!aligned_to(dy, 4) || !aligned_to(x, 4) || !aligned_to(dx, 4) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) ||
+        !aligned_to(gamma, 4) || !aligned_to(part_sums, 8))
+        return fail(DDL_E_ALIGN, "ln backward input: pointers must be 4-byte aligned, the sums 8-byte");
+    const uint32_t blocks = static_cast<uint32_t>((rows + kWavesPerBlock - 1) / kWavesPerBlock);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (vectorizable(cols, {ld_dy, ld_x, ld_dx}, {dy, x, gamma, dx}))
+        hipLaunchKernelGGL(ln_bwd_input<true>, dim3(blocks), dim3(kBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma,
+                           part_sums, nparts, weight, dx, ld_dx);
+    else
+        hipLaunchKernelGGL(ln_bwd_input<false>, dim3(blocks), dim3(kBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma,
+                           part_sums, nparts, weight, dx, ld_dx);
+    return check_launch("ln_bwd_input");
+}
+
+extern "C" int ddl_ln_bwd_params_f32(const float* dy, const float* x, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                     const float* mean, const float* rstd, float* dgamma, float* dbeta, float* workspace,
+                                     int64_t workspace_elems, void* stream) {
+    using namespace ddl;
+    if (int rc = check_rows("ln backward parameters", rows, cols, ld_dy, ld_x)) return rc;
+    if (!dgamma && !dbeta) return 0;
+    if (!workspace || (rows > 0 && (!dy || !x || !mean || !rstd))) return fail(DDL_E_ARG, "ln backward parameters: null pointer");
+    if (!aligned_to(dy, 4) || !aligned_to(x, 4) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) || !aligned_to(dgamma, 4) ||
+        !aligned_to(dbeta, 4) || !aligned_to(workspace, 4))
+        return fail(DDL_E_ALIGN, "ln backward parameters: pointers must be 4-byte aligned");
+    int64_t splits = workspace_elems / (2 * cols);
+    if (splits < 1) return fail(DDL_E_ARG, "ln backward parameters: workspace of %lld floats is smaller than 2 x %lld", (long long)workspace_elems, (long long)cols);
+    if (splits > 256) splits = 256;
+    const int64_t by_rows = (rows + 31) / 32;
+    if (splits > by_rows) splits = by_rows > 0 ? by_rows : 1;
+    const int64_t rows_per_split = rows > 0 ? (rows + splits - 1) / splits : 1;
+    const int64_t strips = (cols + kStrip - 1) / kStrip;
+    if (strips * splits > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "ln backward parameters: too many workgroups");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(ln_bwd_params_partial, dim3(static_cast<uint32_t>(strips * splits)), dim3(kBlock), 0, s, dy, x, rows, cols,
+                       ld_dy, ld_x, mean, rstd, rows_per_split, workspace, static_cast<int>(strips));
+    if (int rc = check_launch("ln_bwd_params_partial")) return rc;
+    hipLaunchKernelGGL(ln_bwd_params_final, dim3(static_cast<uint32_t>((cols + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, workspace,
+                       cols, static_cast<int>(splits), dgamma, dbeta);
+    return check_launch("ln_bwd_params_final");
+}

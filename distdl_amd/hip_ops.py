@@ -270,6 +270,55 @@ def ln_normalize_affine(x2d, part_stats, part_cols, gamma, beta, eps, want_stats
     return (y, mean, rstd) if want_stats else y
 
 
+def _rows2d(t, name):
+    if t.dtype != torch.float32 or t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise ValueError(f"{name}: need a 2-D fp32 tensor with unit column stride")
+    return t.stride(0) if t.shape[0] > 1 else t.shape[1]
+
+
+def ln_backward_partial(dy2d, x2d, mean, rstd, gamma):
+    """Local {sum g, sum g xhat} per row, g = dy gamma: a [rows, 2] fp32 tensor."""
+    _require_gpu(dy2d, x2d, mean, rstd, gamma)
+    ld_dy, ld_x = _rows2d(dy2d, "ln_backward_partial"), _rows2d(x2d, "ln_backward_partial")
+    rows, cols = x2d.shape
+    sums = torch.empty((rows, 2), dtype=torch.float32, device=x2d.device)
+    rc = _lib.load().ddl_ln_bwd_partial_f32(dy2d.data_ptr(), x2d.data_ptr(), rows, cols, ld_dy, ld_x, mean.data_ptr(),
+                                            rstd.data_ptr(), _ptr(gamma), sums.data_ptr(), _stream())
+    _lib.check(rc, "ddl_ln_bwd_partial_f32")
+    return sums
+
+
+def ln_backward_input(dy2d, x2d, mean, rstd, gamma, part_sums, weight):
+    """dx from the gathered [P, rows, 2] sums; ``weight`` = 1 / (P * local columns)."""
+    _require_gpu(dy2d, x2d, mean, rstd, gamma, part_sums)
+    ld_dy, ld_x = _rows2d(dy2d, "ln_backward_input"), _rows2d(x2d, "ln_backward_input")
+    rows, cols = x2d.shape
+    if part_sums.dtype != torch.float32 or part_sums.dim() != 3 or tuple(part_sums.shape[1:]) != (rows, 2) or \
+       not part_sums.is_contiguous():
+        raise ValueError(f"ln_backward_input: part_sums must be contiguous fp32 [P, {rows}, 2]")
+    dx = torch.empty((rows, cols), dtype=torch.float32, device=x2d.device)
+    rc = _lib.load().ddl_ln_bwd_input_f32(dy2d.data_ptr(), x2d.data_ptr(), rows, cols, ld_dy, ld_x, mean.data_ptr(),
+                                          rstd.data_ptr(), _ptr(gamma), part_sums.data_ptr(), part_sums.shape[0],
+                                          float(weight), dx.data_ptr(), cols, _stream())
+    _lib.check(rc, "ddl_ln_bwd_input_f32")
+    return dx
+
+
+def ln_backward_params(dy2d, x2d, mean, rstd, want_gamma=True, want_beta=True):
+    """(dgamma, dbeta) = column sums over the local rows of (dy xhat, dy)."""
+    _require_gpu(dy2d, x2d, mean, rstd)
+    ld_dy, ld_x = _rows2d(dy2d, "ln_backward_params"), _rows2d(x2d, "ln_backward_params")
+    rows, cols = x2d.shape
+    dg = torch.empty(cols, dtype=torch.float32, device=x2d.device) if want_gamma else None
+    db = torch.empty(cols, dtype=torch.float32, device=x2d.device) if want_beta else None
+    splits = max(1, min(256, (rows + 31) // 32))
+    work = torch.empty(2 * splits * cols, dtype=torch.float32, device=x2d.device)
+    rc = _lib.load().ddl_ln_bwd_params_f32(dy2d.data_ptr(), x2d.data_ptr(), rows, cols, ld_dy, ld_x, mean.data_ptr(),
+                                           rstd.data_ptr(), _ptr(dg), _ptr(db), work.data_ptr(), work.numel(), _stream())
+    _lib.check(rc, "ddl_ln_bwd_params_f32")
+    return dg, db
+
+
 def embedding_gather(weight, ids, lo, hi, out=None):
     """out[t] = weight[ids[t] - lo] if lo <= ids[t] < hi else 0."""
     _require_gpu(weight, ids)

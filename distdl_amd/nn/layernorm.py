@@ -25,8 +25,13 @@ from .module import Module
 STATS_TAG = "layernorm_stats"
 
 
+BWD_SUMS_TAG = "layernorm_backward_sums"
+
+
 class _LayerNormShard(torch.autograd.Function):
-    """Local shard of a layer norm whose statistics span ``P_reduce``."""
+    """Local shard of a layer norm whose statistics span ``P_reduce``, and its
+    adjoint: the gradient autograd derives from the reference's forward
+    (nn/layernorm.py:230-247, 295-309), whose all-reduces are self-adjoint."""
 
     @staticmethod
     def forward(ctx, input, weight, bias, P_reduce, part_cols, eps):
@@ -43,12 +48,35 @@ class _LayerNormShard(torch.autograd.Function):
             gathered = stats.unsqueeze(0)
         gamma = None if weight is None else weight.detach().reshape(-1)
         beta = None if bias is None else bias.detach().reshape(-1)
-        y = hip_ops.ln_normalize_affine(x2d, gathered, part_cols, gamma, beta, eps)
+        y, mean, rstd = hip_ops.ln_normalize_affine(x2d, gathered, part_cols, gamma, beta, eps, want_stats=True)
+        ctx.save_for_backward(x2d, mean, rstd, gamma)
+        ctx.P_reduce, ctx.nparts, ctx.cols = P_reduce, len(part_cols), cols
+        ctx.param_shapes = (None if weight is None else weight.shape, None if bias is None else bias.shape)
         return y.view(input.shape)
 
     @staticmethod
     def backward(ctx, grad_output):
-        raise NotImplementedError("the backward pass of DistributedLayerNorm is not part of this build")
+        x2d, mean, rstd, gamma = ctx.saved_tensors
+        need_x, need_w, need_b = ctx.needs_input_grad[:3]
+        dy2d = grad_output.detach().reshape(-1, ctx.cols)
+        if dy2d.shape[1] > 1 and dy2d.stride(1) != 1:
+            dy2d = dy2d.contiguous()
+        dx = dw = db = None
+        if need_x:
+            sums = hip_ops.ln_backward_partial(dy2d, x2d, mean, rstd, gamma)
+            if ctx.nparts > 1:
+                gathered = ctx.P_reduce._world.transport.allgather(ctx.P_reduce, sums, tag=BWD_SUMS_TAG).contiguous()
+            else:
+                gathered = sums.unsqueeze(0)
+            dx = hip_ops.ln_backward_input(dy2d, x2d, mean, rstd, gamma, gathered, 1.0 / (ctx.nparts * ctx.cols))
+            dx = dx.view(grad_output.shape)
+        w_shape, b_shape = ctx.param_shapes
+        want_w, want_b = need_w and w_shape is not None, need_b and b_shape is not None
+        if want_w or want_b:
+            dw, db = hip_ops.ln_backward_params(dy2d, x2d, mean, rstd, want_w, want_b)
+            dw = None if dw is None else dw.view(w_shape)
+            db = None if db is None else db.view(b_shape)
+        return dx, dw, db, None, None, None
 
 
 class DistributedLayerNorm(Module):

@@ -182,6 +182,38 @@ int ddl_ln_normalize_affine_f32(const float* x, int64_t rows, int64_t cols,
                                 float* mean_out, float* rstd_out,
                                 void* stream);
 
+/* Backward of the LayerNorm shard: what autograd derives from the reference's
+ * forward (nn/layernorm.py:230-247, 295-309, all-reduces included).  With
+ * g = dy * gamma (gamma NULL = 1), xhat = (x - mean) * rstd (mean, rstd as
+ * ddl_ln_normalize_affine_f32 returned them) and a = 1 / (P * columns of this
+ * worker), P = workers sharing a row:
+ *
+ *   ddl_ln_bwd_partial_f32   sums[r] = { sum_c g[r,c], sum_c g[r,c] xhat[r,c] }
+ *                            over the LOCAL columns; the caller gathers the
+ *                            pairs of the P workers into part_sums[P, rows, 2]
+ *   ddl_ln_bwd_input_f32     dx[r,c] = rstd[r] * ( g[r,c] - weight * (S1[r] +
+ *                            xhat[r,c] * S2[r]) ), S = sum over the P pairs,
+ *                            weight = a
+ *   ddl_ln_bwd_params_f32    dgamma[c] = sum_r dy[r,c] xhat[r,c],
+ *                            dbeta[c]  = sum_r dy[r,c]   (either may be NULL);
+ *                            `workspace`: device memory for at least 2 * cols
+ *                            floats (up to 512 * cols are used), contents on
+ *                            entry do not matter. */
+int ddl_ln_bwd_partial_f32(const float* dy, const float* x, int64_t rows,
+                           int64_t cols, int64_t ld_dy, int64_t ld_x,
+                           const float* mean, const float* rstd,
+                           const float* gamma, float* sums, void* stream);
+int ddl_ln_bwd_input_f32(const float* dy, const float* x, int64_t rows,
+                         int64_t cols, int64_t ld_dy, int64_t ld_x,
+                         const float* mean, const float* rstd,
+                         const float* gamma, const float* part_sums, int nparts,
+                         float weight, float* dx, int64_t ld_dx, void* stream);
+int ddl_ln_bwd_params_f32(const float* dy, const float* x, int64_t rows,
+                          int64_t cols, int64_t ld_dy, int64_t ld_x,
+                          const float* mean, const float* rstd, float* dgamma,
+                          float* dbeta, float* workspace,
+                          int64_t workspace_elems, void* stream);
+
 /* ------------------------------------------------------------------------ *
  * DistributedEmbedding shard gather
  * ------------------------------------------------------------------------ */

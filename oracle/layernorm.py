@@ -50,3 +50,44 @@ def partial_stats(shard, num_norm_dims=1, dtype=np.float64):
     m2 = ((x - m) ** 2).sum(axis=axes, keepdims=True)
     rows = int(np.prod(x.shape[:x.ndim - num_norm_dims]))
     return np.stack([m.reshape(rows), m2.reshape(rows)], axis=1)
+
+
+def backward_shards(shards, gammas, dys, eps, num_norm_dims=1, dtype=np.float64):
+    """Gradients of ``forward_shards`` with respect to the shards and the
+    affine parameters: returns ``(dxs, dgammas, dbetas)``, lists over the
+    reduction group.
+
+    Every element of shard p enters the reference's mean and variance with
+    weight a_p = 1 / (P n_p), and the all-reduce is its own adjoint, so with
+    g = dy * gamma, xhat = (x - mean) * rstd, S1 = sum of g and S2 = sum of
+    g * xhat over the WHOLE row (all shards):
+
+        dx_p     = rstd * (g_p - a_p * (S1 + xhat_p * S2))
+        dgamma_p = sum over rows of dy_p * xhat_p        dbeta_p = sum over rows of dy_p
+
+    Pinned in tests/test_oracle_golden.py by torch autograd run through a
+    literal torch restatement of nn/layernorm.py:230-309 (equal and unequal
+    shard widths), and by torch.nn.functional.layer_norm for equal widths."""
+    P = len(shards)
+    xs = [np.asarray(s, dtype=dtype) for s in shards]
+    ds = [np.asarray(d, dtype=dtype) for d in dys]
+    lead = xs[0].shape[:xs[0].ndim - num_norm_dims]
+    flat = [x.reshape(int(np.prod(lead)), -1) for x in xs]
+    dflat = [d.reshape(int(np.prod(lead)), -1) for d in ds]
+    ns = [f.shape[1] for f in flat]
+    mean = sum(f.mean(axis=1) for f in flat) / P
+    var = sum(((f - mean[:, None]) ** 2).mean(axis=1) for f in flat) / P
+    rstd = 1.0 / np.sqrt(var + eps)
+    gam = [np.ones(n, dtype=dtype) if g is None else np.asarray(g, dtype=dtype).reshape(-1) for g, n in zip(gammas, ns)]
+    xhat = [(f - mean[:, None]) * rstd[:, None] for f in flat]
+    g = [d * w[None, :] for d, w in zip(dflat, gam)]
+    S1 = sum(v.sum(axis=1) for v in g)
+    S2 = sum((v * h).sum(axis=1) for v, h in zip(g, xhat))
+    dxs, dgs, dbs = [], [], []
+    for p in range(P):
+        a = 1.0 / (P * ns[p])
+        dx = rstd[:, None] * (g[p] - a * (S1[:, None] + xhat[p] * S2[:, None]))
+        dxs.append(dx.reshape(xs[p].shape))
+        dgs.append((dflat[p] * xhat[p]).sum(axis=0))
+        dbs.append(dflat[p].sum(axis=0))
+    return dxs, dgs, dbs

@@ -154,6 +154,100 @@ def test_layernorm_layer_matches_torch(golden):
                 assert np.allclose(got, part, rtol=1e-4, atol=1e-5), geom     # reference tolerance is atol sqrt(1e-7)
 
 
+@pytest.mark.parametrize("cols", [[256, 256, 256, 256], [64, 64], [300, 212], [7, 9], [2048], [5000, 40], [4] * 70])
+@pytest.mark.parametrize("affine", [True, False])
+def test_layernorm_backward_kernels_match_oracle(ops, cols, affine):
+    """dx, dgamma, dbeta of one worker of the reduction group; the row sums of
+    the other workers come from the oracle.  fp32 kernels against the fp64
+    closed form: 1e-5 relative to the gradient's scale."""
+    rng = np.random.default_rng(sum(cols) + len(cols))
+    rows, eps = 37, 1e-5
+    shards = [(rng.standard_normal((rows, c)) * 2 + 0.5).astype(np.float32) for c in cols]
+    dys = [rng.standard_normal((rows, c)).astype(np.float32) for c in cols]
+    gammas = [(1 + 0.1 * rng.standard_normal(c)).astype(np.float32) if affine else None for c in cols]
+    betas = [(0.1 * rng.standard_normal(c)).astype(np.float32) if affine else None for c in cols]
+    want_dx, want_dg, want_db = o_ln.backward_shards(shards, gammas, dys, eps)
+    P = len(cols)
+    for live in {0, P - 1}:
+        x2d = torch.from_numpy(shards[live]).cuda()
+        dy2d = torch.from_numpy(dys[live]).cuda()
+        g = None if not affine else torch.from_numpy(gammas[live]).cuda()
+        b = None if not affine else torch.from_numpy(betas[live]).cuda()
+        parts = [torch.from_numpy(o_ln.partial_stats(s).astype(np.float32)).cuda() for s in shards]
+        parts[live] = ops.ln_partial_stats(x2d)
+        _, mean, rstd = ops.ln_normalize_affine(x2d, torch.stack(parts).contiguous(), cols, g, b, eps, want_stats=True)
+        sums = ops.ln_backward_partial(dy2d, x2d, mean, rstd, g)
+        # the other workers' sums, from the oracle's intermediate quantities (fp64 -> fp32)
+        m64 = sum(s.astype(np.float64).mean(axis=1) for s in shards) / P
+        v64 = sum(((s.astype(np.float64) - m64[:, None]) ** 2).mean(axis=1) for s in shards) / P
+        r64 = 1.0 / np.sqrt(v64 + eps)
+        gathered = []
+        for p in range(P):
+            gp = dys[p].astype(np.float64) * (gammas[p].astype(np.float64) if affine else 1.0)
+            xh = (shards[p].astype(np.float64) - m64[:, None]) * r64[:, None]
+            pair = np.stack([gp.sum(axis=1), (gp * xh).sum(axis=1)], axis=1)
+            if p == live:
+                scale = np.abs(gp).sum(axis=1).max()
+                assert np.allclose(sums.cpu().numpy(), pair, rtol=1e-4, atol=2e-5 * scale)
+                gathered.append(sums)
+            else:
+                gathered.append(torch.from_numpy(pair.astype(np.float32)).cuda())
+        dx = ops.ln_backward_input(dy2d, x2d, mean, rstd, g, torch.stack(gathered).contiguous(), 1.0 / (P * cols[live]))
+        dg, db = ops.ln_backward_params(dy2d, x2d, mean, rstd)
+        torch.cuda.synchronize()
+        tol = 1e-5 * max(1.0, np.abs(want_dx[live]).max())
+        assert np.abs(dx.cpu().numpy() - want_dx[live]).max() <= 4 * tol
+        assert np.allclose(dg.cpu().numpy(), want_dg[live], rtol=1e-4, atol=1e-4)
+        assert np.allclose(db.cpu().numpy(), want_db[live], rtol=1e-4, atol=1e-4)
+
+
+def test_layernorm_layer_backward_matches_torch():
+    """DistributedLayerNorm on every worker (loopback), forward and backward,
+    against torch.nn.functional.layer_norm on the whole tensor."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedLayerNorm
+    torch.manual_seed(5)
+    P, shape, norm = [1, 2, 2], [3, 8, 64], [64]
+    x = torch.randn(shape)
+    dy = torch.randn(shape)
+    gamma = 1 + 0.1 * torch.randn(norm)
+    beta = 0.1 * torch.randn(norm)
+    xs, dys = o_rep.scatter(x.numpy(), P), o_rep.scatter(dy.numpy(), P)
+    gs = o_rep.scatter(gamma.numpy().reshape(1, 1, 64), [1, 1, 2])
+    bs = o_rep.scatter(beta.numpy().reshape(1, 1, 64), [1, 1, 2])
+
+    def body(P_world):
+        P_x = P_world.create_partition_inclusive(list(range(4))).create_cartesian_topology_partition(P)
+        layer = DistributedLayerNorm(P_x, norm)
+        red = int(P_x.index[-1])
+        with torch.no_grad():
+            if layer.P_w.active:
+                layer.weight.copy_(torch.from_numpy(gs[red]))
+                layer.bias.copy_(torch.from_numpy(bs[red]))
+        xin = torch.from_numpy(xs[P_x.rank]).cuda().requires_grad_(True)
+        y = layer(xin)
+        y.backward(torch.from_numpy(dys[P_x.rank]).cuda())
+        torch.cuda.synchronize()
+        wgrad = layer.weight.grad.cpu().numpy() if layer.P_w.active and layer.weight.grad is not None else None
+        bgrad = layer.bias.grad.cpu().numpy() if layer.P_w.active and layer.bias.grad is not None else None
+        return xin.grad.cpu().numpy(), wgrad, bgrad, tuple(int(i) for i in P_x.index)
+
+    outs = SimWorld(4).run(body)
+    xr, gr, br = x.clone().requires_grad_(True), gamma.clone().requires_grad_(True), beta.clone().requires_grad_(True)
+    F.layer_norm(xr, tuple(norm), gr, br, 1e-5).backward(dy)
+    want_dx = o_rep.scatter(xr.grad.numpy(), P)
+    for rank, (dx, wgrad, bgrad, index) in enumerate(outs):
+        assert np.allclose(dx, want_dx[rank], rtol=1e-4, atol=1e-5)
+    # parameter gradients: summed over the workers that share a feature shard
+    for red in range(2):
+        lo, hi = 32 * red, 32 * (red + 1)
+        got_w = [o[1] for o in outs if o[1] is not None and o[3][-1] == red]
+        got_b = [o[2] for o in outs if o[2] is not None and o[3][-1] == red]
+        assert got_w and got_b
+        assert np.allclose(sum(g.reshape(-1) for g in got_w), gr.grad.numpy()[lo:hi], rtol=1e-4, atol=1e-4)
+        assert np.allclose(sum(g.reshape(-1) for g in got_b), br.grad.numpy()[lo:hi], rtol=1e-4, atol=1e-4)
+
+
 # ---------------------------------------------------------------- Embedding --
 
 def test_embedding_config3_rank0_bit_exact(ops):

@@ -366,3 +366,35 @@ def test_linear_backward_oracle_matches_torch_autograd():
     assert np.allclose(db, bd.grad.numpy(), rtol=1e-12, atol=1e-12)
     # a transposed operand or a swapped product would break these shapes / values
     assert dx.shape == (11, 24) and dw.shape == (7, 24) and db.shape == (7,)
+
+
+@pytest.mark.parametrize("widths", [[8, 8], [5, 11, 3], [16]])
+def test_layernorm_backward_oracle_matches_autograd_of_the_reference_sequence(widths):
+    """The reference's forward, restated op by op in torch (nn/layernorm.py:230-247,
+    295-309; an all-reduce is a sum over the shards), differentiated by autograd,
+    against the closed form of oracle.backward_shards -- for unequal widths too,
+    where the result is NOT the gradient of a plain layer norm."""
+    torch.manual_seed(sum(widths))
+    rows, P, eps = 6, len(widths), 1e-5
+    xs = [torch.randn(rows, w, dtype=torch.float64, requires_grad=True) for w in widths]
+    gs = [(1 + 0.1 * torch.randn(w, dtype=torch.float64)).requires_grad_(True) for w in widths]
+    bs = [(0.1 * torch.randn(w, dtype=torch.float64)).requires_grad_(True) for w in widths]
+    dys = [torch.randn(rows, w, dtype=torch.float64) for w in widths]
+    mean = sum(x.mean(dim=-1, keepdim=True) for x in xs) / P                      # :230-233
+    var = sum(((x - mean) ** 2).mean(dim=-1, keepdim=True) for x in xs) / P       # :246-247
+    ys = [g * ((x - mean) / torch.sqrt(var + eps)) + b for x, g, b in zip(xs, gs, bs)]   # :302, :309
+    sum((y * d).sum() for y, d in zip(ys, dys)).backward()
+    dxs, dgs, dbs = o_ln.backward_shards([x.detach().numpy() for x in xs], [g.detach().numpy() for g in gs],
+                                         [d.numpy() for d in dys], eps)
+    for p in range(P):
+        assert np.allclose(dxs[p], xs[p].grad.numpy(), rtol=1e-10, atol=1e-12)
+        assert np.allclose(dgs[p], gs[p].grad.numpy(), rtol=1e-10, atol=1e-12)
+        assert np.allclose(dbs[p], bs[p].grad.numpy(), rtol=1e-10, atol=1e-12)
+    if len(set(widths)) == 1:
+        # equal widths: the gradient of torch's layer norm on the concatenated row
+        x = torch.cat([t.detach() for t in xs], dim=1).requires_grad_(True)
+        g = torch.cat([t.detach() for t in gs]).requires_grad_(True)
+        b = torch.cat([t.detach() for t in bs]).requires_grad_(True)
+        (F.layer_norm(x, (sum(widths),), g, b, eps) * torch.cat(dys, dim=1)).sum().backward()
+        assert np.allclose(np.concatenate(dxs, axis=1), x.grad.numpy(), rtol=1e-9, atol=1e-11)
+        assert np.allclose(np.concatenate(dgs), g.grad.numpy(), rtol=1e-9, atol=1e-11)
