@@ -69,6 +69,8 @@ SIGNATURES = {
                                       c_void_p, c_void_p, c_int64, c_void_p]),
     "ddl_embedding_gather": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_int, c_int64, c_int64, c_int64,
                                      c_void_p, c_void_p]),
+    "ddl_embedding_backward": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64,
+                                       c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "ddl_linear_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                 c_int64, c_void_p]),
     "ddl_transpose_2d": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),

@@ -342,6 +342,32 @@ def embedding_gather(weight, ids, lo, hi, out=None):
     return out
 
 
+def embedding_backward(grad_output, ids, lo, hi, padding_idx=None):
+    """Gradient of :func:`embedding_gather` with respect to the ``[hi-lo, dim]`` table."""
+    _require_gpu(grad_output, ids)
+    if grad_output.dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError("embedding_backward: bfloat16 or float32 gradients only")
+    if ids.dtype not in (torch.int64, torch.int32):
+        raise ValueError("embedding_backward: ids must be int32 or int64")
+    dim = grad_output.shape[-1]
+    if tuple(grad_output.shape[:-1]) != tuple(ids.shape):
+        raise ValueError("embedding_backward: gradient and ids disagree in shape")
+    dy = grad_output.reshape(-1, dim)
+    if dim > 1 and dy.stride(1) != 1:
+        dy = dy.contiguous()
+    ids_c = ids.contiguous()
+    rows, n_ids = int(hi) - int(lo), ids_c.numel()
+    dw = torch.empty((rows, dim), dtype=grad_output.dtype, device=grad_output.device)
+    work = torch.empty(2 * rows + 1 + n_ids, dtype=torch.int32, device=grad_output.device)
+    dt = _lib.DDL_DT_BF16 if grad_output.dtype == torch.bfloat16 else _lib.DDL_DT_F32
+    rc = _lib.load().ddl_embedding_backward(dy.data_ptr(), dt, dim, dy.stride(0) if n_ids > 1 else dim, ids_c.data_ptr(),
+                                            1 if ids.dtype == torch.int64 else 0, n_ids, int(lo), int(hi),
+                                            -1 if padding_idx is None else int(padding_idx), dw.data_ptr(), dim,
+                                            work.data_ptr(), work.numel(), _stream())
+    _lib.check(rc, "ddl_embedding_backward")
+    return dw
+
+
 def linear_bf16(x, weight, bias=None, out=None):
     """y = x @ weight.T + bias; bf16 operands, fp32 accumulation, bf16 result."""
     _require_gpu(x, weight, bias)

@@ -18,14 +18,22 @@ from .module import Module
 
 
 class _EmbeddingShard(torch.autograd.Function):
+    """Row gather from the local table and its adjoint (the dense gradient
+    autograd derives for ``F.embedding``: rows of ``grad_output`` summed per
+    looked-up table row, the ``padding_idx`` row left at zero)."""
 
     @staticmethod
-    def forward(ctx, weight, ids, lo, hi):
+    def forward(ctx, weight, ids, lo, hi, padding_idx=None):
+        ctx.save_for_backward(ids)
+        ctx.window = (lo, hi, padding_idx)
         return hip_ops.embedding_gather(weight.detach(), ids, lo, hi)
 
     @staticmethod
     def backward(ctx, grad_output):
-        raise NotImplementedError("the backward pass of DistributedEmbedding is not part of this build")
+        (ids,) = ctx.saved_tensors
+        lo, hi, padding_idx = ctx.window
+        dw = hip_ops.embedding_backward(grad_output.detach(), ids, lo, hi, padding_idx)
+        return dw, None, None, None, None
 
 
 class DistributedEmbedding(Module):
@@ -128,4 +136,4 @@ class DistributedEmbedding(Module):
         else:
             weight = self.weight_buffer
             self.weight_buffer = None
-        return _EmbeddingShard.apply(weight, input, self.vocab_lo, self.vocab_hi)
+        return _EmbeddingShard.apply(weight, input, self.vocab_lo, self.vocab_hi, self.padding_idx)

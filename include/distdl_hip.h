@@ -231,6 +231,21 @@ int ddl_embedding_gather(const void* weight, int64_t dim, int64_t ldw,
                          int64_t n_ids, int64_t lo, int64_t hi,
                          void* out, void* stream);
 
+/* Adjoint of ddl_embedding_gather with respect to the table:
+ *   dweight[r, :] = sum over t with ids[t] - lo == r and ids[t] != padding_idx
+ *                   of dy[t, :]                        for every r in [0, hi-lo)
+ * (what autograd derives for torch.nn.functional.embedding,
+ * nn/embedding.py:244-246; padding_idx < 0 = none).  dtype = DDL_DT_BF16 or
+ * DDL_DT_F32 for dy and dweight alike; sums are accumulated in fp32 in
+ * ascending token order.  Every element of dweight is written, so it needs no
+ * clearing.  `workspace`: device memory for at least 2 (hi-lo) + 1 + n_ids
+ * int32, contents on entry do not matter. */
+int ddl_embedding_backward(const void* dy, int dtype, int64_t dim, int64_t ld_dy,
+                           const void* ids, int ids_is_i64, int64_t n_ids,
+                           int64_t lo, int64_t hi, int64_t padding_idx,
+                           void* dweight, int64_t ld_dw, int32_t* workspace,
+                           int64_t workspace_elems, void* stream);
+
 /* ------------------------------------------------------------------------ *
  * DistributedLinear shard GEMM (bf16 in, fp32 accumulate, bf16 out)
  * ------------------------------------------------------------------------ */

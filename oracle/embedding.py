@@ -23,3 +23,19 @@ def gather(table, ids, lo=0, hi=None):
     out = table[safe.reshape(-1)].reshape(ids.shape + (table.shape[1],)).copy()
     out[~hit] = 0
     return out
+
+
+def backward(dy, ids, lo, hi, padding_idx=None, dtype=np.float64):
+    """Adjoint of ``gather`` with respect to the table: row r of the result is
+    the sum of dy[t] over the tokens with ids[t] - lo == r (tokens outside the
+    window and tokens equal to padding_idx add nothing) -- the dense gradient
+    of torch.nn.functional.embedding (reference call site nn/embedding.py:244-246).
+    ``dy`` holds values (not bit patterns); sums are exact in ``dtype``.
+    Pinned by torch autograd on CPU in tests/test_oracle_golden.py."""
+    ids = np.asarray(ids).reshape(-1)
+    dy = np.asarray(dy, dtype=dtype).reshape(ids.size, -1)
+    out = np.zeros((hi - lo, dy.shape[1]), dtype=dtype)
+    for t, i in enumerate(ids):
+        if lo <= i < hi and (padding_idx is None or i != padding_idx):
+            out[i - lo] += dy[t]
+    return out

@@ -310,6 +310,73 @@ def test_embedding_layer_full_window_matches_torch():
     assert torch.equal(torch.cat(outs, dim=-1), want)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dim,rows,tokens", [(1, 1, 1), (8, 10, 50), (100, 37, 300), (512, 64, 1000), (1000, 5, 4000),
+                                              (4100, 20, 100)])
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+def test_embedding_backward_small_cases(ops, dtype, dim, rows, tokens, idt):
+    """Window [lo, hi) of a larger vocabulary, a padding row, rows nobody looks
+    up, rows looked up more than 64 times; small integers so that every sum is
+    exact and the result must equal the oracle bit for bit."""
+    gen = torch.Generator().manual_seed(dim + rows + tokens)
+    lo, hi = 3, 3 + rows
+    ids = torch.randint(0, hi + 4, (tokens,), generator=gen).to(idt)
+    dy = torch.randint(-2, 3, (tokens, dim), generator=gen).to(dtype)
+    pad = lo + rows // 2
+    got = ops.embedding_backward(dy.cuda(), ids.cuda(), lo, hi, padding_idx=pad)
+    want = o_emb.backward(dy.double().numpy(), ids.numpy(), lo, hi, padding_idx=pad)
+    assert np.abs(want).max() <= 256 or dtype == torch.float32
+    assert got.shape == (rows, dim) and got.dtype == dtype
+    assert np.array_equal(got.cpu().double().numpy(), want)
+    # no padding row, 2-D ids
+    got = ops.embedding_backward(dy.cuda().reshape(1, tokens, dim), ids.cuda().reshape(1, tokens), lo, hi)
+    want = o_emb.backward(dy.double().numpy(), ids.numpy(), lo, hi)
+    if np.abs(want).max() <= 256 or dtype == torch.float32:
+        assert np.array_equal(got.cpu().double().numpy(), want)
+
+
+def test_embedding_backward_matches_torch_autograd_on_random_data(ops):
+    """Random bf16 gradients: fp32 accumulation and one bf16 rounding, against
+    the exact sums; and the layer-level autograd path."""
+    from distdl_amd.nn.embedding import _EmbeddingShard
+    gen = torch.Generator().manual_seed(12)
+    table = (0.02 * torch.randn(300, 256, generator=gen)).to(torch.bfloat16)
+    ids = torch.randint(0, 300, (8, 500), generator=gen)
+    dy = torch.randn(8, 500, 256, generator=gen).to(torch.bfloat16)
+    w = table.cuda().requires_grad_(True)
+    out = _EmbeddingShard.apply(w, ids.cuda(), 0, 300, None)
+    out.backward(dy.cuda())
+    exact = o_emb.backward(dy.double().numpy(), ids.numpy(), 0, 300)
+    got = w.grad.cpu().double().numpy()
+    assert (np.abs(got - exact) <= 2.0 ** -8 * np.abs(exact) + 1e-6).all()
+    # and the same through torch on the CPU in float32 (the reference's call)
+    tw = table.float().requires_grad_(True)
+    F.embedding(ids, tw).backward(dy.float())
+    assert np.allclose(got, tw.grad.double().numpy(), rtol=2.0 ** -7, atol=1e-4)
+
+
+def test_embedding_backward_config3_rank0(ops):
+    """Config 3 shapes: 131072 tokens over a 128256-row vocabulary, shard rows
+    [0,16032), dim 4096 (gradient restricted to 1024 columns to keep the test
+    small on the host side)."""
+    gen = torch.Generator().manual_seed(1003)
+    ids = torch.randint(0, 128256, (32, 4096), generator=gen)
+    dy = torch.randint(-1, 2, (32, 4096, 1024), generator=gen, dtype=torch.int8).to(torch.bfloat16)
+    got = ops.embedding_backward(dy.cuda(), ids.cuda(), 0, 16032)
+    torch.cuda.synchronize()
+    # size-independent checks: column sums over all rows equal the column sums of the hit tokens' gradients
+    hit = ids < 16032
+    want_total = dy[hit].double().sum(0)
+    assert torch.equal(got.cpu().double().sum(0), want_total)
+    # rows never looked up are zero, a sample of rows is exact
+    looked = torch.zeros(16032, dtype=torch.bool)
+    looked[ids[hit]] = True
+    assert int((got.cpu()[~looked] != 0).sum()) == 0
+    sample = torch.nonzero(looked).flatten()[:64]
+    for r in sample.tolist():
+        assert torch.equal(got[r].cpu().double(), dy[ids == r].double().sum(0))
+
+
 # ------------------------------------------------------------------- Linear --
 
 def _lin_check(got_bits, x, w, b, sample_rows=None):

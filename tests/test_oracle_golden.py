@@ -398,3 +398,16 @@ def test_layernorm_backward_oracle_matches_autograd_of_the_reference_sequence(wi
         (F.layer_norm(x, (sum(widths),), g, b, eps) * torch.cat(dys, dim=1)).sum().backward()
         assert np.allclose(np.concatenate(dxs, axis=1), x.grad.numpy(), rtol=1e-9, atol=1e-11)
         assert np.allclose(np.concatenate(dgs), g.grad.numpy(), rtol=1e-9, atol=1e-11)
+
+
+def test_embedding_backward_oracle_matches_torch_autograd():
+    torch.manual_seed(6)
+    table = torch.randn(20, 5, dtype=torch.float64, requires_grad=True)
+    ids = torch.randint(0, 20, (4, 9))
+    dy = torch.randn(4, 9, 5, dtype=torch.float64)
+    F.embedding(ids, table, padding_idx=3).backward(dy)
+    got = o_emb.backward(dy.numpy(), ids.numpy(), 0, 20, padding_idx=3)
+    assert np.allclose(got, table.grad.numpy(), rtol=1e-13, atol=1e-13)
+    # a window: exactly the rows [lo, hi) of the full gradient (padding row excluded as above)
+    full = o_emb.backward(dy.numpy(), ids.numpy(), 0, 20)
+    assert np.array_equal(o_emb.backward(dy.numpy(), ids.numpy(), 5, 12), full[5:12])
