@@ -27,18 +27,27 @@ from .module import Module
 
 
 class _HaloStaging(torch.autograd.Function):
-    """pad + exchange of one shard through the fused kernel."""
+    """pad + exchange of one shard through the fused kernel.  With respect to
+    the shard the operation is an embedding into the padded tensor (the ghost
+    strips are filled from buffers, not from the shard), so its adjoint is the
+    crop of the padded gradient -- a strided box copy."""
 
     @staticmethod
     def forward(ctx, input, plan, ghost_bufs, bulk_bufs):
         x = input.detach()
         if not x.is_contiguous():
             x = x.contiguous()
+        ctx.plan = plan
         return plan.run(x, ghost_bufs, bulk_bufs)
 
     @staticmethod
     def backward(ctx, grad_output):
-        raise NotImplementedError("the adjoint of the fused halo staging is not part of this build")
+        plan = ctx.plan
+        g = grad_output.detach()
+        dx = torch.empty(plan.x_shape, dtype=g.dtype, device=g.device)
+        inner = [slice(p[0], p[0] + n) for p, n in zip(plan.pad, plan.x_shape)]
+        hip_ops.copy_box(g, inner, dx, [slice(0, n) for n in plan.x_shape])
+        return dx, None, None, None
 
 
 class DistributedFeatureConvBase(Module, HaloMixin, ConvMixin):
@@ -98,9 +107,12 @@ class DistributedFeatureConvBase(Module, HaloMixin, ConvMixin):
             else:
                 self.register_buffer('bias', None)
         else:
-            self.register_buffer('weight', zero_volume_tensor(device=P_x.device))
+            # Like the parameters they stand for, the empty tensors of the other
+            # workers require gradients (reference :174-187): autograd then runs
+            # the broadcast adjoint -- a collective -- on every worker.
+            self.register_buffer('weight', zero_volume_tensor(device=P_x.device, requires_grad=True))
             if bias:
-                self.register_buffer('bias', zero_volume_tensor(device=P_x.device))
+                self.register_buffer('bias', zero_volume_tensor(device=P_x.device, requires_grad=True))
             else:
                 self.register_buffer('bias', None)
 
