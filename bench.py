@@ -37,13 +37,15 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # WRITE_SIZE runs of these same workloads, each counter scaled by what it reads
 # for a plain 64 MiB device copy (FETCH_SIZE x1.9993, WRITE_SIZE x1.0000); the
 # summaries are profiles/*_hbm_traffic_pmc.txt.  layernorm is the mean of its two
-# kernels (stats 8 498 546 B, normalize 17 132 572 B), like its launch time.
+# kernels (stats 8 482 114 B, normalize 17 875 673 B), like its launch time;
+# linear is the sum of the two launches of a step (256-wide tiles 436 357 536 B,
+# 192-wide tiles 396 782 657 B).
 MEASURED_TRAFFIC_BYTES = {
-    "repartition": 134419452,
-    "layernorm": 12815559,
-    "embedding": 1210713945,
-    "linear": 1009567583,
-    "halo": 579156303,
+    "repartition": 134414544,
+    "layernorm": 13178894,
+    "embedding": 1210703742,
+    "linear": 833140193,
+    "halo": 579271283,
 }
 
 
