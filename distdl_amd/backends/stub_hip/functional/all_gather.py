@@ -1,9 +1,61 @@
-"""All-gather stand-in (reference: backends/mpi_numpy/functional/all_gather.py:88-149).
-A collective followed by a local re-layout; outside this build."""
+"""All-gather along one partitioned axis and its adjoint (reference:
+backends/mpi_numpy/functional/all_gather.py:88-149, :152-230).  The collective
+itself belongs to the transport; what runs here is the local re-layout the
+reference does with einops (``p a b c -> a (p b) c``, zero-padding and stripping
+uneven shards): the P received pieces are unpacked into their slabs of the
+output by one launch of the box kernel, uneven pieces included.  The adjoint is
+a reduce-scatter: every worker sums its slab of all workers' gradients
+(strided reads, accumulating box copies)."""
 
-__all__ = ["AllGatherFunction"]
+__all__ = ["AllGatherFunction", "gather_slabs", "reduce_scatter_slabs"]
 
+import numpy as np
 import torch
+
+from .... import hip_ops
+from ....utilities.slicing import compute_subshape
+
+
+def gather_slabs(P, local, axis, tag):
+    """``local`` of every worker of ``P``, concatenated along ``axis`` in rank order."""
+    transport = P._world.transport
+    x = local if local.is_contiguous() else local.contiguous()
+    parts = transport.gather_list(P, x, tag=tag)
+    extent = sum(int(p.shape[axis]) for p in parts)
+    shape = list(x.shape)
+    shape[axis] = extent
+    out = torch.empty(shape, dtype=x.dtype, device=x.device)
+    boxes, start = [], 0
+    for p in parts:
+        origin = [0] * out.dim()
+        origin[axis] = start
+        boxes.append((origin, list(p.shape)))
+        start += int(p.shape[axis])
+    hip_ops.BoxPlan(out.shape, out.stride(), boxes).unpack(out, parts)
+    transport.release(P, tag=tag)
+    return out
+
+
+def reduce_scatter_slabs(P, full, axis, tag):
+    """Sum over the workers of ``P`` of their ``full`` tensors, of which this
+    worker keeps its balanced slab along ``axis``."""
+    transport = P._world.transport
+    g = full if full.is_contiguous() else full.contiguous()
+    grads = transport.gather_list(P, g, tag=tag)
+    me = int(P.rank)
+    extent = int(g.shape[axis])
+    sizes = [int(np.asarray(compute_subshape(P.size, r, extent)).reshape(-1)[0]) for r in range(P.size)]
+    start = sum(sizes[:me])
+    shape = list(g.shape)
+    shape[axis] = sizes[me]
+    out = torch.empty(shape, dtype=g.dtype, device=g.device)
+    src = [slice(0, int(n)) for n in g.shape]
+    src[axis] = slice(start, start + sizes[me])
+    dst = [slice(0, int(n)) for n in shape]
+    for q, gq in enumerate(grads):
+        hip_ops.copy_box(gq, src, out, dst, accumulate=q > 0)
+    transport.release(P, tag=tag)
+    return out
 
 
 class AllGatherFunction(torch.autograd.Function):
@@ -11,9 +63,15 @@ class AllGatherFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input, P_allgather, axis=None, tag=None):
         if not P_allgather.active or P_allgather.size == 1:
+            ctx.identity = True
             return input
-        raise NotImplementedError("AllGather is a collective, not part of this build")
+        ctx.identity = False
+        ctx.P, ctx.axis, ctx.tag = P_allgather, int(axis), tag
+        return gather_slabs(P_allgather, input.detach(), int(axis), ("all_gather", tag))
 
     @staticmethod
     def backward(ctx, grad_output):
-        raise NotImplementedError("the adjoint of AllGather is a collective, not part of this build")
+        if ctx.identity:
+            return grad_output, None, None, None
+        dx = reduce_scatter_slabs(ctx.P, grad_output.detach(), ctx.axis, ("all_gather_adjoint", ctx.tag))
+        return dx, None, None, None

@@ -110,6 +110,21 @@ class SoloTransport:
         absent too."""
         return grad if P_src.active else None
 
+    def gather_list(self, P, tensor, tag=None):
+        """The tensors of all workers of ``P`` in rank order.  The absent
+        workers hold what the live one holds unless a provider says otherwise."""
+        fn = self._gather_providers.get(tag)
+        if fn is None:
+            return [tensor] * P.size
+        parts = list(fn(P, tensor))
+        if len(parts) != P.size:
+            raise TransportError(f"gather provider for {tag!r} returned {len(parts)} parts for {P.size} workers")
+        parts[P.rank] = tensor
+        return parts
+
+    def release(self, P, tag=None):
+        return None
+
 
 # ---------------------------------------------------------------------------
 # Loopback
@@ -301,6 +316,17 @@ class LoopbackTransport:
             out = match.clone()
         self._allgather_obj(union, None, ("tbcast-done", tag))
         return out
+
+    def gather_list(self, P, tensor, tag=None):
+        """The tensors of all workers of ``P`` in rank order (shapes may differ).
+        They are the peers' own tensors: read them, then call :meth:`release`."""
+        return self._allgather_obj(P, tensor, ("tlist", tag))
+
+    def release(self, P, tag=None):
+        """Every worker of ``P`` has enqueued its reads of the tensors handed
+        out by :meth:`gather_list`; the rank threads share one stream, so the
+        owners may reuse them from here on."""
+        self._allgather_obj(P, None, ("tlist-done", tag))
 
     def broadcast_adjoint(self, P_src, P_dst, grad, tag=None):
         """Sum-reduce: every worker of ``P_src`` receives the sum of the

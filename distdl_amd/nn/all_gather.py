@@ -1,9 +1,10 @@
-"""AllGather layer stand-in (reference: nn/all_gather.py).  Under the solo
-transport the caller supplies the already gathered activation and the layer is
-the identity; under loopback the shards are concatenated along the axis."""
+"""AllGather layer (reference: nn/all_gather.py): concatenates the shards of
+the workers that differ along ``axes_all_gather``.  Under the solo transport the
+caller supplies the already gathered activation and the layer is the identity;
+otherwise the backend's AllGatherFunction runs (box-kernel re-layout forward,
+reduce-scatter adjoint)."""
 
 import numpy as np
-import torch
 
 from .module import Module
 
@@ -15,6 +16,8 @@ class AllGather(Module):
         self.P_x = P_x
         if not P_x.active:
             return
+        if scale_backward is not None:
+            raise NotImplementedError("scale_backward is not part of this build")
         if axes_all_gather is None:
             axes_all_gather = [d for d in range(P_x.dim) if d not in [int(a) for a in axes_keep]]
         self.axes = tuple(int(a) for a in axes_all_gather)
@@ -30,5 +33,5 @@ class AllGather(Module):
             return input  # solo: the input already is the gathered tensor
         if len(self.axes) != 1:
             raise NotImplementedError("AllGather along several axes is not part of this build")
-        parts = transport.allgather(self.P_allgather, input.detach(), tag="all_gather")
-        return torch.cat(list(parts), dim=self.axes[0])
+        Function = self._distdl_backend.functional.all_gather.AllGatherFunction
+        return Function.apply(input, self.P_allgather, self.axes[0], None)

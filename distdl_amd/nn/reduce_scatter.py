@@ -1,0 +1,33 @@
+"""ReduceScatter layer (reference: nn/reduce_scatter.py): sums the tensors of
+the workers that differ along ``axes_reduce_scatter`` and leaves every worker
+its balanced slab of the sum.  Under the solo transport the layer keeps the live
+worker's slab of its own tensor (the absent workers contribute nothing)."""
+
+import numpy as np
+
+from .module import Module
+
+
+class ReduceScatter(Module):
+
+    def __init__(self, P_x, axes_reduce_scatter=None, axes_keep=None, scale_backward=None):
+        super().__init__()
+        self.P_x = P_x
+        if not P_x.active:
+            return
+        if scale_backward is not None:
+            raise NotImplementedError("scale_backward is not part of this build")
+        if axes_reduce_scatter is None:
+            axes_reduce_scatter = [d for d in range(P_x.dim) if d not in [int(a) for a in axes_keep]]
+        self.axes = tuple(int(a) for a in axes_reduce_scatter)
+        keep = [d in self.axes for d in range(P_x.dim)]
+        self.P_reducescatter = P_x.create_cartesian_subtopology_partition(keep)
+        self.identity = int(np.prod(self.P_reducescatter.shape)) == 1
+
+    def forward(self, input):
+        if not self.P_x.active or self.identity:
+            return input
+        if len(self.axes) != 1:
+            raise NotImplementedError("ReduceScatter along several axes is not part of this build")
+        Function = self._distdl_backend.functional.reduce_scatter.ReduceScatterFunction
+        return Function.apply(input, self.P_reducescatter, self.axes[0], None)

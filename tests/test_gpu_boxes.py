@@ -286,3 +286,50 @@ def test_transpose_network_buffers_and_adjoint(golden):
     y, dx = res[0][1], res[0][2]
     assert torch.equal(y, x0)                      # scatter ... gather is the identity
     assert torch.equal(dx, dy0)
+
+
+# ------------------------------------------------- all-gather / reduce-scatter --
+
+@pytest.mark.parametrize("P,shape,axis", [([1, 4], [3, 10], 1), ([3, 1, 1], [7, 2, 5], 0), ([1, 2, 1], [2, 9, 4], 1),
+                                          ([1, 1, 4], [2, 3, 8], 2)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_all_gather_and_reduce_scatter_layers(P, shape, axis, dtype):
+    """Loopback over all workers.  AllGather: every worker ends with the
+    concatenation of the (possibly uneven) shards, bit for bit; its backward is
+    the reduce-scatter of the gradients.  ReduceScatter: the slab of the sum;
+    its backward is the all-gather.  Values are small integers, so the sums are
+    exact in either dtype."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import AllGather
+    from distdl_amd.nn import ReduceScatter
+    from oracle import repartition as o_rep
+    n = int(np.prod(P))
+    rng = np.random.default_rng(sum(shape) + axis)
+    x = rng.integers(-3, 4, size=shape).astype(np.float32)
+    shards = o_rep.scatter(x, P)                                   # balanced split, first workers larger
+    dys = [rng.integers(-3, 4, size=shape).astype(np.float32) for _ in range(n)]
+    fulls = [rng.integers(-3, 4, size=shape).astype(np.float32) for _ in range(n)]
+    dzs = o_rep.scatter(rng.integers(-3, 4, size=shape).astype(np.float32), P)
+
+    def body(P_world):
+        P_x = P_world.create_partition_inclusive(list(range(n))).create_cartesian_topology_partition(P)
+        r = P_x.rank
+        xin = torch.from_numpy(shards[r]).to(dtype).cuda().requires_grad_(True)
+        y = AllGather(P_x, axes_all_gather=(axis,))(xin)
+        y.backward(torch.from_numpy(dys[r]).to(dtype).cuda())
+        fin = torch.from_numpy(fulls[r]).to(dtype).cuda().requires_grad_(True)
+        z = ReduceScatter(P_x, axes_reduce_scatter=(axis,))(fin)
+        z.backward(torch.from_numpy(dzs[r]).to(dtype).cuda())
+        torch.cuda.synchronize()
+        return (y.detach().float().cpu().numpy(), xin.grad.float().cpu().numpy(),
+                z.detach().float().cpu().numpy(), fin.grad.float().cpu().numpy())
+
+    outs = SimWorld(n).run(body)
+    want_dx = o_rep.scatter(sum(dys), P)
+    want_z = o_rep.scatter(sum(fulls), P)
+    dz_full = np.concatenate([dzs[r] for r in range(n)], axis=axis)
+    for r, (y, dx, z, dfull) in enumerate(outs):
+        assert np.array_equal(y, x)
+        assert np.array_equal(dx, want_dx[r])
+        assert np.array_equal(z, want_z[r])
+        assert np.array_equal(dfull, dz_full)
