@@ -55,7 +55,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default=None, help="run a single workload (repartition, layernorm, embedding, linear, halo, calib)")
+    ap.add_argument("--only", default=None, help="run a single workload (repartition, layernorm, layernorm_long, embedding, linear, halo, calib)")
     ap.add_argument("--no-graph", action="store_true", help="launch on the stream instead of replaying a HIP graph")
     return ap.parse_args()
 
@@ -216,6 +216,39 @@ def build_layernorm(torch, lib, _lib, nsets):
     return steps, keep, 25298944
 
 
+def build_layernorm_long(torch, lib, _lib, nsets):
+    """The kernels of config 1 on 32 times its rows ([262144, 256] fp32, 268 MB):
+    the streaming rate of the same code once launch ramp and memory latency no
+    longer dominate.  Not a BASELINE configuration; reported next to config 1."""
+    rows, cols = 32 * 16 * 512, 256
+    keep, steps = [], []
+    part_cols = _lib.i64_array([256] * 4)
+    for s in range(nsets):
+        gen = torch.Generator(device="cuda").manual_seed(2001 + s)
+        x = torch.randn(rows, cols, generator=gen, device="cuda")
+        gamma = 1 + 0.1 * torch.randn(cols, generator=gen, device="cuda")
+        beta = 0.1 * torch.randn(cols, generator=gen, device="cuda")
+        gathered = torch.zeros(4, rows, 2, device="cuda")
+        gathered[1:, :, 1] = 256.0                                   # peers: mean 0, M2 = n (unit variance)
+        y = torch.empty_like(x)
+        stats_args = (x.data_ptr(), rows, cols, cols, gathered.data_ptr())
+        norm_args = (x.data_ptr(), rows, cols, cols, gathered.data_ptr(), 4, part_cols, gamma.data_ptr(),
+                     beta.data_ptr(), 1e-5, y.data_ptr(), cols, None, None)
+        keep.append((x, gamma, beta, gathered, y, stats_args, norm_args))
+
+        def stats(a=stats_args):
+            rc = lib.ddl_ln_partial_stats_f32(*a, STREAM[0])
+            if rc:
+                _lib.check(rc, "ddl_ln_partial_stats_f32")
+
+        def norm(a=norm_args):
+            rc = lib.ddl_ln_normalize_affine_f32(*a, STREAM[0])
+            if rc:
+                _lib.check(rc, "ddl_ln_normalize_affine_f32")
+        steps.append([stats, norm])
+    return steps, keep, 32 * 25298944 - 31 * 2 * 256 * 4
+
+
 def build_embedding(torch, lib, _lib, nsets):
     """Config 3: rank-0 vocabulary shard [16032,4096] bf16, ids [32,4096] int64."""
     gen = torch.Generator().manual_seed(1003)
@@ -362,6 +395,7 @@ def main():
     builders = {
         "repartition": (build_repartition, 8, 2, "hbm"),
         "layernorm": (build_layernorm, 64, 2, "hbm"),
+        "layernorm_long": (build_layernorm_long, 3, 2, "hbm"),
         "embedding": (build_embedding, 4, 1, "hbm"),
         "linear": (build_linear, 4, 1, "mfma"),
         "halo": (build_halo, 4, 1, "hbm"),
