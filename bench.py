@@ -55,7 +55,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default=None, help="run a single workload (repartition, layernorm, layernorm_long, embedding, linear, halo, calib)")
+    ap.add_argument("--only", default=None, help="run a single workload (repartition, layernorm, layernorm_long, embedding, linear, halo, layernorm_bwd, embedding_bwd, linear_bwd, calib)")
     ap.add_argument("--no-graph", action="store_true", help="launch on the stream instead of replaying a HIP graph")
     return ap.parse_args()
 
@@ -325,6 +325,100 @@ def build_halo(torch, lib, _lib, nsets):
     return steps, keep, 562531072
 
 
+# ----------------------------------------------------------------------------
+# backward (adjoint) workloads: the same shapes as the forward configurations
+# ----------------------------------------------------------------------------
+
+def _call(lib, _lib, name, args):
+    def fn(a=args, f=getattr(lib, name), n=name):
+        rc = f(*a, STREAM[0])
+        if rc:
+            _lib.check(rc, n)
+    return fn
+
+
+def build_layernorm_bwd(torch, lib, _lib, nsets):
+    """Backward of config 1 on rank 0: row sums, input gradient, parameter
+    gradients.  Algorithmic bytes: dy and x are read three times (once per
+    kernel), dx is written once: 7 x 8 388 608 B, plus the small vectors."""
+    rows, cols = 16 * 512, 256
+    keep, steps = [], []
+    for s in range(nsets):
+        gen = torch.Generator(device="cuda").manual_seed(4001 + s)
+        x = torch.randn(rows, cols, generator=gen, device="cuda")
+        dy = torch.randn(rows, cols, generator=gen, device="cuda")
+        gamma = 1 + 0.1 * torch.randn(cols, generator=gen, device="cuda")
+        mean = 0.01 * torch.randn(rows, generator=gen, device="cuda")
+        rstd = 1 + 0.01 * torch.randn(rows, generator=gen, device="cuda")
+        sums = torch.zeros(4, rows, 2, device="cuda")                     # slot 0 is written by the kernel, 1..3 seeded
+        dx = torch.empty_like(x)
+        dg, db = torch.empty(cols, device="cuda"), torch.empty(cols, device="cuda")
+        work = torch.empty(2 * 256 * cols, device="cuda")
+        keep.append((x, dy, gamma, mean, rstd, sums, dx, dg, db, work))
+        a1 = (dy.data_ptr(), x.data_ptr(), rows, cols, cols, cols, mean.data_ptr(), rstd.data_ptr(), gamma.data_ptr(),
+              sums.data_ptr())
+        a2 = (dy.data_ptr(), x.data_ptr(), rows, cols, cols, cols, mean.data_ptr(), rstd.data_ptr(), gamma.data_ptr(),
+              sums.data_ptr(), 4, 1.0 / (4 * cols), dx.data_ptr(), cols)
+        a3 = (dy.data_ptr(), x.data_ptr(), rows, cols, cols, cols, mean.data_ptr(), rstd.data_ptr(), dg.data_ptr(),
+              db.data_ptr(), work.data_ptr(), work.numel())
+        steps.append([_call(lib, _lib, "ddl_ln_bwd_partial_f32", a1), _call(lib, _lib, "ddl_ln_bwd_input_f32", a2),
+                      _call(lib, _lib, "ddl_ln_bwd_params_f32", a3)])
+    return steps, keep, 7 * rows * cols * 4 + 3 * (2 * rows * 4) + 5 * rows * 2 * 4 + 3 * cols * 4
+
+
+def build_embedding_bwd(torch, lib, _lib, nsets):
+    """Backward of config 3 on rank 0: gradient of the [16032, 4096] bf16 shard
+    from dy [32, 4096, 4096].  Algorithmic bytes: the dy rows of the hit tokens,
+    the ids (read twice), the whole gradient written once."""
+    keep, steps, nbytes = [], [], []
+    gen = torch.Generator(device="cuda").manual_seed(5003)
+    dy = torch.randn(32, 4096, 4096, generator=gen, device="cuda").to(torch.bfloat16)
+    keep.append(dy)
+    for s in range(nsets):
+        g = torch.Generator().manual_seed(2003 + s)
+        ids = torch.randint(0, 128256, (32, 4096), generator=g)
+        n_hit = int((ids < 16032).sum())
+        nbytes.append(n_hit * 8192 + 2 * ids.numel() * 8 + 16032 * 4096 * 2)
+        ids = ids.cuda()
+        dw = torch.empty(16032, 4096, dtype=torch.bfloat16, device="cuda")
+        work = torch.empty(2 * 16032 + 1 + ids.numel(), dtype=torch.int32, device="cuda")
+        keep.append((ids, dw, work))
+        args = (dy.data_ptr(), _lib.DDL_DT_BF16, 4096, 4096, ids.data_ptr(), 1, ids.numel(), 0, 16032, -1, dw.data_ptr(),
+                4096, work.data_ptr(), work.numel())
+        steps.append([_call(lib, _lib, "ddl_embedding_backward", args)])
+    return steps, keep, sum(nbytes) / len(nbytes)
+
+
+def build_linear_bwd(torch, lib, _lib, nsets):
+    """Backward of config 4 on rank 0: dx = dy w and dw = dy^T x through the
+    shard GEMM on transposed operands (the three transposes are part of the
+    step), db = column sums of dy.  Work: 2 x 2 M N K flop."""
+    M, N, K = 8192, 3584, 8192
+    gen = torch.Generator(device="cuda").manual_seed(6004)
+    w = (0.02 * torch.randn(N, K, generator=gen, device="cuda")).to(torch.bfloat16)
+    w_t = torch.empty(K, N, dtype=torch.bfloat16, device="cuda")
+    dy_t = torch.empty(N, M, dtype=torch.bfloat16, device="cuda")
+    x_t = torch.empty(K, M, dtype=torch.bfloat16, device="cuda")
+    work = torch.empty(64 * N, device="cuda")
+    keep, steps = [w, w_t, dy_t, x_t, work], []
+    for s in range(nsets):
+        x = torch.randn(M, K, generator=gen, device="cuda").to(torch.bfloat16)
+        dy = torch.randn(M, N, generator=gen, device="cuda").to(torch.bfloat16)
+        dx = torch.empty(M, K, dtype=torch.bfloat16, device="cuda")
+        dw = torch.empty(N, K, dtype=torch.bfloat16, device="cuda")
+        db = torch.empty(N, dtype=torch.bfloat16, device="cuda")
+        keep.append((x, dy, dx, dw, db))
+        steps.append([
+            _call(lib, _lib, "ddl_transpose_2d", (w.data_ptr(), w_t.data_ptr(), N, K, K, N, 2)),
+            _call(lib, _lib, "ddl_linear_bf16", (dy.data_ptr(), w_t.data_ptr(), None, dx.data_ptr(), M, K, N, N, N, K)),
+            _call(lib, _lib, "ddl_transpose_2d", (dy.data_ptr(), dy_t.data_ptr(), M, N, N, M, 2)),
+            _call(lib, _lib, "ddl_transpose_2d", (x.data_ptr(), x_t.data_ptr(), M, K, K, M, 2)),
+            _call(lib, _lib, "ddl_linear_bf16", (dy_t.data_ptr(), x_t.data_ptr(), None, dw.data_ptr(), N, K, M, M, M, K)),
+            _call(lib, _lib, "ddl_colsum_bf16", (dy.data_ptr(), M, N, N, db.data_ptr(), work.data_ptr(), work.numel())),
+        ])
+    return steps, keep, 2 * 2 * M * N * K
+
+
 def build_calib(torch, lib, _lib, nsets):
     """Counter calibration: a plain contiguous device-to-device copy of 64 MiB
     (torch's own copy kernel), so that FETCH_SIZE / WRITE_SIZE readings of the
@@ -399,6 +493,9 @@ def main():
         "embedding": (build_embedding, 4, 1, "hbm"),
         "linear": (build_linear, 4, 1, "mfma"),
         "halo": (build_halo, 4, 1, "hbm"),
+        "layernorm_bwd": (build_layernorm_bwd, 32, 3, "hbm"),
+        "embedding_bwd": (build_embedding_bwd, 4, 1, "hbm"),
+        "linear_bwd": (build_linear_bwd, 2, 1, "mfma"),
         "calib": (build_calib, 4, 1, "hbm"),     # only with --only calib
     }
     names = [args.only] if args.only else [n for n in builders if n != "calib"]

@@ -15,7 +15,7 @@
 //   emb_bwd_clear    counters = 0
 //   emb_bwd_count    count[row]++ per token in the window
 //   emb_bwd_scan     start[row] = exclusive prefix sum of count (one workgroup)
-//   emb_bwd_fill     bucket[start[row] + cursor[row]++] = t
+//   emb_bwd_fill     bucket[start[row]++] = t, which leaves start[row] at the bucket's end
 //   emb_bwd_reduce   sort each bucket (it is short), sum, convert, store
 #include "ddl_common.h"
 
@@ -48,40 +48,75 @@ __global__ __launch_bounds__(kBlock) void emb_bwd_count(const IdT* __restrict__ 
     if (r >= 0) atomicAdd(&count[r], 1);
 }
 
-// Exclusive prefix sum of count[0..n) into start[0..n], start[n] = total.
+// Exclusive prefix sum of count[0..n) into start[0..n), one workgroup, 16384
+// counters per round.  The counters come in and the sums go out with
+// consecutive lanes on consecutive addresses; in between they sit in LDS, where
+// a thread owns 16 consecutive ones (pitch 17 keeps the lanes on different
+// banks).  Thread totals are scanned across the wavefront with shuffles, the 16
+// wavefront totals through LDS.
+constexpr int kScanItems = 16;
+constexpr int kScanWaves = kScanBlock / kWave;
+constexpr int kScanRound = kScanBlock * kScanItems;
+__device__ inline int scan_slot(int i) { return i + (i >> 4); }
 __global__ __launch_bounds__(kScanBlock) void emb_bwd_scan(const int32_t* __restrict__ count, int64_t n, int32_t* __restrict__ start) {
-    __shared__ int32_t part[kScanBlock];
-    __shared__ int32_t carry_s;
-    if (threadIdx.x == 0) carry_s = 0;
-    __syncthreads();
-    for (int64_t base = 0; base < n; base += kScanBlock) {
-        const int64_t i = base + threadIdx.x;
-        const int32_t v = i < n ? count[i] : 0;
-        part[threadIdx.x] = v;
-        __syncthreads();
-        for (int off = 1; off < kScanBlock; off <<= 1) {     // Hillis-Steele inclusive scan
-            const int32_t add = threadIdx.x >= static_cast<unsigned>(off) ? part[threadIdx.x - off] : 0;
-            __syncthreads();
-            part[threadIdx.x] += add;
-            __syncthreads();
+    __shared__ int32_t stage[kScanRound + kScanRound / 16];
+    __shared__ int32_t wave_total[kScanWaves];
+    const int t = threadIdx.x, lane = t & (kWave - 1), wave = t / kWave;
+    int32_t carry = 0;                                         // sum of all earlier rounds, the same in every thread
+    for (int64_t base = 0; base < n; base += kScanRound) {
+#pragma unroll
+        for (int j = 0; j < kScanItems; ++j) {
+            const int i = j * kScanBlock + t;
+            stage[scan_slot(i)] = base + i < n ? count[base + i] : 0;
         }
-        const int32_t carry = carry_s;
-        if (i < n) start[i] = carry + part[threadIdx.x] - v;
         __syncthreads();
-        if (threadIdx.x == kScanBlock - 1) carry_s = carry + part[kScanBlock - 1];
+        int32_t v[kScanItems];
+        int32_t total = 0;
+#pragma unroll
+        for (int k = 0; k < kScanItems; ++k) {
+            v[k] = stage[scan_slot(t * kScanItems + k)];
+            total += v[k];
+        }
+        int32_t incl = total;                                  // inclusive scan over the wavefront
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            const int32_t up = __shfl_up(incl, off, kWave);
+            if (lane >= off) incl += up;
+        }
+        if (lane == kWave - 1) wave_total[wave] = incl;
         __syncthreads();
+        int32_t before = 0, all = 0;
+#pragma unroll
+        for (int k = 0; k < kScanWaves; ++k) {
+            const int32_t wt = wave_total[k];
+            before += k < wave ? wt : 0;
+            all += wt;
+        }
+        int32_t run = carry + before + incl - total;
+#pragma unroll
+        for (int k = 0; k < kScanItems; ++k) {
+            stage[scan_slot(t * kScanItems + k)] = run;
+            run += v[k];
+        }
+        carry += all;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < kScanItems; ++j) {
+            const int i = j * kScanBlock + t;
+            if (base + i < n) start[base + i] = stage[scan_slot(i)];
+        }
+        __syncthreads();                                       // stage and wave_total are rewritten by the next round
     }
-    if (threadIdx.x == 0) start[n] = carry_s;
 }
 
 template <typename IdT>
 __global__ __launch_bounds__(kBlock) void emb_bwd_fill(const IdT* __restrict__ ids, int64_t n_ids, int64_t lo, int64_t hi,
-                                                       int64_t padding_idx, const int32_t* __restrict__ start,
-                                                       int32_t* __restrict__ cursor, int32_t* __restrict__ bucket) {
+                                                       int64_t padding_idx, int32_t* __restrict__ start,
+                                                       int32_t* __restrict__ bucket) {
     const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
     if (t >= n_ids) return;
     const int64_t r = token_row(ids, t, lo, hi, padding_idx);
-    if (r >= 0) bucket[start[r] + atomicAdd(&cursor[r], 1)] = static_cast<int32_t>(t);
+    if (r >= 0) bucket[atomicAdd(&start[r], 1)] = static_cast<int32_t>(t);   // start[r] ends as the end of bucket r
 }
 
 __device__ inline float load_as_f32(const uint16_t* p) { return __uint_as_float(static_cast<uint32_t>(*p) << 16); }
@@ -98,6 +133,22 @@ __device__ inline void store_from_f32(uint16_t* p, float f) {
 }
 __device__ inline void store_from_f32(float* p, float f) { *p = f; }
 
+// Order of the tokens of a bucket of at most 64: lane i holds one token and
+// counts the smaller ones (its rank), then every lane picks the token whose
+// rank is its own lane number.  Ascending token order makes the sums
+// independent of how the fill kernel's atomics interleaved; longer buckets are
+// taken as they are.
+__device__ inline int32_t sort_bucket(int32_t mine, int32_t m, int lane) {
+    int32_t rank = 0;
+    for (int k = 0; k < m; ++k) rank += __shfl(mine, k, kWave) < mine ? 1 : 0;
+    int32_t sorted = 0x7FFFFFFF;
+    for (int k = 0; k < m; ++k) {
+        const int32_t tk = __shfl(mine, k, kWave), rk = __shfl(rank, k, kWave);
+        if (rk == lane) sorted = tk;
+    }
+    return sorted;
+}
+
 // Wavefront (row, chunk): columns chunk * kChunk + lane + 64 j, j = 0..7.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void emb_bwd_reduce(const T* __restrict__ dy, int64_t dim, int64_t ld_dy,
@@ -108,27 +159,13 @@ __global__ __launch_bounds__(kBlock) void emb_bwd_reduce(const T* __restrict__ d
     const int64_t row = w / chunks;
     const int chunk = static_cast<int>(w - row * chunks);
     if (row >= rows) return;
-    const int32_t b0 = start[row], n = start[row + 1] - b0;
+    const int32_t b0 = row ? start[row - 1] : 0, n = start[row] - b0;   // the fill pass moved start[r] to the end of bucket r
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const int64_t c0 = static_cast<int64_t>(chunk) * kChunk + lane;
-    // Ascending token order makes the sum independent of how the fill kernel's
-    // atomics interleaved.  Buckets of up to 64 tokens are ordered by rank (lane
-    // i holds one token and counts the smaller ones); longer ones are taken as
-    // they are.
     for (int32_t base = 0; base < n; base += kWave) {
         const int32_t m = n - base < kWave ? n - base : kWave;
         int32_t mine = lane < m ? bucket[b0 + base + lane] : 0x7FFFFFFF;
-        if (n <= kWave) {
-            int32_t rank = 0;
-            for (int k = 0; k < m; ++k) rank += __shfl(mine, k, kWave) < mine ? 1 : 0;
-            // scatter by rank: lane r reads the token whose rank is r
-            int32_t sorted = 0x7FFFFFFF;
-            for (int k = 0; k < m; ++k) {
-                const int32_t tk = __shfl(mine, k, kWave), rk = __shfl(rank, k, kWave);
-                if (rk == lane) sorted = tk;
-            }
-            mine = sorted;
-        }
+        if (n <= kWave) mine = sort_bucket(mine, m, lane);
         for (int k = 0; k < m; ++k) {
             const int64_t t = __shfl(mine, k, kWave);
             const T* src = dy + t * ld_dy;
@@ -147,24 +184,95 @@ __global__ __launch_bounds__(kBlock) void emb_bwd_reduce(const T* __restrict__ d
     }
 }
 
+// The same for bf16 rows that can be moved 16 bytes at a time: a lane owns the
+// eight consecutive columns chunk * kChunk + 8 lane .. + 7, so one load
+// instruction of the wavefront covers a chunk, and a wavefront takes CPW
+// chunks of its row so that the loads of a token overlap and the walk through
+// start and bucket is paid once for all of them.
+template <int CPW>
+__global__ __launch_bounds__(kBlock) void emb_bwd_reduce_bf16x8(const uint16_t* __restrict__ dy, int64_t dim, int64_t ld_dy,
+                                                                const int32_t* __restrict__ start, int32_t* __restrict__ bucket,
+                                                                int64_t rows, int groups, uint16_t* __restrict__ dw, int64_t ld_dw) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t w = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + threadIdx.x / kWave;
+    const int64_t row = w / groups;
+    const int group = static_cast<int>(w - row * groups);
+    if (row >= rows) return;
+    const int32_t b0 = row ? start[row - 1] : 0, n = start[row] - b0;   // the fill pass moved start[r] to the end of bucket r
+    float acc[CPW][8];
+#pragma unroll
+    for (int j = 0; j < CPW; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
+    const int64_t c0 = static_cast<int64_t>(group) * CPW * kChunk + lane * 8;   // dim is a multiple of 8 on this path
+    for (int32_t base = 0; base < n; base += kWave) {
+        const int32_t m = n - base < kWave ? n - base : kWave;
+        int32_t mine = lane < m ? bucket[b0 + base + lane] : 0x7FFFFFFF;
+        if (n <= kWave) mine = sort_bucket(mine, m, lane);
+        for (int k = 0; k < m; ++k) {
+            const int64_t t = __shfl(mine, k, kWave);
+            const uint16_t* src = dy + t * ld_dy + c0;
+            uint4 q[CPW];
+#pragma unroll
+            for (int j = 0; j < CPW; ++j) q[j] = c0 + j * kChunk < dim ? *reinterpret_cast<const uint4*>(src + j * kChunk) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < CPW; ++j) {
+                const uint32_t w4[4] = {q[j].x, q[j].y, q[j].z, q[j].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    acc[j][2 * e] += __uint_as_float(w4[e] << 16);
+                    acc[j][2 * e + 1] += __uint_as_float(w4[e] & 0xFFFF0000u);
+                }
+            }
+        }
+    }
+    uint16_t* dst = dw + row * ld_dw + c0;
+#pragma unroll
+    for (int j = 0; j < CPW; ++j) {
+        if (c0 + j * kChunk >= dim) continue;
+        uint16_t o[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) store_from_f32(&o[e], acc[j][e]);
+        uint4 q;
+        q.x = o[0] | (static_cast<uint32_t>(o[1]) << 16);
+        q.y = o[2] | (static_cast<uint32_t>(o[3]) << 16);
+        q.z = o[4] | (static_cast<uint32_t>(o[5]) << 16);
+        q.w = o[6] | (static_cast<uint32_t>(o[7]) << 16);
+        *reinterpret_cast<uint4*>(dst + j * kChunk) = q;
+    }
+}
+
+template <int CPW>
+void launch_reduce_x8(const void* dy, int64_t dim, int64_t ld_dy, const int32_t* start, int32_t* bucket, int64_t rows, int chunks,
+                      void* dw, int64_t ld_dw, hipStream_t s) {
+    const int groups = (chunks + CPW - 1) / CPW;
+    const int64_t waves = rows * groups;
+    hipLaunchKernelGGL((emb_bwd_reduce_bf16x8<CPW>), dim3(static_cast<uint32_t>((waves + kWavesPerBlock - 1) / kWavesPerBlock)),
+                       dim3(kBlock), 0, s, static_cast<const uint16_t*>(dy), dim, ld_dy, start, bucket, rows, groups,
+                       static_cast<uint16_t*>(dw), ld_dw);
+}
+
 template <typename IdT>
 int run(const void* dy, int dtype, int64_t dim, int64_t ld_dy, const IdT* ids, int64_t n_ids, int64_t lo, int64_t hi,
         int64_t padding_idx, void* dw, int64_t ld_dw, int32_t* ws, hipStream_t s) {
     const int64_t rows = hi - lo;
-    int32_t* count = ws;                 // [rows]   -> reused as cursor after the scan
-    int32_t* start = ws + rows;          // [rows + 1]
+    int32_t* count = ws;                 // [rows]
+    int32_t* start = ws + rows;          // [rows + 1]: begin of each bucket, advanced to its end by the fill pass
     int32_t* bucket = start + rows + 1;  // [n_ids]
     auto grid = [](int64_t n) { return dim3(static_cast<uint32_t>((n + kBlock - 1) / kBlock)); };
     hipLaunchKernelGGL(emb_bwd_clear, grid(rows), dim3(kBlock), 0, s, count, rows);
     if (n_ids > 0) hipLaunchKernelGGL((emb_bwd_count<IdT>), grid(n_ids), dim3(kBlock), 0, s, ids, n_ids, lo, hi, padding_idx, count);
     hipLaunchKernelGGL(emb_bwd_scan, dim3(1), dim3(kScanBlock), 0, s, count, rows, start);
-    hipLaunchKernelGGL(emb_bwd_clear, grid(rows), dim3(kBlock), 0, s, count, rows);
     if (n_ids > 0)
-        hipLaunchKernelGGL((emb_bwd_fill<IdT>), grid(n_ids), dim3(kBlock), 0, s, ids, n_ids, lo, hi, padding_idx, start, count, bucket);
+        hipLaunchKernelGGL((emb_bwd_fill<IdT>), grid(n_ids), dim3(kBlock), 0, s, ids, n_ids, lo, hi, padding_idx, start, bucket);
     const int chunks = static_cast<int>((dim + kChunk - 1) / kChunk);
     const int64_t waves = rows * chunks;
     const dim3 rgrid(static_cast<uint32_t>((waves + kWavesPerBlock - 1) / kWavesPerBlock));
-    if (dtype == DDL_DT_BF16)
+    const bool vec = dtype == DDL_DT_BF16 && dim % 8 == 0 && ld_dy % 8 == 0 && ld_dw % 8 == 0 && aligned_to(dy, 16) && aligned_to(dw, 16);
+    if (vec) {
+        if (chunks >= 2) launch_reduce_x8<2>(dy, dim, ld_dy, start, bucket, rows, chunks, dw, ld_dw, s);
+        else launch_reduce_x8<1>(dy, dim, ld_dy, start, bucket, rows, chunks, dw, ld_dw, s);
+    } else if (dtype == DDL_DT_BF16)
         hipLaunchKernelGGL((emb_bwd_reduce<uint16_t>), rgrid, dim3(kBlock), 0, s, static_cast<const uint16_t*>(dy), dim, ld_dy,
                            start, bucket, rows, chunks, static_cast<uint16_t*>(dw), ld_dw);
     else

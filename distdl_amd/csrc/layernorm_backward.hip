@@ -145,17 +145,46 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_params_partial(const float* __r
     }
 }
 
+// Workgroup per 64-column strip: lane group g = t / 64 adds the splits g, g+4,
+// ... of column t % 64 (independent loads, eight in flight), LDS folds the four
+// groups.
 __global__ __launch_bounds__(kBlock) void ln_bwd_params_final(const float* __restrict__ partial, int64_t cols, int splits,
                                                               float* __restrict__ dgamma, float* __restrict__ dbeta) {
-    const int64_t c = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    if (c >= cols) return;
+    __shared__ float fold[2][kWavesPerBlock][kStrip];
+    const int g = threadIdx.x / kStrip, t = threadIdx.x % kStrip;
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * kStrip + t;
     float a = 0.f, b = 0.f;
-    for (int k = 0; k < splits; ++k) {
-        a += partial[(static_cast<int64_t>(k) * 2) * cols + c];
-        b += partial[(static_cast<int64_t>(k) * 2 + 1) * cols + c];
+    if (c < cols) {
+        int k = g;
+        for (; k + 7 * kWavesPerBlock < splits; k += 8 * kWavesPerBlock) {
+            float va[8], vb[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                va[u] = partial[(static_cast<int64_t>(k + u * kWavesPerBlock) * 2) * cols + c];
+                vb[u] = partial[(static_cast<int64_t>(k + u * kWavesPerBlock) * 2 + 1) * cols + c];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                a += va[u];
+                b += vb[u];
+            }
+        }
+        for (; k < splits; k += kWavesPerBlock) {
+            a += partial[(static_cast<int64_t>(k) * 2) * cols + c];
+            b += partial[(static_cast<int64_t>(k) * 2 + 1) * cols + c];
+        }
     }
-    if (dgamma) dgamma[c] = a;
-    if (dbeta) dbeta[c] = b;
+    fold[0][g][t] = a;
+    fold[1][g][t] = b;
+    __syncthreads();
+    if (threadIdx.x < 2 * kStrip && c < cols) {
+        const int which = threadIdx.x / kStrip;
+        float s = 0.f;
+#pragma unroll
+        for (int k = 0; k < kWavesPerBlock; ++k) s += fold[which][k][t];
+        float* out = which == 0 ? dgamma : dbeta;
+        if (out) out[c] = s;
+    }
 }
 
 bool vectorizable(int64_t cols, std::initializer_list<int64_t> lds, std::initializer_list<const void*> ptrs) {
@@ -239,7 +268,7 @@ extern "C" int ddl_ln_bwd_params_f32(const float* dy, const float* x, int64_t ro
     hipLaunchKernelGGL(ln_bwd_params_partial, dim3(static_cast<uint32_t>(strips * splits)), dim3(kBlock), 0, s, dy, x, rows, cols,
                        ld_dy, ld_x, mean, rstd, rows_per_split, workspace, static_cast<int>(strips));
     if (int rc = check_launch("ln_bwd_params_partial")) return rc;
-    hipLaunchKernelGGL(ln_bwd_params_final, dim3(static_cast<uint32_t>((cols + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, workspace,
-                       cols, static_cast<int>(splits), dgamma, dbeta);
+    hipLaunchKernelGGL(ln_bwd_params_final, dim3(static_cast<uint32_t>(strips)), dim3(kBlock), 0, s, workspace, cols,
+                       static_cast<int>(splits), dgamma, dbeta);
     return check_launch("ln_bwd_params_final");
 }
