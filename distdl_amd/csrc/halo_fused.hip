@@ -45,6 +45,40 @@ struct Slab {
     int64_t stride[HD - 1];  // element strides of dimensions 0..L-1 (dimension L has stride 1)
 };
 
+// Arguments of halo_flat_kernel are laid out for few, wide scalar loads.
+struct FlatTop {
+    const char* x;           // shard
+    char* xpad;
+    const char* gm[2];       // ghost slabs of M (nullptr when absent)
+    const char* gl;          // ghost slabs of L
+    const char* gr;
+    int64_t xstrM;           // shard stride of M
+    int64_t x_off0;          // -(padl[M] * xstrM + padl[L]): shard offset of padded (h, w) = (0, 0) in shard plane 0
+    uint32_t total;          // elements of the padded tensor (< 2^31)
+    uint32_t nstages;        // pieces of kStage consecutive elements
+    uint32_t W, H;           // ps[L], ps[M]
+    uint32_t fdW_mul, fdW_shr, fdH_mul, fdH_shr;
+    uint32_t glo, ghi;       // bulk range of L
+    uint32_t hlo, hhi;       // bulk range of M
+    uint32_t padL, xhiL;     // shard columns [padL, xhiL)
+    uint32_t padM, xsM;
+    uint32_t m_l1, m_r0;     // rows [hlo, m_l1) and [m_r0, hhi) feed the bulk slabs of M (empty without a slab)
+    uint32_t n_ghost;        // ghost columns of a row, recvl[L] + recvr[L]
+    uint32_t fdg_mul, fdg_shr;
+    uint32_t any_outer;      // some dimension below M has a bulk slab
+    uint32_t n_bl, n_br;     // columns of the left / right bulk strip of L (0 without a slab)
+    uint32_t sl, sr;         // sendl[L], sendr[L]
+    uint32_t fds_mul, fds_shr;   // division by n_bl + n_br
+};
+struct FlatDim {
+    uint32_t ps, fd_mul, fd_shr;
+    uint32_t lo, hi;         // bulk range
+    uint32_t padl, xs;
+    uint32_t strip_l1, strip_r0;   // coordinates [lo, strip_l1) and [strip_r0, hi) feed this dimension's bulk slabs
+    uint32_t unused;
+    int64_t xstride;
+};
+
 struct HaloArgs {
     const char* x;
     char* xpad;
@@ -60,6 +94,8 @@ struct HaloArgs {
     uint32_t rows_per_block;
     uint32_t max_vecs;       // vectors of the longest run of any row
     uint32_t max_edge;       // single-element tasks per row, upper bound
+    FlatTop top;             // halo_flat_kernel: what every wavefront reads first, kept together
+    FlatDim outer[HD - 2];   // halo_flat_kernel: the dimensions below M
 };
 static_assert(sizeof(HaloArgs) <= 3900, "halo arguments must fit the kernel-argument segment");
 
@@ -445,6 +481,321 @@ __global__ __launch_bounds__(kBlock) void halo_pad_kernel(const HaloArgs args_by
     }
 }
 
+// ---------------------------------------------------------------------------
+// 4-byte elements, whole-line stores.  Rows of the padded tensor are seldom
+// whole 128-byte lines (130 floats in the convolution case), and writing them
+// row by row costs a quarter of the store rate.  The padded tensor is
+// contiguous, though, so it is also a plain run of elements: a wavefront takes
+// kStage consecutive elements (4 KiB, aligned in memory), assembles them in its
+// own LDS area and writes the area out with aligned 16-byte vectors, 1 KiB per
+// instruction.
+//
+// Assembly: at most 64 padded rows meet a piece, so lane k classifies row k --
+// all rows at once, in vector arithmetic: plane and row number, the plane's
+// coordinates, whether it is a shard row (then where it starts in the shard)
+// or all zeros, whether a bulk slab below L contains it.  The few rows that come
+// from a ghost slab are then settled one by one in scalar code.  The result is
+// one source pointer per row, held by lane k (a row is either a shard row, whose
+// run is the shard's columns, or a ghost row, whose run is the bulk range of L:
+// bit 0 of the pointer says which).  The area is cleared and filled by 16
+// global -> LDS loads of 4 bytes per lane: lane l of load m owns element
+// 64 m + l of the piece, takes its row's pointer from lane k with a cross-lane
+// read and fetches from there (or stays idle: zeros), so consecutive lanes
+// fetch consecutive addresses.
+// The ghost columns of L (a few elements per row) are fetched one element per
+// lane for all rows of the piece at once.  The bulk slabs are served from the
+// assembled area.  Wavefronts do not share data: no barriers.
+constexpr uint32_t kStage = 1024;            // elements per wavefront
+constexpr uint32_t kFlatMinPitch = 32;       // shortest padded row: keeps a piece within 64 rows
+constexpr uint32_t kArea = kStage;
+
+typedef const __attribute__((address_space(1))) void* global_ptr;
+typedef __attribute__((address_space(3))) void* lds_ptr;
+
+// Offset of row h of plane c inside a slab whose dimensions 0..M are the tensor's.
+template <int M>
+__device__ inline int64_t slab_row_offset(SlabPtr b, const uint32_t (&c)[HD], uint32_t h) {
+    int64_t off = b->base + static_cast<int64_t>(h) * b->stride[M];
+#pragma unroll
+    for (int j = 0; j < M; ++j) off += static_cast<int64_t>(c[j]) * b->stride[j];
+    return off;
+}
+
+template <int ND>
+__global__ __launch_bounds__(kBlock) void halo_flat_kernel(const HaloArgs args_by_value) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    ArgsPtr a = (ArgsPtr)__builtin_amdgcn_kernarg_segment_ptr();
+#else
+    ArgsPtr a = &args_by_value;
+#endif
+    typedef uint32_t T;
+    constexpr int L = ND - 1, M = ND - 2;
+    __shared__ __attribute__((aligned(16))) T stage_mem[kWavesPerBlock * kArea];
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const uint32_t stage = blockIdx.x * kWavesPerBlock + wave;
+    if (stage >= a->top.nstages) return;
+    T* const area = stage_mem + wave * kArea;                    // element g0 of the padded tensor
+    const uint32_t g0 = stage * kStage;
+    const uint32_t total = a->top.total;
+    const uint32_t n_el = total - g0 < kStage ? total - g0 : kStage;
+
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4*>(area + j * 256 + lane * 4) = make_uint4(0, 0, 0, 0);
+
+    const uint32_t W = a->top.W, H = a->top.H;
+    const uint32_t glo = a->top.glo, ghi = a->top.ghi, hlo = a->top.hlo, hhi = a->top.hhi;
+    const uint32_t padL = a->top.padL, xhiL = a->top.xhiL, padM = a->top.padM, xsM = a->top.xsM;
+    const uint32_t m_l1 = a->top.m_l1, m_r0 = a->top.m_r0;
+    const int64_t xstrM = a->top.xstrM;
+    const T* const xbase = reinterpret_cast<const T*>(a->top.x) + a->top.x_off0;
+    const uint32_t any_outer = a->top.any_outer;
+
+    // First row of the piece: its global row number and the (non-positive)
+    // position of its column 0 relative to the piece.
+    const uint32_t row0 = __umulhi(g0, a->top.fdW_mul) >> a->top.fdW_shr;
+    const int rowq0 = static_cast<int>(row0 * W) - static_cast<int>(g0);
+    const uint32_t nrows = (n_el - rowq0 + W - 1) / W;           // rows that meet the piece, at most 64
+
+    // ---- lane k: row k of the piece ----
+    const uint32_t vrow = row0 + lane;
+    const uint32_t vplane = H == 1 ? vrow : (__umulhi(vrow, a->top.fdH_mul) >> a->top.fdH_shr);
+    const uint32_t vh = vrow - vplane * H;
+    uint32_t v_inx = 1, v_ghost = 0, v_fwd = 0;
+    int64_t v_xoff = static_cast<int64_t>(vh) * xstrM;
+    {
+        uint32_t vc[HD] = {0, 0, 0, 0, 0, 0};
+        uint32_t r = vplane;
+#pragma unroll
+        for (int j = M - 1; j > 0; --j) {
+            const uint32_t n = a->outer[j].ps;
+            const uint32_t q = n == 1 ? r : (__umulhi(r, a->outer[j].fd_mul) >> a->outer[j].fd_shr);
+            vc[j] = r - q * n;
+            r = q;
+        }
+        if (M > 0) vc[0] = r;
+        uint32_t inner = 1;
+#pragma unroll
+        for (int i = M - 1; i >= 0; --i) {                        // a slab of dimension i holds the bulk range of the dimensions above i
+            const uint32_t ci = vc[i], lo = a->outer[i].lo, hi = a->outer[i].hi;
+            const uint32_t inb = (ci >= lo) & (ci < hi);
+            const uint32_t strip = ((ci >= lo) & (ci < a->outer[i].strip_l1)) | ((ci >= a->outer[i].strip_r0) & (ci < hi));
+            v_fwd |= inner & strip;
+            inner &= inb;
+            v_ghost |= inb ^ 1u;
+            const uint32_t xc = ci - a->outer[i].padl;           // wraps when left of the shard
+            v_inx &= xc < a->outer[i].xs ? 1u : 0u;
+            v_xoff += static_cast<int64_t>(xc) * a->outer[i].xstride;
+        }
+    }
+    const bool v_valid = lane < nrows;
+    const bool v_hbulk = vh >= hlo && vh < hhi;
+    // rows of a ghost plane or a ghost strip of M may come from a slab: settled below, one by one
+    const bool v_complex = v_valid && (v_ghost != 0 || !v_hbulk);
+    const bool v_shard = v_inx != 0 && vh - padM < xsM;
+    const bool v_forward = v_valid && ((vh >= hlo && vh < m_l1) || (vh >= m_r0 && vh < hhi) || (any_outer != 0 && v_fwd != 0 && v_hbulk));
+    // Element w of the row is vp[w] for w in its run: the shard's columns, or
+    // the bulk range of L when bit 0 is set (a row from a ghost slab).
+    uint64_t vp = v_shard ? reinterpret_cast<uint64_t>(xbase + v_xoff) : 0;
+
+    // ---- what a plane decides (scalar; used for the few rows handled one by one) ----
+    uint32_t c[HD] = {0, 0, 0, 0, 0, 0};
+    const T* gplane = nullptr;                                    // ghost slab of an outer dimension: row h at gplane + h * gstr
+    int64_t gstr = 0;
+    auto setup_plane = [&](uint32_t plane) {
+        uint32_t r = plane;
+#pragma unroll
+        for (int j = M - 1; j > 0; --j) {
+            const uint32_t n = a->outer[j].ps;
+            const uint32_t q = n == 1 ? r : (__umulhi(r, a->outer[j].fd_mul) >> a->outer[j].fd_shr);
+            c[j] = r - q * n;
+            r = q;
+        }
+        if (M > 0) c[0] = r;
+        int gh = -1, gside = 0;
+#pragma unroll
+        for (int j = 0; j < M; ++j) {
+            const uint32_t left = c[j] < a->outer[j].lo, right = c[j] >= a->outer[j].hi;
+            gh = (left | right) ? j : gh;
+            gside = right ? 1 : (left ? 0 : gside);
+        }
+        gplane = nullptr;
+        if (gh >= 0 && a->ghost[gh][gside].ptr != nullptr) {
+            SlabPtr g = &a->ghost[gh][gside];
+            gplane = reinterpret_cast<const T*>(g->ptr) + slab_row_offset<M>(g, c, 0);
+            gstr = g->stride[M];
+        }
+    };
+    auto plane_and_row = [&](uint32_t k, uint32_t& plane, uint32_t& h) {
+        const uint32_t row = row0 + k;
+        plane = H == 1 ? row : (__umulhi(row, a->top.fdH_mul) >> a->top.fdH_shr);
+        h = row - plane * H;
+    };
+
+    // ---- rows that may come from a ghost slab (scalar, few) ----
+    {
+        uint64_t todo = __ballot(v_complex);
+        uint32_t decoded = ~0u;
+        const T* const gm0 = reinterpret_cast<const T*>(a->top.gm[0]);
+        const T* const gm1 = reinterpret_cast<const T*>(a->top.gm[1]);
+        while (todo != 0) {
+            const uint32_t k = static_cast<uint32_t>(__builtin_ctzll(todo));
+            todo &= todo - 1;
+            uint32_t plane, h;
+            plane_and_row(k, plane, h);
+            if (decoded != plane) {
+                setup_plane(plane);
+                decoded = plane;
+            }
+            const T* p = nullptr;                                 // a ghost row spans the bulk range of L; without a slab it is zeros
+            if (gplane != nullptr) p = gplane + static_cast<int64_t>(h) * gstr;
+            if (h < hlo && gm0 != nullptr) p = gm0 + slab_row_offset<M>(&a->ghost[M][0], c, h);
+            if (h >= hhi && gm1 != nullptr) p = gm1 + slab_row_offset<M>(&a->ghost[M][1], c, h);
+            if (lane == k) vp = p != nullptr ? (reinterpret_cast<uint64_t>(p) | 1u) : 0;
+        }
+    }
+    // The zeros must be in place before a global -> LDS load can land (those do
+    // not queue behind LDS instructions).
+    __builtin_amdgcn_s_waitcnt(0xC07F);                          // lgkmcnt(0)
+
+    // ---- the runs: lane l of load m fetches element 64 m + l of the piece ----
+    {
+        const uint32_t t0 = lane - static_cast<uint32_t>(rowq0);  // position counted from column 0 of the first row
+        uint32_t k = __umulhi(t0, a->top.fdW_mul) >> a->top.fdW_shr;
+        uint32_t w = t0 - k * W;
+#pragma unroll 4
+        for (uint32_t m = 0; m < kStage / kWave; ++m) {
+            const int from = static_cast<int>((k < kWave ? k : kWave - 1) * 4);
+            const uint32_t plo = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(static_cast<uint32_t>(vp))));
+            const uint32_t phi = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(from, static_cast<int>(static_cast<uint32_t>(vp >> 32))));
+            const bool ghost_row = (plo & 1u) != 0;
+            const uint32_t lo = ghost_row ? glo : padL, hi = ghost_row ? ghi : xhiL;
+            const T* p = reinterpret_cast<const T*>(static_cast<uint64_t>(plo & ~1u) | (static_cast<uint64_t>(phi) << 32));
+            if (m * kWave + lane < n_el && p != nullptr && w >= lo && w < hi)
+                __builtin_amdgcn_global_load_lds((global_ptr)(p + w), (lds_ptr)(area + m * kWave), 4, 0, 0);
+            w += kWave;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {                         // rows hold at least 32 elements
+                const bool wrap = w >= W;
+                w = wrap ? w - W : w;
+                k = wrap ? k + 1 : k;
+            }
+        }
+    }
+
+    // ---- ghost columns of L: one element per lane, all rows of the piece ----
+    const uint32_t n_ghost = a->top.n_ghost;
+    if (n_ghost != 0) {
+        const T* gl = reinterpret_cast<const T*>(a->top.gl);
+        const T* gr = reinterpret_cast<const T*>(a->top.gr);
+        const uint32_t rl = glo, rr = W - ghi;
+        for (uint32_t e0 = 0; e0 < nrows * n_ghost; e0 += kWave) {
+            const uint32_t e = e0 + lane;
+            const uint32_t k = n_ghost == 1 ? e : (__umulhi(e, a->top.fdg_mul) >> a->top.fdg_shr);
+            const uint32_t i = e - k * n_ghost;
+            const uint32_t w = i < rl ? i : ghi + (i - rl);
+            const uint32_t q = static_cast<uint32_t>(rowq0 + static_cast<int>(k * W + w));
+            const bool on = e < nrows * n_ghost && q < n_el;
+            const int64_t row = static_cast<int64_t>(row0) + k;
+            const T* p = i < rl ? gl + row * rl + w : gr + row * rr + (w - ghi);
+            T v = 0;
+            if (on) v = *p;
+            if (on) area[q] = v;
+        }
+    }
+
+    __builtin_amdgcn_s_waitcnt(0x0070);                          // every load has landed, every LDS write is done
+    asm volatile("" ::: "memory");
+
+    // ---- the piece leaves in whole lines ----
+    {
+        T* const out = reinterpret_cast<T*>(a->top.xpad) + g0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t o = j * 256 + lane * 4;
+            const uint4 v = *reinterpret_cast<const uint4*>(area + o);
+            if (o + 4 <= n_el) {
+                *reinterpret_cast<uint4*>(out + o) = v;
+            } else {
+                const T ev[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    if (o + t < n_el) out[o + t] = ev[t];
+            }
+        }
+    }
+
+    // ---- bulk strips of L: one element per lane ----
+    const uint32_t n_bl = a->top.n_bl, n_br = a->top.n_br, n_strip = n_bl + n_br;
+    if (n_strip != 0) {
+        T* bl = reinterpret_cast<T*>(a->bulk[L][0].ptr);
+        T* br = reinterpret_cast<T*>(a->bulk[L][1].ptr);
+        const uint32_t sl = a->top.sl, sr = a->top.sr;
+        for (uint32_t e0 = 0; e0 < nrows * n_strip; e0 += kWave) {
+            const uint32_t e = e0 + lane;
+            const uint32_t k = n_strip == 1 ? e : (__umulhi(e, a->top.fds_mul) >> a->top.fds_shr);
+            const uint32_t i = e - k * n_strip;
+            const uint32_t w = i < n_bl ? glo + i : ghi - sr + (i - n_bl);
+            const uint32_t q = static_cast<uint32_t>(rowq0 + static_cast<int>(k * W + w));
+            const int64_t row = static_cast<int64_t>(row0) + k;
+            if (e < nrows * n_strip && q < n_el) {
+                const T v = area[q];
+                if (i < n_bl)
+                    bl[row * sl + (w - glo)] = v;
+                else
+                    br[row * sr + (w - (ghi - sr))] = v;
+            }
+        }
+    }
+
+    // ---- bulk slabs below L: the bulk range of L of the rows they contain (scalar, few) ----
+    {
+        uint64_t todo = __ballot(v_forward);
+        uint32_t decoded = ~0u;
+        while (todo != 0) {
+            const uint32_t k = static_cast<uint32_t>(__builtin_ctzll(todo));
+            todo &= todo - 1;
+            uint32_t plane, h;
+            plane_and_row(k, plane, h);
+            if (decoded != plane) {
+                setup_plane(plane);
+                decoded = plane;
+            }
+            const int rowq = rowq0 + static_cast<int>(k * W);
+            auto copy_row = [&](SlabPtr b) {
+                T* const dst = reinterpret_cast<T*>(b->ptr) + slab_row_offset<M>(b, c, h);
+                // the part of [glo, ghi) inside the piece, in 64-element steps counted from glo
+                const int before = -rowq - static_cast<int>(glo);
+                uint32_t w0 = glo + (before > 0 ? (static_cast<uint32_t>(before) >> 6) << 6 : 0u);
+                for (; w0 < ghi && rowq + static_cast<int>(w0) < static_cast<int>(n_el); w0 += kWave) {
+                    const uint32_t w = w0 + lane;
+                    const uint32_t q = static_cast<uint32_t>(rowq + static_cast<int>(w));
+                    if (w < ghi && q < n_el) dst[w] = area[q];
+                }
+            };
+            // dimension M: the row's own strips; outer dimensions are unrestricted
+            if (h >= hlo && h < m_l1) copy_row(&a->bulk[M][0]);
+            if (h >= m_r0 && h < hhi) copy_row(&a->bulk[M][1]);
+            // outer dimension i: decided by the plane, and the row must be in the bulk range of M
+            if (any_outer != 0 && h >= hlo && h < hhi) {
+                bool inner_bulk = true;                           // outer dimensions above i inside their bulk range
+#pragma unroll
+                for (int i = M - 1; i >= 0; --i) {
+                    const uint32_t blo = a->outer[i].lo, bhi = a->outer[i].hi;
+                    if (inner_bulk) {
+                        if (c[i] >= blo && c[i] < a->outer[i].strip_l1) copy_row(&a->bulk[i][0]);
+                        if (c[i] >= a->outer[i].strip_r0 && c[i] < bhi) copy_row(&a->bulk[i][1]);
+                    }
+                    inner_bulk = inner_bulk && c[i] >= blo && c[i] < bhi;
+                }
+            }
+        }
+    }
+}
+
+// Rows at least this long (shard elements) take halo_flat_kernel.
+int g_flat_min_row = 32;
+
 template <typename T>
 int launch_halo(const HaloArgs& a, uint32_t lpr, hipStream_t s) {
     const uint32_t blocks = a.nplanes * a.row_chunks;
@@ -459,6 +810,12 @@ int launch_halo(const HaloArgs& a, uint32_t lpr, hipStream_t s) {
 
 }  // namespace
 }  // namespace ddl
+
+extern "C" int ddl_halo_set_flat_min_row(int64_t elements) {
+    if (elements < 1) return ddl::fail(DDL_E_ARG, "halo: row threshold %lld below 1", (long long)elements);
+    ddl::g_flat_min_row = elements > 0x7FFFFFFFll ? 0x7FFFFFFF : static_cast<int>(elements);
+    return 0;
+}
 
 extern "C" int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x_shape, int ndim, int elem_size,
                                      const int64_t* pad, const int64_t* recv, const int64_t* send,
@@ -589,6 +946,70 @@ extern "C" int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x
     if (nplanes * static_cast<int64_t>(a.row_chunks) >= (1ll << 31)) return fail(DDL_E_UNSUPP, "halo: too many workgroups");
     a.nplanes = static_cast<uint32_t>(nplanes);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (elem_size == 4 && total < (1ll << 31) && xs[L] >= g_flat_min_row && ps[L] >= kFlatMinPitch && aligned_to(xpad, 16)) {
+        const int64_t nstages = (total + kStage - 1) / kStage;
+        FlatTop& t = a.top;
+        t.x = a.x;
+        t.xpad = a.xpad;
+        t.gm[0] = a.ghost[M][0].ptr;
+        t.gm[1] = a.ghost[M][1].ptr;
+        t.gl = a.ghost[L][0].ptr;
+        t.gr = a.ghost[L][1].ptr;
+        t.xstrM = a.xstride[M];
+        t.x_off0 = -(pl[M] * a.xstride[M] + pl[L]);
+        t.total = static_cast<uint32_t>(total);
+        t.nstages = static_cast<uint32_t>(nstages);
+        t.W = a.ps[L];
+        t.H = a.ps[M];
+        t.fdW_mul = a.fd[L].mul;
+        t.fdW_shr = a.fd[L].shr;
+        t.fdH_mul = a.fd[M].mul;
+        t.fdH_shr = a.fd[M].shr;
+        t.glo = a.recvl[L];
+        t.ghi = a.ps[L] - a.recvr[L];
+        t.hlo = a.recvl[M];
+        t.hhi = a.ps[M] - a.recvr[M];
+        t.padL = a.padl[L];
+        t.xhiL = a.padl[L] + a.xs[L];
+        t.padM = a.padl[M];
+        t.xsM = a.xs[M];
+        t.m_l1 = a.bulk[M][0].ptr ? t.hlo + a.sendl[M] : t.hlo;
+        t.m_r0 = a.bulk[M][1].ptr ? t.hhi - a.sendr[M] : t.hhi;
+        t.n_ghost = a.recvl[L] + a.recvr[L];
+        t.n_bl = a.bulk[L][0].ptr ? a.sendl[L] : 0u;
+        t.n_br = a.bulk[L][1].ptr ? a.sendr[L] : 0u;
+        t.sl = a.sendl[L];
+        t.sr = a.sendr[L];
+        const FastDiv fdg = make_fastdiv(t.n_ghost > 0 ? t.n_ghost : 1), fds = make_fastdiv(t.n_bl + t.n_br > 0 ? t.n_bl + t.n_br : 1);
+        t.fdg_mul = fdg.mul;
+        t.fdg_shr = fdg.shr;
+        t.fds_mul = fds.mul;
+        t.fds_shr = fds.shr;
+        t.any_outer = 0;
+        for (int j = 0; j < M; ++j) {
+            FlatDim& o = a.outer[j];
+            o.ps = a.ps[j];
+            o.fd_mul = a.fd[j].mul;
+            o.fd_shr = a.fd[j].shr;
+            o.lo = a.recvl[j];
+            o.hi = a.ps[j] - a.recvr[j];
+            o.padl = a.padl[j];
+            o.xs = a.xs[j];
+            o.strip_l1 = a.bulk[j][0].ptr ? o.lo + a.sendl[j] : o.lo;
+            o.strip_r0 = a.bulk[j][1].ptr ? o.hi - a.sendr[j] : o.hi;
+            o.xstride = a.xstride[j];
+            if (a.bulk[j][0].ptr || a.bulk[j][1].ptr) t.any_outer = 1;
+        }
+        const dim3 grid(static_cast<uint32_t>((nstages + kWavesPerBlock - 1) / kWavesPerBlock));
+        switch (nd) {
+            case 2: hipLaunchKernelGGL(halo_flat_kernel<2>, grid, dim3(kBlock), 0, s, a); break;
+            case 3: hipLaunchKernelGGL(halo_flat_kernel<3>, grid, dim3(kBlock), 0, s, a); break;
+            case 4: hipLaunchKernelGGL(halo_flat_kernel<4>, grid, dim3(kBlock), 0, s, a); break;
+            case 5: hipLaunchKernelGGL(halo_flat_kernel<5>, grid, dim3(kBlock), 0, s, a); break;
+            default: hipLaunchKernelGGL(halo_flat_kernel<6>, grid, dim3(kBlock), 0, s, a); break;
+        }
+        return check_launch("halo_flat_kernel");
+    }
     switch (elem_size) {
         case 1: return launch_halo<uint8_t>(a, lpr, s);
         case 2: return launch_halo<uint16_t>(a, lpr, s);

@@ -230,6 +230,13 @@ class HaloPadPlan:
         return out
 
 
+def halo_set_flat_min_row(elements):
+    """Shard rows of at least ``elements`` 4-byte elements take the whole-line
+    kernel of ``ddl_halo_pad_exchange`` (library default 32); shorter rows are
+    written row by row.  Results are identical either way."""
+    _lib.check(_lib.load().ddl_halo_set_flat_min_row(int(elements)), "ddl_halo_set_flat_min_row")
+
+
 def ln_partial_stats(x2d, out=None):
     """{mean, M2} per row of a [rows, cols] fp32 view (last stride 1)."""
     _require_gpu(x2d)

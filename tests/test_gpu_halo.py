@@ -85,6 +85,17 @@ def test_halo_exchange_layer_matches_oracle(P, gshape, kernel):
 
 # ------------------------------------------------------------ fused kernel --
 
+@pytest.fixture(params=["rows", "lines", "default"])
+def halo_path(request, ops):
+    """The fused kernel has two ways of writing fp32 tensors (row by row, or in
+    whole 128-byte lines through LDS); every fused case runs on both and on the
+    library's own choice."""
+    if request.param != "default":
+        ops.halo_set_flat_min_row(1 << 40 if request.param == "rows" else 1)
+    yield request.param
+    ops.halo_set_flat_min_row(32)
+
+
 def _fused_case(ops, x_shape, pad, recv, send, dtype, seed):
     gen = torch.Generator().manual_seed(seed)
     x = torch.randn(x_shape, generator=gen).to(dtype)
@@ -116,19 +127,19 @@ def _fused_case(ops, x_shape, pad, recv, send, dtype, seed):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16])
-def test_fused_halo_interior_rank_3d(ops, dtype):
+def test_fused_halo_interior_rank_3d(ops, dtype, halo_path):
     # every side has a ghost and a bulk strip, widths differ per side
     _fused_case(ops, (2, 3, 9, 10, 70), [[0, 0], [0, 0], [1, 2], [2, 1], [1, 3]],
                 [[0, 0], [0, 0], [1, 2], [2, 1], [1, 3]], [[0, 0], [0, 0], [2, 1], [1, 2], [3, 1]], dtype, 51)
 
 
-def test_fused_halo_corner_rank_with_explicit_padding(ops):
+def test_fused_halo_corner_rank_with_explicit_padding(ops, halo_path):
     # rank 0 of a 2x2x2 split, kernel 3 / padding 1: left sides are zero padding, right sides ghosts
     _fused_case(ops, (1, 4, 16, 16, 16), [[0, 0], [0, 0], [1, 1], [1, 1], [1, 1]],
                 [[0, 0], [0, 0], [0, 1], [0, 1], [0, 1]], [[0, 0], [0, 0], [0, 1], [0, 1], [0, 1]], torch.float32, 52)
 
 
-def test_fused_halo_long_rows_and_other_ranks(ops):
+def test_fused_halo_long_rows_and_other_ranks(ops, halo_path):
     _fused_case(ops, (3, 5, 300), [[0, 0], [2, 2], [4, 4]], [[0, 0], [2, 2], [4, 0]], [[0, 0], [1, 2], [0, 3]],
                 torch.float32, 53)
     _fused_case(ops, (40,), [[3, 2]], [[3, 2]], [[2, 3]], torch.float32, 54)
@@ -137,7 +148,27 @@ def test_fused_halo_long_rows_and_other_ranks(ops):
                 torch.float32, 56)                                                                        # F.pad only
 
 
-def test_fused_halo_config5_rank0_bit_exact(ops):
+def test_fused_halo_wide_rows_geometries(ops, halo_path):
+    # rows longer than a 1024-element piece; pieces that begin and end inside a row
+    _fused_case(ops, (2, 3, 2500), [[0, 0], [1, 1], [2, 3]], [[0, 0], [1, 1], [2, 3]], [[0, 0], [1, 1], [3, 2]],
+                torch.float32, 57)
+    # padding wider than the ghosts on every side, missing neighbours on some sides
+    _fused_case(ops, (2, 7, 9, 100), [[0, 0], [3, 2], [2, 3], [4, 5]], [[0, 0], [1, 0], [0, 2], [2, 0]],
+                [[0, 0], [2, 0], [0, 1], [1, 0]], torch.float32, 58)
+    # four exchanged dimensions, output volume not a multiple of four elements
+    _fused_case(ops, (3, 5, 6, 33), [[1, 1], [1, 1], [1, 1], [1, 1]], [[1, 1], [1, 1], [1, 1], [1, 1]],
+                [[1, 1], [1, 1], [1, 1], [1, 1]], torch.float32, 59)
+    # 2-D and 1-D tensors with long rows, int32 payload of the same element size
+    _fused_case(ops, (5, 1030), [[2, 2], [1, 1]], [[2, 2], [1, 1]], [[2, 2], [1, 1]], torch.float32, 60)
+    _fused_case(ops, (4099,), [[3, 2]], [[3, 2]], [[2, 3]], torch.float32, 61)
+    # ghost strips without bulk strips and the reverse
+    _fused_case(ops, (2, 6, 40, 64), [[0, 0], [2, 2], [1, 1], [2, 2]], [[0, 0], [2, 2], [1, 1], [2, 2]],
+                [[0, 0], [0, 0], [0, 0], [0, 0]], torch.float32, 62)
+    _fused_case(ops, (2, 6, 40, 64), [[0, 0], [2, 2], [1, 1], [2, 2]], [[0, 0], [0, 0], [0, 0], [0, 0]],
+                [[0, 0], [2, 1], [1, 1], [1, 2]], torch.float32, 63)
+
+
+def test_fused_halo_config5_rank0_bit_exact(ops, halo_path):
     """[1,32,128,128,128] fp32 shard of a 2x2x2 split, kernel 3, padding 1."""
     g = [1, 32, 256, 256, 256]
     P = (1, 1, 2, 2, 2)
