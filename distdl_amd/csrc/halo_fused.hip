@@ -506,7 +506,7 @@ __global__ __launch_bounds__(kBlock) void halo_pad_kernel(const HaloArgs args_by
 // lane for all rows of the piece at once.  The bulk slabs are served from the
 // assembled area.  Wavefronts do not share data: no barriers.
 constexpr uint32_t kStage = 1024;            // elements per wavefront
-constexpr uint32_t kFlatMinPitch = 32;       // shortest padded row: keeps a piece within 64 rows
+constexpr uint32_t kFlatMinPitch = kStage / 32;   // shortest padded row: keeps a piece within 64 rows (and a load within 3)
 constexpr uint32_t kArea = kStage;
 
 typedef const __attribute__((address_space(1))) void* global_ptr;
@@ -541,7 +541,7 @@ __global__ __launch_bounds__(kBlock) void halo_flat_kernel(const HaloArgs args_b
     const uint32_t n_el = total - g0 < kStage ? total - g0 : kStage;
 
 #pragma unroll
-    for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4*>(area + j * 256 + lane * 4) = make_uint4(0, 0, 0, 0);
+    for (uint32_t j = 0; j < kStage / 256; ++j) *reinterpret_cast<uint4*>(area + j * 256 + lane * 4) = make_uint4(0, 0, 0, 0);
 
     const uint32_t W = a->top.W, H = a->top.H;
     const uint32_t glo = a->top.glo, ghi = a->top.ghi, hlo = a->top.hlo, hhi = a->top.hhi;
@@ -711,11 +711,14 @@ __global__ __launch_bounds__(kBlock) void halo_flat_kernel(const HaloArgs args_b
     {
         T* const out = reinterpret_cast<T*>(a->top.xpad) + g0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (uint32_t j = 0; j < kStage / 256; ++j) {
             const uint32_t o = j * 256 + lane * 4;
             const uint4 v = *reinterpret_cast<const uint4*>(area + o);
             if (o + 4 <= n_el) {
-                *reinterpret_cast<uint4*>(out + o) = v;
+                typedef typename VecType<T, 4>::type V;          // the padded tensor is not read again here: streaming store
+                V nv;
+                nv[0] = v.x, nv[1] = v.y, nv[2] = v.z, nv[3] = v.w;
+                __builtin_nontemporal_store(nv, reinterpret_cast<V*>(out + o));
             } else {
                 const T ev[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
