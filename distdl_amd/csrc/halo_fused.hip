@@ -858,6 +858,14 @@ extern "C" int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x
         ++nd;
     }
     if (nd > HD) return fail(DDL_E_UNSUPP, "halo: %d dimensions left after folding, at most %d supported", nd, HD);
+    // 8-byte elements are moved as pairs of 4-byte ones: the same tensor and the
+    // same slabs with every extent of the last dimension doubled.
+    int es = elem_size;
+    if (elem_size == 8 && aligned_to(xpad, 16)) {
+        const int l = nd - 1;
+        xs[l] *= 2; pl[l] *= 2; pr[l] *= 2; rl[l] *= 2; rr[l] *= 2; sl[l] *= 2; sr[l] *= 2;
+        es = 4;
+    }
 
     HaloArgs a{};
     a.nd = nd;
@@ -929,7 +937,7 @@ extern "C" int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x
     // Work split: LPR lanes per row (a power of two covering the longest run in
     // vectors, at most a wavefront); the rows of a plane are cut into about
     // 64-row chunks, one workgroup each.
-    const int epv = elem_size >= 4 ? 16 / elem_size : 1;
+    const int epv = es >= 4 ? 16 / es : 1;
     const int64_t bulk_l = ps[L] - rl[L] - rr[L];
     const int64_t longest = bulk_l > xs[L] ? bulk_l : xs[L];
     const int64_t shortest = bulk_l < xs[L] ? bulk_l : xs[L];
@@ -949,7 +957,7 @@ extern "C" int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x
     if (nplanes * static_cast<int64_t>(a.row_chunks) >= (1ll << 31)) return fail(DDL_E_UNSUPP, "halo: too many workgroups");
     a.nplanes = static_cast<uint32_t>(nplanes);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (elem_size == 4 && total < (1ll << 31) && xs[L] >= g_flat_min_row && ps[L] >= kFlatMinPitch && aligned_to(xpad, 16)) {
+    if (es == 4 && total < (1ll << 31) && xs[L] >= g_flat_min_row && ps[L] >= kFlatMinPitch && aligned_to(xpad, 16)) {
         const int64_t nstages = (total + kStage - 1) / kStage;
         FlatTop& t = a.top;
         t.x = a.x;
@@ -1013,7 +1021,7 @@ extern "C" int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x
         }
         return check_launch("halo_flat_kernel");
     }
-    switch (elem_size) {
+    switch (es) {
         case 1: return launch_halo<uint8_t>(a, lpr, s);
         case 2: return launch_halo<uint16_t>(a, lpr, s);
         case 4: return launch_halo<uint32_t>(a, lpr, s);
