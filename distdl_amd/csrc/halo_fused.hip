@@ -16,9 +16,13 @@
 // source (a ghost slab, the shard, or zero) and is forwarded to the bulk slabs
 // that contain it.
 //
-// Mapping.  Dimensions are named L (last, columns), M (second to last, rows)
-// and "outer" (the rest, a plane index).  A workgroup owns one plane and a
-// chunk of its rows: everything that depends on the outer coordinates only
+// Two kernels.  halo_flat_kernel (further down) serves 4- and 8-byte elements
+// and writes the padded tensor in whole 128-byte lines; halo_pad_kernel serves
+// everything else and writes it row by row.
+//
+// Mapping of halo_pad_kernel.  Dimensions are named L (last, columns), M (second
+// to last, rows) and "outer" (the rest, a plane index).  A workgroup owns one
+// plane and a chunk of its rows: everything that depends on the outer coordinates only
 // (which slab or shard plane feeds the rows, which bulk slabs take them, all
 // base offsets) is wave-uniform scalar work done once per workgroup.  Each row
 // is then a run [wlo, whi) copied from one source with 16-byte vectors -- the
