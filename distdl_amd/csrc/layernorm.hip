@@ -182,7 +182,11 @@ __global__ __launch_bounds__(kBlock) void ln_norm_rows(const float* __restrict__
                     o.z = g[k].z * o.z + b[k].z;
                     o.w = g[k].w * o.w + b[k].w;
                 }
-                reinterpret_cast<float4*>(y + r * ldy)[c] = o;
+                // y is not read again by this kernel: streaming store
+                typedef float f32x4 __attribute__((ext_vector_type(4)));
+                f32x4 ov;
+                ov[0] = o.x, ov[1] = o.y, ov[2] = o.z, ov[3] = o.w;
+                __builtin_nontemporal_store(ov, reinterpret_cast<f32x4*>(y + r * ldy) + c);
             }
         }
     }
