@@ -102,7 +102,10 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_input(const float* __restrict__
             o.y = rs * (d.y * g.y - (S1 + ((v.y - m) * rs) * S2));
             o.z = rs * (d.z * g.z - (S1 + ((v.z - m) * rs) * S2));
             o.w = rs * (d.w * g.w - (S1 + ((v.w - m) * rs) * S2));
-            *reinterpret_cast<float4*>(dxr + c) = o;
+            typedef float f32x4 __attribute__((ext_vector_type(4)));   // dx is not read again here: streaming store
+            f32x4 ov;
+            ov[0] = o.x, ov[1] = o.y, ov[2] = o.z, ov[3] = o.w;
+            __builtin_nontemporal_store(ov, reinterpret_cast<f32x4*>(dxr + c));
         }
     } else {
         for (int64_t c = lane; c < cols; c += kWave) {

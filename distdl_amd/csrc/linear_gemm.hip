@@ -324,7 +324,10 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
             if (m >= M || n >= N) continue;
             uint16_t* dst = y + m * ldy + n;
             if (n + 8 <= N) {
-                *reinterpret_cast<uint4*>(dst) = v;
+                typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // y is not read again here: streaming store
+                u32x4 nv;
+                nv[0] = v.x, nv[1] = v.y, nv[2] = v.z, nv[3] = v.w;
+                __builtin_nontemporal_store(nv, reinterpret_cast<u32x4*>(dst));
             } else {
                 const uint32_t words[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
