@@ -37,15 +37,15 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # WRITE_SIZE runs of these same workloads, each counter scaled by what it reads
 # for a plain 64 MiB device copy (FETCH_SIZE x1.9993, WRITE_SIZE x1.0000); the
 # summaries are profiles/*_hbm_traffic_pmc.txt.  layernorm is the mean of its two
-# kernels (stats 8 482 114 B, normalize 17 875 673 B), like its launch time;
-# linear is the sum of the two launches of a step (256-wide tiles 436 357 536 B,
-# 192-wide tiles 396 782 657 B).
+# kernels (stats 8 482 120 B, normalize 17 875 696 B), like its launch time;
+# linear is the sum of the two launches of a step (256-wide tiles 436 339 712 B,
+# 192-wide tiles 397 789 146 B).
 MEASURED_TRAFFIC_BYTES = {
-    "repartition": 134414544,
-    "layernorm": 13178894,
-    "embedding": 1210703742,
-    "linear": 833140193,
-    "halo": 579271283,
+    "repartition": 134416460,
+    "layernorm": 13178908,
+    "embedding": 1210744581,
+    "linear": 834128858,
+    "halo": 568004548,
 }
 
 
@@ -55,7 +55,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default=None, help="run a single workload (repartition, layernorm, layernorm_long, embedding, linear, halo, layernorm_bwd, embedding_bwd, linear_bwd, calib)")
+    ap.add_argument("--only", default=None, help="run only these workloads, comma-separated (repartition, layernorm, layernorm_long, embedding, linear, halo, layernorm_bwd, embedding_bwd, linear_bwd, calib)")
     ap.add_argument("--no-graph", action="store_true", help="launch on the stream instead of replaying a HIP graph")
     return ap.parse_args()
 
@@ -498,7 +498,10 @@ def main():
         "linear_bwd": (build_linear_bwd, 2, 1, "mfma"),
         "calib": (build_calib, 4, 1, "hbm"),     # only with --only calib
     }
-    names = [args.only] if args.only else [n for n in builders if n != "calib"]
+    names = [n.strip() for n in args.only.split(",")] if args.only else [n for n in builders if n != "calib"]
+    for n in names:
+        if n not in builders:
+            raise SystemExit(f"bench.py: unknown workload {n!r}; choose from {', '.join(builders)}")
     results = {}
     for name in names:
         build, nsets, launches, bound = builders[name]

@@ -131,14 +131,35 @@ __global__ __launch_bounds__(kBlock) void colsum_partial_kernel(const uint16_t* 
     }
 }
 
-// Stage 2: out[col] = bf16(sum over splits of partial[split, col]).
+// Stage 2: out[col] = bf16(sum over splits of partial[split, col]).  A workgroup
+// per 64-column strip; lane group t / 64 adds every fourth split (eight
+// independent loads in flight), LDS folds the four groups.
 __global__ __launch_bounds__(kBlock) void colsum_final_kernel(const float* __restrict__ partial, int64_t cols, int splits,
                                                               uint16_t* __restrict__ out) {
-    const int64_t col = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    if (col >= cols) return;
+    constexpr int kGroups = kBlock / kTile;
+    __shared__ float fold[kGroups][kTile];
+    const int g = threadIdx.x / kTile, t = threadIdx.x % kTile;
+    const int64_t col = static_cast<int64_t>(blockIdx.x) * kTile + t;
     float s = 0.f;
-    for (int k = 0; k < splits; ++k) s += partial[static_cast<int64_t>(k) * cols + col];
-    out[col] = f32_to_bf16(s);
+    if (col < cols) {
+        int k = g;
+        for (; k + 7 * kGroups < splits; k += 8 * kGroups) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = partial[static_cast<int64_t>(k + u * kGroups) * cols + col];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += v[u];
+        }
+        for (; k < splits; k += kGroups) s += partial[static_cast<int64_t>(k) * cols + col];
+    }
+    fold[g][t] = s;
+    __syncthreads();
+    if (g == 0 && col < cols) {
+        float r = 0.f;
+#pragma unroll
+        for (int k = 0; k < kGroups; ++k) r += fold[k][t];
+        out[col] = f32_to_bf16(r);
+    }
 }
 
 }  // namespace
@@ -185,7 +206,7 @@ extern "C" int ddl_colsum_bf16(const void* a, int64_t rows, int64_t cols, int64_
                        (aligned_to(a, 16) && ld % 8 == 0) ? 1 : 0);
     int rc = check_launch("colsum_partial_kernel");
     if (rc) return rc;
-    hipLaunchKernelGGL(colsum_final_kernel, dim3(static_cast<uint32_t>((cols + kBlock - 1) / kBlock)), dim3(kBlock), 0, s,
+    hipLaunchKernelGGL(colsum_final_kernel, dim3(static_cast<uint32_t>(strips)), dim3(kBlock), 0, s,
                        workspace, cols, static_cast<int>(splits), static_cast<uint16_t*>(out));
     return check_launch("colsum_final_kernel");
 }
