@@ -168,6 +168,27 @@ def test_fused_halo_wide_rows_geometries(ops, halo_path):
                 [[0, 0], [2, 1], [1, 1], [1, 2]], torch.float32, 63)
 
 
+def test_fused_halo_random_geometries(ops, halo_path):
+    """Seeded sweep over ranks, widths, missing neighbours and row lengths either
+    side of the whole-line kernel's limits; every case bit-exact against the oracle."""
+    rng = np.random.default_rng(20240611)
+    for case in range(36):
+        nd = int(rng.integers(1, 6))
+        x_shape, pad, recv, send = [], [], [], []
+        for d in range(nd):
+            last = d == nd - 1
+            n = int(rng.integers(20, 140)) if last else int(rng.integers(1, 7))
+            exchanged = last or rng.random() < 0.6
+            r = [int(rng.integers(0, 3)) if exchanged else 0 for _ in range(2)]
+            p = [r[k] + (int(rng.integers(0, 3)) if exchanged and rng.random() < 0.3 else 0) for k in range(2)]
+            s_ = [int(rng.integers(0, min(3, n) + 1)) if exchanged else 0 for _ in range(2)]
+            x_shape.append(n)
+            pad.append(p)
+            recv.append(r)
+            send.append(s_)
+        _fused_case(ops, tuple(x_shape), pad, recv, send, torch.float32, 1000 + case)
+
+
 def test_fused_halo_config5_rank0_bit_exact(ops, halo_path):
     """[1,32,128,128,128] fp32 shard of a 2x2x2 split, kernel 3, padding 1."""
     g = [1, 32, 256, 256, 256]
