@@ -238,7 +238,10 @@ __global__ __launch_bounds__(kBlock) void emb_bwd_reduce_bf16x8(const uint16_t* 
         q.y = o[2] | (static_cast<uint32_t>(o[3]) << 16);
         q.z = o[4] | (static_cast<uint32_t>(o[5]) << 16);
         q.w = o[6] | (static_cast<uint32_t>(o[7]) << 16);
-        *reinterpret_cast<uint4*>(dst + j * kChunk) = q;
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // streaming store: the gradient is not read again here
+        u32x4 nv;
+        nv[0] = q.x, nv[1] = q.y, nv[2] = q.z, nv[3] = q.w;
+        __builtin_nontemporal_store(nv, reinterpret_cast<u32x4*>(dst + j * kChunk));
     }
 }
 
