@@ -65,11 +65,19 @@ def _self_slices(overlaps):
 
 
 def _covered(overlaps, shape):
+    """Do the (disjoint) overlaps tile a tensor of this shape completely?"""
+    cache = getattr(overlaps, "plans", None)
+    key = ("covered", shape)
+    if cache is not None and key in cache:
+        return cache[key]
     volume = 0
     for sl, sh, partner in overlaps:
         if sl is not None:
             volume += int(np.prod(sh, dtype=np.int64))
-    return volume == int(np.prod(shape, dtype=np.int64))
+    covered = volume == int(np.prod(shape, dtype=np.int64))
+    if cache is not None:
+        cache[key] = covered
+    return covered
 
 
 def _move(src, P_union, dtype, P_src, src_overlaps, src_buffers, P_dst, dst_overlaps, dst_buffers, dst_shape,

@@ -17,7 +17,14 @@ _ADD_DTYPES = {
 }
 
 
+# torch's raw-stream query costs a microsecond; building a torch.cuda.Stream
+# object for every launch costs ten.
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+    if _raw_stream is not None:
+        return ctypes.c_void_p(_raw_stream(torch.cuda.current_device()))
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
