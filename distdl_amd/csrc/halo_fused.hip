@@ -16,9 +16,9 @@
 // source (a ghost slab, the shard, or zero) and is forwarded to the bulk slabs
 // that contain it.
 //
-// Two kernels.  halo_flat_kernel (further down) serves 4- and 8-byte elements
-// and writes the padded tensor in whole 128-byte lines; halo_pad_kernel serves
-// everything else and writes it row by row.
+// Two kernels.  halo_flat_kernel (further down) serves 2-, 4- and 8-byte
+// elements and writes the padded tensor in whole 128-byte lines;
+// halo_pad_kernel serves everything else and writes it row by row.
 //
 // Mapping of halo_pad_kernel.  Dimensions are named L (last, columns), M (second
 // to last, rows) and "outer" (the rest, a plane index).  A workgroup owns one
@@ -486,13 +486,13 @@ __global__ __launch_bounds__(kBlock) void halo_pad_kernel(const HaloArgs args_by
 }
 
 // ---------------------------------------------------------------------------
-// 4-byte elements, whole-line stores.  Rows of the padded tensor are seldom
+// 2- and 4-byte elements, whole-line stores.  Rows of the padded tensor are seldom
 // whole 128-byte lines (130 floats in the convolution case), and writing them
 // row by row costs a quarter of the store rate.  The padded tensor is
 // contiguous, though, so it is also a plain run of elements: a wavefront takes
-// kStage consecutive elements (4 KiB, aligned in memory), assembles them in its
-// own LDS area and writes the area out with aligned 16-byte vectors, 1 KiB per
-// instruction.
+// kStage consecutive elements (4 or 2 KiB, aligned in memory), assembles them in
+// its own LDS area and writes the area out with aligned 16-byte vectors, 1 KiB
+// per instruction.
 //
 // Assembly: at most 64 padded rows meet a piece, so lane k classifies row k --
 // all rows at once, in vector arithmetic: plane and row number, the plane's
@@ -502,7 +502,7 @@ __global__ __launch_bounds__(kBlock) void halo_pad_kernel(const HaloArgs args_by
 // one source pointer per row, held by lane k (a row is either a shard row, whose
 // run is the shard's columns, or a ghost row, whose run is the bulk range of L:
 // bit 0 of the pointer says which).  The area is cleared and filled by 16
-// global -> LDS loads of 4 bytes per lane: lane l of load m owns element
+// global -> LDS loads of one element per lane: lane l of load m owns element
 // 64 m + l of the piece, takes its row's pointer from lane k with a cross-lane
 // read and fetches from there (or stays idle: zeros), so consecutive lanes
 // fetch consecutive addresses.
@@ -525,21 +525,23 @@ __device__ inline int64_t slab_row_offset(SlabPtr b, const uint32_t (&c)[HD], ui
     return off;
 }
 
-template <int ND>
+// T: uint32_t or uint16_t.  In LDS every element has a 4-byte slot (a 2-byte
+// global -> LDS load writes its lane's slot, zero-extended); 2-byte elements are
+// packed when the piece is read back.
+template <int ND, typename T>
 __global__ __launch_bounds__(kBlock) void halo_flat_kernel(const HaloArgs args_by_value) {
 #if defined(__HIP_DEVICE_COMPILE__)
     ArgsPtr a = (ArgsPtr)__builtin_amdgcn_kernarg_segment_ptr();
 #else
     ArgsPtr a = &args_by_value;
 #endif
-    typedef uint32_t T;
     constexpr int L = ND - 1, M = ND - 2;
-    __shared__ __attribute__((aligned(16))) T stage_mem[kWavesPerBlock * kArea];
+    __shared__ __attribute__((aligned(16))) uint32_t stage_mem[kWavesPerBlock * kArea];
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const uint32_t stage = blockIdx.x * kWavesPerBlock + wave;
     if (stage >= a->top.nstages) return;
-    T* const area = stage_mem + wave * kArea;                    // element g0 of the padded tensor
+    uint32_t* const area = stage_mem + wave * kArea;             // slot of element g0 of the padded tensor
     const uint32_t g0 = stage * kStage;
     const uint32_t total = a->top.total;
     const uint32_t n_el = total - g0 < kStage ? total - g0 : kStage;
@@ -675,8 +677,12 @@ __global__ __launch_bounds__(kBlock) void halo_flat_kernel(const HaloArgs args_b
             const bool ghost_row = (plo & 1u) != 0;
             const uint32_t lo = ghost_row ? glo : padL, hi = ghost_row ? ghi : xhiL;
             const T* p = reinterpret_cast<const T*>(static_cast<uint64_t>(plo & ~1u) | (static_cast<uint64_t>(phi) << 32));
-            if (m * kWave + lane < n_el && p != nullptr && w >= lo && w < hi)
-                __builtin_amdgcn_global_load_lds((global_ptr)(p + w), (lds_ptr)(area + m * kWave), 4, 0, 0);
+            if (m * kWave + lane < n_el && p != nullptr && w >= lo && w < hi) {
+                if (sizeof(T) == 4)
+                    __builtin_amdgcn_global_load_lds((global_ptr)(p + w), (lds_ptr)(area + m * kWave), 4, 0, 0);
+                else
+                    __builtin_amdgcn_global_load_lds((global_ptr)(p + w), (lds_ptr)(area + m * kWave), 2, 0, 0);
+            }
             w += kWave;
 #pragma unroll
             for (int t = 0; t < 2; ++t) {                         // rows hold at least 32 elements
@@ -711,23 +717,34 @@ __global__ __launch_bounds__(kBlock) void halo_flat_kernel(const HaloArgs args_b
     __builtin_amdgcn_s_waitcnt(0x0070);                          // every load has landed, every LDS write is done
     asm volatile("" ::: "memory");
 
-    // ---- the piece leaves in whole lines ----
+    // ---- the piece leaves in whole lines: 16 bytes per lane, 1 KiB per instruction ----
     {
         T* const out = reinterpret_cast<T*>(a->top.xpad) + g0;
+        constexpr uint32_t EPV = 16 / sizeof(T);                 // elements per store
+        typedef typename VecType<uint32_t, 4>::type V;           // the padded tensor is not read again here: streaming store
 #pragma unroll
-        for (uint32_t j = 0; j < kStage / 256; ++j) {
-            const uint32_t o = j * 256 + lane * 4;
-            const uint4 v = *reinterpret_cast<const uint4*>(area + o);
-            if (o + 4 <= n_el) {
-                typedef typename VecType<T, 4>::type V;          // the padded tensor is not read again here: streaming store
+        for (uint32_t j = 0; j < kStage / (kWave * EPV); ++j) {
+            const uint32_t o = (j * kWave + lane) * EPV;
+            uint32_t e[EPV];
+#pragma unroll
+            for (uint32_t t = 0; t < EPV; t += 4) {
+                const uint4 v = *reinterpret_cast<const uint4*>(area + o + t);
+                e[t] = v.x, e[t + 1] = v.y, e[t + 2] = v.z, e[t + 3] = v.w;
+            }
+            if (o + EPV <= n_el) {
                 V nv;
-                nv[0] = v.x, nv[1] = v.y, nv[2] = v.z, nv[3] = v.w;
+                if (sizeof(T) == 4) {
+#pragma unroll
+                    for (uint32_t t = 0; t < 4; ++t) nv[t] = e[t];
+                } else {
+#pragma unroll
+                    for (uint32_t t = 0; t < 4; ++t) nv[t] = e[(2 * t) % EPV] | (e[(2 * t + 1) % EPV] << 16);
+                }
                 __builtin_nontemporal_store(nv, reinterpret_cast<V*>(out + o));
             } else {
-                const T ev[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    if (o + t < n_el) out[o + t] = ev[t];
+                for (uint32_t t = 0; t < EPV; ++t)
+                    if (o + t < n_el) out[o + t] = static_cast<T>(e[t]);
             }
         }
     }
@@ -746,7 +763,7 @@ __global__ __launch_bounds__(kBlock) void halo_flat_kernel(const HaloArgs args_b
             const uint32_t q = static_cast<uint32_t>(rowq0 + static_cast<int>(k * W + w));
             const int64_t row = static_cast<int64_t>(row0) + k;
             if (e < nrows * n_strip && q < n_el) {
-                const T v = area[q];
+                const T v = static_cast<T>(area[q]);
                 if (i < n_bl)
                     bl[row * sl + (w - glo)] = v;
                 else
@@ -777,7 +794,7 @@ __global__ __launch_bounds__(kBlock) void halo_flat_kernel(const HaloArgs args_b
                 for (; w0 < ghi && rowq + static_cast<int>(w0) < static_cast<int>(n_el); w0 += kWave) {
                     const uint32_t w = w0 + lane;
                     const uint32_t q = static_cast<uint32_t>(rowq + static_cast<int>(w));
-                    if (w < ghi && q < n_el) dst[w] = area[q];
+                    if (w < ghi && q < n_el) dst[w] = static_cast<T>(area[q]);
                 }
             };
             // dimension M: the row's own strips; outer dimensions are unrestricted
@@ -961,7 +978,7 @@ extern "C" int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x
     if (nplanes * static_cast<int64_t>(a.row_chunks) >= (1ll << 31)) return fail(DDL_E_UNSUPP, "halo: too many workgroups");
     a.nplanes = static_cast<uint32_t>(nplanes);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (es == 4 && total < (1ll << 31) && xs[L] >= g_flat_min_row && ps[L] >= kFlatMinPitch && aligned_to(xpad, 16)) {
+    if ((es == 4 || es == 2) && total < (1ll << 31) && xs[L] >= g_flat_min_row && ps[L] >= kFlatMinPitch && aligned_to(xpad, 16)) {
         const int64_t nstages = (total + kStage - 1) / kStage;
         FlatTop& t = a.top;
         t.x = a.x;
@@ -1016,12 +1033,22 @@ extern "C" int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x
             if (a.bulk[j][0].ptr || a.bulk[j][1].ptr) t.any_outer = 1;
         }
         const dim3 grid(static_cast<uint32_t>((nstages + kWavesPerBlock - 1) / kWavesPerBlock));
-        switch (nd) {
-            case 2: hipLaunchKernelGGL(halo_flat_kernel<2>, grid, dim3(kBlock), 0, s, a); break;
-            case 3: hipLaunchKernelGGL(halo_flat_kernel<3>, grid, dim3(kBlock), 0, s, a); break;
-            case 4: hipLaunchKernelGGL(halo_flat_kernel<4>, grid, dim3(kBlock), 0, s, a); break;
-            case 5: hipLaunchKernelGGL(halo_flat_kernel<5>, grid, dim3(kBlock), 0, s, a); break;
-            default: hipLaunchKernelGGL(halo_flat_kernel<6>, grid, dim3(kBlock), 0, s, a); break;
+        if (es == 4) {
+            switch (nd) {
+                case 2: hipLaunchKernelGGL((halo_flat_kernel<2, uint32_t>), grid, dim3(kBlock), 0, s, a); break;
+                case 3: hipLaunchKernelGGL((halo_flat_kernel<3, uint32_t>), grid, dim3(kBlock), 0, s, a); break;
+                case 4: hipLaunchKernelGGL((halo_flat_kernel<4, uint32_t>), grid, dim3(kBlock), 0, s, a); break;
+                case 5: hipLaunchKernelGGL((halo_flat_kernel<5, uint32_t>), grid, dim3(kBlock), 0, s, a); break;
+                default: hipLaunchKernelGGL((halo_flat_kernel<6, uint32_t>), grid, dim3(kBlock), 0, s, a); break;
+            }
+        } else {
+            switch (nd) {
+                case 2: hipLaunchKernelGGL((halo_flat_kernel<2, uint16_t>), grid, dim3(kBlock), 0, s, a); break;
+                case 3: hipLaunchKernelGGL((halo_flat_kernel<3, uint16_t>), grid, dim3(kBlock), 0, s, a); break;
+                case 4: hipLaunchKernelGGL((halo_flat_kernel<4, uint16_t>), grid, dim3(kBlock), 0, s, a); break;
+                case 5: hipLaunchKernelGGL((halo_flat_kernel<5, uint16_t>), grid, dim3(kBlock), 0, s, a); break;
+                default: hipLaunchKernelGGL((halo_flat_kernel<6, uint16_t>), grid, dim3(kBlock), 0, s, a); break;
+            }
         }
         return check_launch("halo_flat_kernel");
     }

@@ -149,12 +149,12 @@ int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x_shape,
                           void* stream);
 
 /* Tuning knob of ddl_halo_pad_exchange (no counterpart in the reference):
- * tensors of 4- or 8-byte elements whose shard rows hold at least `elements`
- * 4-byte words (and whose padded rows hold at least 32) are assembled through
- * LDS and stored in whole 128-byte lines; shorter rows, 1- and 2-byte elements,
- * outputs not aligned to 16 bytes and tensors of 2^31 words or more are written
- * row by row.  Both ways give identical results.
- * Default 32.  Process-wide; not synchronised with concurrent calls. */
+ * tensors of 2-, 4- or 8-byte elements whose shard rows hold at least
+ * `elements` elements (8-byte ones count as two) and whose padded rows hold at
+ * least 32 are assembled through LDS and stored in whole 128-byte lines;
+ * shorter rows, 1-byte elements, outputs not aligned to 16 bytes and tensors of
+ * 2^31 elements or more are written row by row.  Both ways give identical
+ * results.  Default 32.  Process-wide; not synchronised with concurrent calls. */
 int ddl_halo_set_flat_min_row(int64_t elements);
 
 /* ------------------------------------------------------------------------ *

@@ -166,6 +166,11 @@ def test_fused_halo_wide_rows_geometries(ops, halo_path):
                 [[0, 0], [0, 0], [0, 0], [0, 0]], torch.float32, 62)
     _fused_case(ops, (2, 6, 40, 64), [[0, 0], [2, 2], [1, 1], [2, 2]], [[0, 0], [0, 0], [0, 0], [0, 0]],
                 [[0, 0], [2, 1], [1, 1], [1, 2]], torch.float32, 63)
+    # 2-byte elements: odd widths, pieces of 1024 elements that end inside a row, a volume that is not a multiple of 8
+    _fused_case(ops, (3, 9, 131), [[0, 0], [1, 1], [1, 1]], [[0, 0], [1, 1], [1, 1]], [[0, 0], [1, 1], [1, 1]],
+                torch.float16, 64)
+    _fused_case(ops, (2, 3, 2500), [[0, 0], [1, 1], [2, 3]], [[0, 0], [1, 1], [2, 3]], [[0, 0], [1, 1], [3, 2]],
+                torch.float16, 65)
 
 
 def test_fused_halo_random_geometries(ops, halo_path):
@@ -186,7 +191,8 @@ def test_fused_halo_random_geometries(ops, halo_path):
             pad.append(p)
             recv.append(r)
             send.append(s_)
-        _fused_case(ops, tuple(x_shape), pad, recv, send, torch.float32, 1000 + case)
+        dtype = (torch.float32, torch.float16, torch.float64)[case % 3]
+        _fused_case(ops, tuple(x_shape), pad, recv, send, dtype, 1000 + case)
 
 
 def test_fused_halo_config5_rank0_bit_exact(ops, halo_path):
