@@ -37,15 +37,15 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # WRITE_SIZE runs of these same workloads, each counter scaled by what it reads
 # for a plain 64 MiB device copy (FETCH_SIZE x1.9993, WRITE_SIZE x1.0000); the
 # summaries are profiles/*_hbm_traffic_pmc.txt.  layernorm is the mean of its two
-# kernels (stats 8 482 120 B, normalize 17 875 696 B), like its launch time;
-# linear is the sum of the two launches of a step (256-wide tiles 436 339 712 B,
-# 192-wide tiles 397 789 146 B).
+# kernels (stats 8 482 132 B, normalize 17 875 667 B), like its launch time;
+# linear is the sum of the two launches of a step (256-wide tiles 436 344 160 B,
+# 192-wide tiles 398 065 226 B).
 MEASURED_TRAFFIC_BYTES = {
-    "repartition": 134416460,
-    "layernorm": 13178908,
-    "embedding": 1210744581,
-    "linear": 834128858,
-    "halo": 568004548,
+    "repartition": 134414634,
+    "layernorm": 13178900,
+    "embedding": 1210721771,
+    "linear": 834409386,
+    "halo": 568008812,
 }
 
 
