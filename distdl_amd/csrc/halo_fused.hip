@@ -79,7 +79,7 @@ struct FlatDim {
     uint32_t lo, hi;         // bulk range
     uint32_t padl, xs;
     uint32_t strip_l1, strip_r0;   // coordinates [lo, strip_l1) and [strip_r0, hi) feed this dimension's bulk slabs
-    uint32_t unused;
+    uint32_t reserved;       // keeps xstride 8-byte aligned
     int64_t xstride;
 };
 
