@@ -338,9 +338,11 @@ def _call(lib, _lib, name, args):
 
 
 def build_layernorm_bwd(torch, lib, _lib, nsets):
-    """Backward of config 1 on rank 0: row sums, input gradient, parameter
-    gradients.  Algorithmic bytes: dy and x are read three times (once per
-    kernel), dx is written once: 7 x 8 388 608 B, plus the small vectors."""
+    """Backward of config 1 on rank 0 as the layer runs it when every gradient
+    is wanted: row sums + partial column sums in one launch, then (after the
+    gather of the row sums) input gradient + final parameter sums in one launch.
+    Algorithmic bytes: dy and x are read twice (once per launch), dx is written
+    once: 5 x 8 388 608 B, plus the small vectors and the partial column sums."""
     rows, cols = 16 * 512, 256
     keep, steps = [], []
     for s in range(nsets):
@@ -356,14 +358,13 @@ def build_layernorm_bwd(torch, lib, _lib, nsets):
         work = torch.empty(2 * 256 * cols, device="cuda")
         keep.append((x, dy, gamma, mean, rstd, sums, dx, dg, db, work))
         a1 = (dy.data_ptr(), x.data_ptr(), rows, cols, cols, cols, mean.data_ptr(), rstd.data_ptr(), gamma.data_ptr(),
-              sums.data_ptr())
+              sums.data_ptr(), work.data_ptr(), work.numel())
         a2 = (dy.data_ptr(), x.data_ptr(), rows, cols, cols, cols, mean.data_ptr(), rstd.data_ptr(), gamma.data_ptr(),
-              sums.data_ptr(), 4, 1.0 / (4 * cols), dx.data_ptr(), cols)
-        a3 = (dy.data_ptr(), x.data_ptr(), rows, cols, cols, cols, mean.data_ptr(), rstd.data_ptr(), dg.data_ptr(),
-              db.data_ptr(), work.data_ptr(), work.numel())
-        steps.append([_call(lib, _lib, "ddl_ln_bwd_partial_f32", a1), _call(lib, _lib, "ddl_ln_bwd_input_f32", a2),
-                      _call(lib, _lib, "ddl_ln_bwd_params_f32", a3)])
-    return steps, keep, 7 * rows * cols * 4 + 3 * (2 * rows * 4) + 5 * rows * 2 * 4 + 3 * cols * 4
+              sums.data_ptr(), 4, 1.0 / (4 * cols), dx.data_ptr(), cols, work.data_ptr(), work.numel(), dg.data_ptr(),
+              db.data_ptr())
+        steps.append([_call(lib, _lib, "ddl_ln_bwd_partial_params_f32", a1),
+                      _call(lib, _lib, "ddl_ln_bwd_input_params_f32", a2)])
+    return steps, keep, 5 * rows * cols * 4 + 2 * (2 * rows * 4) + 5 * rows * 2 * 4 + 3 * cols * 4 + 2 * (2 * 256 * cols * 4)
 
 
 def build_embedding_bwd(torch, lib, _lib, nsets):
@@ -493,7 +494,7 @@ def main():
         "embedding": (build_embedding, 4, 1, "hbm"),
         "linear": (build_linear, 4, 1, "mfma"),
         "halo": (build_halo, 4, 1, "hbm"),
-        "layernorm_bwd": (build_layernorm_bwd, 32, 3, "hbm"),
+        "layernorm_bwd": (build_layernorm_bwd, 32, 2, "hbm"),
         "embedding_bwd": (build_embedding_bwd, 4, 1, "hbm"),
         "linear_bwd": (build_linear_bwd, 2, 1, "mfma"),
         "calib": (build_calib, 4, 1, "hbm"),     # only with --only calib

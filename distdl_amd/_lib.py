@@ -68,6 +68,11 @@ SIGNATURES = {
                                      c_void_p, c_int, c_float, c_void_p, c_int64, c_void_p]),
     "ddl_ln_bwd_params_f32": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
                                       c_void_p, c_void_p, c_int64, c_void_p]),
+    "ddl_ln_bwd_partial_params_f32": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
+                                              c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
+    "ddl_ln_bwd_input_params_f32": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
+                                            c_void_p, c_void_p, c_int, c_float, c_void_p, c_int64, c_void_p, c_int64,
+                                            c_void_p, c_void_p, c_void_p]),
     "ddl_embedding_gather": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_int, c_int64, c_int64, c_int64,
                                      c_void_p, c_void_p]),
     "ddl_embedding_backward": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64,

@@ -71,13 +71,13 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_partial(const float* __restrict
 }
 
 template <bool VEC>
-__global__ __launch_bounds__(kBlock) void ln_bwd_input(const float* __restrict__ dy, const float* __restrict__ x, int64_t rows,
-                                                       int64_t cols, int64_t ld_dy, int64_t ld_x,
-                                                       const float* __restrict__ mean, const float* __restrict__ rstd,
-                                                       const float* __restrict__ gamma, const float* __restrict__ part_sums,
-                                                       int nparts, float weight, float* __restrict__ dx, int64_t ld_dx) {
+__device__ inline void ln_bwd_input_body(uint32_t block, const float* __restrict__ dy, const float* __restrict__ x, int64_t rows,
+                                         int64_t cols, int64_t ld_dy, int64_t ld_x, const float* __restrict__ mean,
+                                         const float* __restrict__ rstd, const float* __restrict__ gamma,
+                                         const float* __restrict__ part_sums, int nparts, float weight, float* __restrict__ dx,
+                                         int64_t ld_dx) {
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t r = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + threadIdx.x / kWave;
+    const int64_t r = static_cast<int64_t>(block) * kWavesPerBlock + threadIdx.x / kWave;
     if (r >= rows) return;
     // the pairs of all workers of this row, one worker per lane (and round)
     float p1 = 0.f, p2 = 0.f;
@@ -113,6 +113,15 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_input(const float* __restrict__
             dxr[c] = rs * (g - (S1 + ((xr[c] - m) * rs) * S2));
         }
     }
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void ln_bwd_input(const float* __restrict__ dy, const float* __restrict__ x, int64_t rows,
+                                                       int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                                       const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                       const float* __restrict__ gamma, const float* __restrict__ part_sums,
+                                                       int nparts, float weight, float* __restrict__ dx, int64_t ld_dx) {
+    ln_bwd_input_body<VEC>(blockIdx.x, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, part_sums, nparts, weight, dx, ld_dx);
 }
 
 // Workgroup (strip, split): rows [split * rows_per_split, ...) of a 64-column
@@ -151,11 +160,11 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_params_partial(const float* __r
 // Workgroup per 64-column strip: lane group g = t / 64 adds the splits g, g+4,
 // ... of column t % 64 (independent loads, eight in flight), LDS folds the four
 // groups.
-__global__ __launch_bounds__(kBlock) void ln_bwd_params_final(const float* __restrict__ partial, int64_t cols, int splits,
-                                                              float* __restrict__ dgamma, float* __restrict__ dbeta) {
+__device__ inline void ln_bwd_params_final_body(uint32_t block, const float* __restrict__ partial, int64_t cols, int splits,
+                                                float* __restrict__ dgamma, float* __restrict__ dbeta) {
     __shared__ float fold[2][kWavesPerBlock][kStrip];
     const int g = threadIdx.x / kStrip, t = threadIdx.x % kStrip;
-    const int64_t c = static_cast<int64_t>(blockIdx.x) * kStrip + t;
+    const int64_t c = static_cast<int64_t>(block) * kStrip + t;
     float a = 0.f, b = 0.f;
     if (c < cols) {
         int k = g;
@@ -190,6 +199,113 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_params_final(const float* __res
     }
 }
 
+__global__ __launch_bounds__(kBlock) void ln_bwd_params_final(const float* __restrict__ partial, int64_t cols, int splits,
+                                                              float* __restrict__ dgamma, float* __restrict__ dbeta) {
+    ln_bwd_params_final_body(blockIdx.x, partial, cols, splits, dgamma, dbeta);
+}
+
+// dx and the final parameter sums in one launch: the first final_blocks
+// workgroups (one per 64-column strip) add up the partial column sums -- a chain
+// of dependent loads, so they start first -- and the rest write dx.  The two
+// parts are independent.
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void ln_bwd_input_final(const float* __restrict__ dy, const float* __restrict__ x, int64_t rows,
+                                                             int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                                             const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                             const float* __restrict__ gamma, const float* __restrict__ part_sums,
+                                                             int nparts, float weight, float* __restrict__ dx, int64_t ld_dx,
+                                                             uint32_t final_blocks, const float* __restrict__ partial, int splits,
+                                                             float* __restrict__ dgamma, float* __restrict__ dbeta) {
+    if (blockIdx.x < final_blocks)
+        ln_bwd_params_final_body(blockIdx.x, partial, cols, splits, dgamma, dbeta);
+    else
+        ln_bwd_input_body<VEC>(blockIdx.x - final_blocks, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, part_sums, nparts,
+                               weight, dx, ld_dx);
+}
+
+constexpr int kFusedBlock = 512;   // eight wavefronts: a split of 32 rows is one round of four rows per wavefront
+constexpr int kFusedWaves = kFusedBlock / kWave;
+
+// Row sums {sum g, sum g xhat} and the partial column sums of a row split in one
+// pass over dy and x: workgroup = split, its wavefronts take every eighth row
+// and each lane keeps the columns (lane + 64 k) * 4 .. + 3, k < NV, in registers.
+// partial has the layout of ln_bwd_params_partial.
+template <int NV>
+__global__ __launch_bounds__(kFusedBlock) void ln_bwd_partial_cols(const float* __restrict__ dy, const float* __restrict__ x, int64_t rows,
+                                                              int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                                              const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                              const float* __restrict__ gamma, float* __restrict__ sums,
+                                                              int64_t rows_per_split, float* __restrict__ partial) {
+    __shared__ float fold[2][kFusedWaves][NV * kWave * 4];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int nv = static_cast<int>(cols >> 2);
+    const int64_t r_begin = static_cast<int64_t>(blockIdx.x) * rows_per_split;
+    const int64_t r_end = r_begin + rows_per_split < rows ? r_begin + rows_per_split : rows;
+    float4 g[NV], ca[NV], cb[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int c = lane + k * kWave;
+        g[k] = make_float4(1.f, 1.f, 1.f, 1.f);
+        if (gamma && c < nv) g[k] = reinterpret_cast<const float4*>(gamma)[c];
+        ca[k] = cb[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    constexpr int RU = NV <= 2 ? 4 : 2;   // rows whose loads are in flight together
+    for (int64_t r0 = r_begin + wave; r0 < r_end; r0 += kFusedWaves * RU) {
+        float m[RU], rs[RU];
+        float4 d[RU][NV], v[RU][NV];
+#pragma unroll
+        for (int u = 0; u < RU; ++u) {
+            const int64_t r = r0 + u * kFusedWaves;
+            const bool on = r < r_end;
+            m[u] = on ? mean[r] : 0.f;
+            rs[u] = on ? rstd[r] : 0.f;
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                const int c = lane + k * kWave;
+                d[u][k] = v[u][k] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (on && c < nv) {
+                    d[u][k] = reinterpret_cast<const float4*>(dy + r * ld_dy)[c];
+                    v[u][k] = reinterpret_cast<const float4*>(x + r * ld_x)[c];
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < RU; ++u) {
+            const int64_t r = r0 + u * kFusedWaves;
+            if (r >= r_end) break;                              // wave-uniform
+            float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+            for (int k = 0; k < NV; ++k) {
+                // columns past the row hold zeros in d, so they add nothing
+                const float4 dd = d[u][k], vv = v[u][k];
+                const float h0 = (vv.x - m[u]) * rs[u], h1 = (vv.y - m[u]) * rs[u], h2 = (vv.z - m[u]) * rs[u], h3 = (vv.w - m[u]) * rs[u];
+                const float g0 = dd.x * g[k].x, g1 = dd.y * g[k].y, g2 = dd.z * g[k].z, g3 = dd.w * g[k].w;
+                s1 += (g0 + g1) + (g2 + g3);
+                s2 += (g0 * h0 + g1 * h1) + (g2 * h2 + g3 * h3);
+                ca[k].x += dd.x * h0, ca[k].y += dd.y * h1, ca[k].z += dd.z * h2, ca[k].w += dd.w * h3;
+                cb[k].x += dd.x, cb[k].y += dd.y, cb[k].z += dd.z, cb[k].w += dd.w;
+            }
+            s1 = wave_sum(s1);
+            s2 = wave_sum(s2);
+            if (lane == 0) reinterpret_cast<float2*>(sums)[r] = make_float2(s1, s2);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int c4 = (lane + k * kWave) * 4;
+        *reinterpret_cast<float4*>(&fold[0][wave][c4]) = ca[k];
+        *reinterpret_cast<float4*>(&fold[1][wave][c4]) = cb[k];
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 2 * static_cast<int>(cols); i += kFusedBlock) {
+        const int which = i >= static_cast<int>(cols) ? 1 : 0, c = i - which * static_cast<int>(cols);
+        float t = 0.f;
+#pragma unroll
+        for (int w = 0; w < kFusedWaves; ++w) t += fold[which][w][c];
+        partial[(static_cast<int64_t>(blockIdx.x) * 2 + which) * cols + c] = t;
+    }
+}
+
 bool vectorizable(int64_t cols, std::initializer_list<int64_t> lds, std::initializer_list<const void*> ptrs) {
     if (cols % 4 != 0) return false;
     for (int64_t ld : lds)
@@ -205,6 +321,17 @@ int check_rows(const char* what, int64_t rows, int64_t cols, int64_t ld_dy, int6
                     (long long)ld_dy, (long long)ld_x);
     if (rows > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "%s: more than 2^31 rows", what);
     return 0;
+}
+
+// Row splits of the parameter gradients: as many as the workspace holds, at most
+// 256 and at least 32 rows each.  0 when the workspace cannot hold one split.
+int64_t param_splits(int64_t rows, int64_t cols, int64_t workspace_elems) {
+    int64_t splits = workspace_elems / (2 * cols);
+    if (splits < 1) return 0;
+    if (splits > 256) splits = 256;
+    const int64_t by_rows = (rows + 31) / 32;
+    if (splits > by_rows) splits = by_rows > 0 ? by_rows : 1;
+    return splits;
 }
 
 }  // namespace
@@ -259,11 +386,8 @@ extern "C" int ddl_ln_bwd_params_f32(const float* dy, const float* x, int64_t ro
     if (!aligned_to(dy, 4) || !aligned_to(x, 4) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) || !aligned_to(dgamma, 4) ||
         !aligned_to(dbeta, 4) || !aligned_to(workspace, 4))
         return fail(DDL_E_ALIGN, "ln backward parameters: pointers must be 4-byte aligned");
-    int64_t splits = workspace_elems / (2 * cols);
+    const int64_t splits = param_splits(rows, cols, workspace_elems);
     if (splits < 1) return fail(DDL_E_ARG, "ln backward parameters: workspace of %lld floats is smaller than 2 x %lld", (long long)workspace_elems, (long long)cols);
-    if (splits > 256) splits = 256;
-    const int64_t by_rows = (rows + 31) / 32;
-    if (splits > by_rows) splits = by_rows > 0 ? by_rows : 1;
     const int64_t rows_per_split = rows > 0 ? (rows + splits - 1) / splits : 1;
     const int64_t strips = (cols + kStrip - 1) / kStrip;
     if (strips * splits > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "ln backward parameters: too many workgroups");
@@ -274,4 +398,70 @@ extern "C" int ddl_ln_bwd_params_f32(const float* dy, const float* x, int64_t ro
     hipLaunchKernelGGL(ln_bwd_params_final, dim3(static_cast<uint32_t>(strips)), dim3(kBlock), 0, s, workspace, cols,
                        static_cast<int>(splits), dgamma, dbeta);
     return check_launch("ln_bwd_params_final");
+}
+
+extern "C" int ddl_ln_bwd_partial_params_f32(const float* dy, const float* x, int64_t rows, int64_t cols, int64_t ld_dy,
+                                             int64_t ld_x, const float* mean, const float* rstd, const float* gamma, float* sums,
+                                             float* workspace, int64_t workspace_elems, void* stream) {
+    using namespace ddl;
+    if (int rc = check_rows("ln backward sums", rows, cols, ld_dy, ld_x)) return rc;
+    if (!workspace) return fail(DDL_E_ARG, "ln backward sums: null workspace");
+    const int64_t splits = param_splits(rows, cols, workspace_elems);
+    if (splits < 1) return fail(DDL_E_ARG, "ln backward sums: workspace of %lld floats is smaller than 2 x %lld", (long long)workspace_elems, (long long)cols);
+    if (rows > 0 && (!dy || !x || !mean || !rstd || !sums)) return fail(DDL_E_ARG, "ln backward sums: null pointer");
+    if (!aligned_to(dy, 4) || !aligned_to(x, 4) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) || !aligned_to(gamma, 4) ||
+        !aligned_to(sums, 8) || !aligned_to(workspace, 4))
+        return fail(DDL_E_ALIGN, "ln backward sums: pointers must be 4-byte aligned, the sums 8-byte");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t rows_per_split = rows > 0 ? (rows + splits - 1) / splits : 1;
+    if (rows > 0 && cols <= 4 * kWave * 4 && vectorizable(cols, {ld_dy, ld_x}, {dy, x, gamma})) {
+        const dim3 grid(static_cast<uint32_t>(splits));
+        if (cols <= kWave * 4)
+            hipLaunchKernelGGL(ln_bwd_partial_cols<1>, grid, dim3(kFusedBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, sums, rows_per_split, workspace);
+        else if (cols <= 2 * kWave * 4)
+            hipLaunchKernelGGL(ln_bwd_partial_cols<2>, grid, dim3(kFusedBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, sums, rows_per_split, workspace);
+        else
+            hipLaunchKernelGGL(ln_bwd_partial_cols<4>, grid, dim3(kFusedBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, sums, rows_per_split, workspace);
+        return check_launch("ln_bwd_partial_cols");
+    }
+    // long or unaligned rows: the two passes separately, same results in the same places
+    if (rows > 0) {
+        if (int rc = ddl_ln_bwd_partial_f32(dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, sums, stream)) return rc;
+    }
+    const int64_t strips = (cols + kStrip - 1) / kStrip;
+    if (strips * splits > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "ln backward sums: too many workgroups");
+    hipLaunchKernelGGL(ln_bwd_params_partial, dim3(static_cast<uint32_t>(strips * splits)), dim3(kBlock), 0, s, dy, x, rows, cols,
+                       ld_dy, ld_x, mean, rstd, rows_per_split, workspace, static_cast<int>(strips));
+    return check_launch("ln_bwd_params_partial");
+}
+
+extern "C" int ddl_ln_bwd_input_params_f32(const float* dy, const float* x, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                           const float* mean, const float* rstd, const float* gamma, const float* part_sums,
+                                           int nparts, float weight, float* dx, int64_t ld_dx, const float* workspace,
+                                           int64_t workspace_elems, float* dgamma, float* dbeta, void* stream) {
+    using namespace ddl;
+    if (int rc = check_rows("ln backward input", rows, cols, ld_dy, ld_x)) return rc;
+    if (ld_dx < cols || nparts < 1) return fail(DDL_E_ARG, "ln backward input: ld_dx=%lld nparts=%d", (long long)ld_dx, nparts);
+    if (!workspace) return fail(DDL_E_ARG, "ln backward input: null workspace");
+    const int64_t splits = param_splits(rows, cols, workspace_elems);
+    if (splits < 1) return fail(DDL_E_ARG, "ln backward input: workspace of %lld floats is smaller than 2 x %lld", (long long)workspace_elems, (long long)cols);
+    if (rows > 0 && (!dy || !x || !mean || !rstd || !part_sums || !dx)) return fail(DDL_E_ARG, "ln backward input: null pointer");
+    if (!aligned_to(dy, 4) || !aligned_to(x, 4) || !aligned_to(dx, 4) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) ||
+        !aligned_to(gamma, 4) || !aligned_to(part_sums, 8) || !aligned_to(workspace, 4) || !aligned_to(dgamma, 4) || !aligned_to(dbeta, 4))
+        return fail(DDL_E_ALIGN, "ln backward input: pointers must be 4-byte aligned, the sums 8-byte");
+    const int64_t input_blocks = (rows + kWavesPerBlock - 1) / kWavesPerBlock;
+    const int64_t strips = (dgamma || dbeta) ? (cols + kStrip - 1) / kStrip : 0;
+    if (input_blocks + strips == 0) return 0;
+    if (input_blocks + strips > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "ln backward input: too many workgroups");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 grid(static_cast<uint32_t>(input_blocks + strips));
+    if (vectorizable(cols, {ld_dy, ld_x, ld_dx}, {dy, x, gamma, dx}))
+        hipLaunchKernelGGL(ln_bwd_input_final<true>, grid, dim3(kBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma,
+                           part_sums, nparts, weight, dx, ld_dx, static_cast<uint32_t>(strips), workspace,
+                           static_cast<int>(splits), dgamma, dbeta);
+    else
+        hipLaunchKernelGGL(ln_bwd_input_final<false>, grid, dim3(kBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma,
+                           part_sums, nparts, weight, dx, ld_dx, static_cast<uint32_t>(strips), workspace,
+                           static_cast<int>(splits), dgamma, dbeta);
+    return check_launch("ln_bwd_input_final");
 }

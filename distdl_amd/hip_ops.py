@@ -325,12 +325,54 @@ def ln_backward_params(dy2d, x2d, mean, rstd, want_gamma=True, want_beta=True):
     rows, cols = x2d.shape
     dg = torch.empty(cols, dtype=torch.float32, device=x2d.device) if want_gamma else None
     db = torch.empty(cols, dtype=torch.float32, device=x2d.device) if want_beta else None
-    splits = max(1, min(256, (rows + 31) // 32))
-    work = torch.empty(2 * splits * cols, dtype=torch.float32, device=x2d.device)
+    work = _ln_param_workspace(rows, cols, x2d.device)
     rc = _lib.load().ddl_ln_bwd_params_f32(dy2d.data_ptr(), x2d.data_ptr(), rows, cols, ld_dy, ld_x, mean.data_ptr(),
                                            rstd.data_ptr(), _ptr(dg), _ptr(db), work.data_ptr(), work.numel(), _stream())
     _lib.check(rc, "ddl_ln_bwd_params_f32")
     return dg, db
+
+
+def _ln_param_workspace(rows, cols, device):
+    splits = max(1, min(256, (rows + 31) // 32))
+    return torch.empty(2 * splits * cols, dtype=torch.float32, device=device)
+
+
+def ln_backward_partial_params(dy2d, x2d, mean, rstd, gamma):
+    """``ln_backward_partial`` plus, in the same pass, the partial column sums
+    for the parameter gradients.  Returns (sums [rows, 2], workspace); hand the
+    workspace to ``ln_backward_input_params``."""
+    _require_gpu(dy2d, x2d, mean, rstd, gamma)
+    ld_dy, ld_x = _rows2d(dy2d, "ln_backward_partial_params"), _rows2d(x2d, "ln_backward_partial_params")
+    rows, cols = x2d.shape
+    sums = torch.empty((rows, 2), dtype=torch.float32, device=x2d.device)
+    work = _ln_param_workspace(rows, cols, x2d.device)
+    rc = _lib.load().ddl_ln_bwd_partial_params_f32(dy2d.data_ptr(), x2d.data_ptr(), rows, cols, ld_dy, ld_x,
+                                                   mean.data_ptr(), rstd.data_ptr(), _ptr(gamma), sums.data_ptr(),
+                                                   work.data_ptr(), work.numel(), _stream())
+    _lib.check(rc, "ddl_ln_bwd_partial_params_f32")
+    return sums, work
+
+
+def ln_backward_input_params(dy2d, x2d, mean, rstd, gamma, part_sums, weight, work, want_gamma=True, want_beta=True):
+    """dx as ``ln_backward_input`` and, in the same launch, (dgamma, dbeta) from
+    the workspace that ``ln_backward_partial_params`` filled."""
+    _require_gpu(dy2d, x2d, mean, rstd, gamma, part_sums, work)
+    ld_dy, ld_x = _rows2d(dy2d, "ln_backward_input_params"), _rows2d(x2d, "ln_backward_input_params")
+    rows, cols = x2d.shape
+    if part_sums.dtype != torch.float32 or part_sums.dim() != 3 or tuple(part_sums.shape[1:]) != (rows, 2) or \
+       not part_sums.is_contiguous():
+        raise ValueError(f"ln_backward_input_params: part_sums must be contiguous fp32 [P, {rows}, 2]")
+    if work.dtype != torch.float32 or not work.is_contiguous():
+        raise ValueError("ln_backward_input_params: the workspace must be a contiguous fp32 tensor")
+    dx = torch.empty((rows, cols), dtype=torch.float32, device=x2d.device)
+    dg = torch.empty(cols, dtype=torch.float32, device=x2d.device) if want_gamma else None
+    db = torch.empty(cols, dtype=torch.float32, device=x2d.device) if want_beta else None
+    rc = _lib.load().ddl_ln_bwd_input_params_f32(dy2d.data_ptr(), x2d.data_ptr(), rows, cols, ld_dy, ld_x, mean.data_ptr(),
+                                                 rstd.data_ptr(), _ptr(gamma), part_sums.data_ptr(), part_sums.shape[0],
+                                                 float(weight), dx.data_ptr(), cols, work.data_ptr(), work.numel(),
+                                                 _ptr(dg), _ptr(db), _stream())
+    _lib.check(rc, "ddl_ln_bwd_input_params_f32")
+    return dx, dg, db
 
 
 def embedding_gather(weight, ids, lo, hi, out=None):

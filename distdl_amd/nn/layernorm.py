@@ -62,20 +62,29 @@ class _LayerNormShard(torch.autograd.Function):
         if dy2d.shape[1] > 1 and dy2d.stride(1) != 1:
             dy2d = dy2d.contiguous()
         dx = dw = db = None
+        w_shape, b_shape = ctx.param_shapes
+        want_w, want_b = need_w and w_shape is not None, need_b and b_shape is not None
+        fused = need_x and (want_w or want_b)        # two launches instead of four
         if need_x:
-            sums = hip_ops.ln_backward_partial(dy2d, x2d, mean, rstd, gamma)
+            if fused:
+                sums, work = hip_ops.ln_backward_partial_params(dy2d, x2d, mean, rstd, gamma)
+            else:
+                sums = hip_ops.ln_backward_partial(dy2d, x2d, mean, rstd, gamma)
             if ctx.nparts > 1:
                 gathered = ctx.P_reduce._world.transport.allgather(ctx.P_reduce, sums, tag=BWD_SUMS_TAG).contiguous()
             else:
                 gathered = sums.unsqueeze(0)
-            dx = hip_ops.ln_backward_input(dy2d, x2d, mean, rstd, gamma, gathered, 1.0 / (ctx.nparts * ctx.cols))
+            weight_a = 1.0 / (ctx.nparts * ctx.cols)
+            if fused:
+                dx, dw, db = hip_ops.ln_backward_input_params(dy2d, x2d, mean, rstd, gamma, gathered, weight_a, work,
+                                                              want_w, want_b)
+            else:
+                dx = hip_ops.ln_backward_input(dy2d, x2d, mean, rstd, gamma, gathered, weight_a)
             dx = dx.view(grad_output.shape)
-        w_shape, b_shape = ctx.param_shapes
-        want_w, want_b = need_w and w_shape is not None, need_b and b_shape is not None
-        if want_w or want_b:
+        elif want_w or want_b:
             dw, db = hip_ops.ln_backward_params(dy2d, x2d, mean, rstd, want_w, want_b)
-            dw = None if dw is None else dw.view(w_shape)
-            db = None if db is None else db.view(b_shape)
+        dw = None if dw is None else dw.view(w_shape)
+        db = None if db is None else db.view(b_shape)
         return dx, dw, db, None, None, None
 
 

@@ -223,6 +223,35 @@ int ddl_ln_bwd_params_f32(const float* dy, const float* x, int64_t rows,
                           float* dbeta, float* workspace,
                           int64_t workspace_elems, void* stream);
 
+/* The same three results in two launches instead of four, for a caller that
+ * wants dx and the parameter gradients (rows of a few hundred floats are
+ * launch-bound, so this halves the time):
+ *
+ *   ddl_ln_bwd_partial_params_f32   sums[] as ddl_ln_bwd_partial_f32, and in the
+ *                                   same pass over dy and x the row-split
+ *                                   partial column sums, left in `workspace`
+ *   ddl_ln_bwd_input_params_f32     dx as ddl_ln_bwd_input_f32, and in the same
+ *                                   launch dgamma / dbeta (either may be NULL)
+ *                                   from the partial sums in `workspace`
+ *
+ * Both calls take the same rows, cols, workspace and workspace_elems (at least
+ * 2 * cols floats, up to 512 * cols are used); the second must follow the first
+ * on the same stream. */
+int ddl_ln_bwd_partial_params_f32(const float* dy, const float* x, int64_t rows,
+                                  int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                  const float* mean, const float* rstd,
+                                  const float* gamma, float* sums,
+                                  float* workspace, int64_t workspace_elems,
+                                  void* stream);
+int ddl_ln_bwd_input_params_f32(const float* dy, const float* x, int64_t rows,
+                                int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                const float* mean, const float* rstd,
+                                const float* gamma, const float* part_sums,
+                                int nparts, float weight, float* dx,
+                                int64_t ld_dx, const float* workspace,
+                                int64_t workspace_elems, float* dgamma,
+                                float* dbeta, void* stream);
+
 /* ------------------------------------------------------------------------ *
  * DistributedEmbedding shard gather
  * ------------------------------------------------------------------------ */

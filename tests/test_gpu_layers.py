@@ -187,7 +187,7 @@ def test_layernorm_backward_kernels_match_oracle(ops, cols, affine):
             xh = (shards[p].astype(np.float64) - m64[:, None]) * r64[:, None]
             pair = np.stack([gp.sum(axis=1), (gp * xh).sum(axis=1)], axis=1)
             if p == live:
-                scale = np.abs(gp).sum(axis=1).max()
+                scale = scale_live = np.abs(gp).sum(axis=1).max()
                 assert np.allclose(sums.cpu().numpy(), pair, rtol=1e-4, atol=2e-5 * scale)
                 gathered.append(sums)
             else:
@@ -199,6 +199,41 @@ def test_layernorm_backward_kernels_match_oracle(ops, cols, affine):
         assert np.abs(dx.cpu().numpy() - want_dx[live]).max() <= 4 * tol
         assert np.allclose(dg.cpu().numpy(), want_dg[live], rtol=1e-4, atol=1e-4)
         assert np.allclose(db.cpu().numpy(), want_db[live], rtol=1e-4, atol=1e-4)
+        # the two-launch variant: same sums, same gradients
+        sums2, work = ops.ln_backward_partial_params(dy2d, x2d, mean, rstd, g)
+        assert np.allclose(sums2.cpu().numpy(), sums.cpu().numpy(), rtol=1e-5, atol=1e-5 * scale_live)
+        gathered[live] = sums2
+        dx2, dg2, db2 = ops.ln_backward_input_params(dy2d, x2d, mean, rstd, g, torch.stack(gathered).contiguous(),
+                                                     1.0 / (P * cols[live]), work)
+        torch.cuda.synchronize()
+        assert np.abs(dx2.cpu().numpy() - want_dx[live]).max() <= 4 * tol
+        assert np.allclose(dg2.cpu().numpy(), want_dg[live], rtol=1e-4, atol=1e-4)
+        assert np.allclose(db2.cpu().numpy(), want_db[live], rtol=1e-4, atol=1e-4)
+        dx3, dg3, db3 = ops.ln_backward_input_params(dy2d, x2d, mean, rstd, g, torch.stack(gathered).contiguous(),
+                                                     1.0 / (P * cols[live]), work, want_gamma=False, want_beta=True)
+        assert dg3 is None and torch.equal(db3, db2) and torch.equal(dx3, dx2)
+
+
+def test_layernorm_backward_two_launch_variant_many_rows(ops):
+    """Row splits of more than one wavefront round, a last split that is short,
+    rows of 256 / 512 / 1024 floats (one, two, four vectors per lane)."""
+    rng = np.random.default_rng(77)
+    for rows, cols in ((8192, 256), (1000, 512), (333, 1024), (70, 1028)):
+        x = (rng.standard_normal((rows, cols)) * 1.5 + 0.25).astype(np.float32)
+        dy = rng.standard_normal((rows, cols)).astype(np.float32)
+        gamma = (1 + 0.1 * rng.standard_normal(cols)).astype(np.float32)
+        want_dx, want_dg, want_db = o_ln.backward_shards([x], [gamma], [dy], 1e-5)
+        xg, dyg, gg = torch.from_numpy(x).cuda(), torch.from_numpy(dy).cuda(), torch.from_numpy(gamma).cuda()
+        stats = ops.ln_partial_stats(xg)
+        _, mean, rstd = ops.ln_normalize_affine(xg, stats.unsqueeze(0).contiguous(), [cols], gg, gg, 1e-5, want_stats=True)
+        sums, work = ops.ln_backward_partial_params(dyg, xg, mean, rstd, gg)
+        dx, dg, db = ops.ln_backward_input_params(dyg, xg, mean, rstd, gg, sums.unsqueeze(0).contiguous(), 1.0 / cols, work)
+        torch.cuda.synchronize()
+        tol = 1e-5 * max(1.0, np.abs(want_dx[0]).max())
+        assert np.abs(dx.cpu().numpy() - want_dx[0]).max() <= 4 * tol
+        scale = np.sqrt(rows)
+        assert np.allclose(dg.cpu().numpy(), want_dg[0], rtol=1e-4, atol=1e-4 * scale)
+        assert np.allclose(db.cpu().numpy(), want_db[0], rtol=1e-4, atol=1e-4 * scale)
 
 
 def test_layernorm_layer_backward_matches_torch():
