@@ -72,6 +72,17 @@ __device__ inline void dma16(__amdgpu_buffer_rsrc_t buffer, int voffset, int sof
     __builtin_amdgcn_raw_ptr_buffer_load_lds(buffer, (lds_ptr)dst, 16, voffset, soffset, 0, 0);
 }
 
+// acc += a . b (32 x 32 x 16, bf16 in, fp32 accumulate).  Written as assembly
+// so that the accumulators live in the accumulation registers ("a" operands):
+// left to itself the compiler keeps them in the vector registers next to the
+// fragments, which measures 2 % slower.  The compiler still tracks the
+// operands (it waits for the LDS reads that produce a and b); what it does not
+// do for assembly is pad the distance between an MFMA and a later non-MFMA
+// read of acc -- the kernel does that once, in front of the epilogue.
+__device__ inline void mfma_32x32x16(floatx16& acc, const bf16x8& a, const bf16x8& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+
 // s_waitcnt immediate (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4,
 // lgkmcnt 11:8): wait until at most n vector-memory requests are outstanding
 // and all LDS reads have returned.
@@ -222,7 +233,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
 #pragma unroll
             for (int i = 0; i < TN * TM; ++i) {
                 const int a = i / TM, b = i % TM;
-                acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][a], fb[ks & 1][b], acc[a][b], 0, 0, 0);
+                mfma_32x32x16(acc[a][b], fa[ks & 1][a], fb[ks & 1][b]);
                 if (i < TN + TM) read_frag(wt, xt, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1], i);
                 if (STEADY && ks == 0 && i % kGapW == kGapW - 1 && i / kGapW < JW_W) request_part(buf_w, off_gw, t + 2, w2_off, i / kGapW);
                 __builtin_amdgcn_sched_barrier(0);
@@ -239,7 +250,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
 #pragma unroll
         for (int i = 0; i < TN * TM; ++i) {
             const int a = i / TM, b = i % TM;
-            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][a], fb[1][b], acc[a][b], 0, 0, 0);
+            mfma_32x32x16(acc[a][b], fa[1][a], fb[1][b]);
             // Past the last tile these reads fetch stale LDS contents that are never used.
             if (i < TN + TM) read_frag(wn1, xn1, 0, fa[0], fb[0], i);
             if (STEADY && i % kGapX == kGapX - 1 && i / kGapX < JW_X) request_part(buf_x, off_gx, t + 2, x2_off, i / kGapX);
@@ -269,6 +280,9 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
 #pragma unroll 1
     for (; t < ktiles; ++t) k_tile(t, std::false_type{});
 
+    // The last MFMAs must have left the pipeline before acc is read by anything
+    // else (18 wait states cover every case; these are 32).
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     // Epilogue.  Lane holds, per 32x32 tile, output row m = l32 and the columns
     // n = 8*g + 4*kg + {0,1,2,3} for g = 0..3 in acc[...][4*g + {0..3}].
     if (vec_store == 2) {
