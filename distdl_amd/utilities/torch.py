@@ -17,17 +17,15 @@ class TensorStructure:
     """(shape, dtype, requires_grad) of a tensor; layers re-run their setup when
     it changes (utilities/torch.py:16-40)."""
 
+    __slots__ = ("shape", "dtype", "requires_grad")
+
     def __init__(self, tensor=None):
-        self.shape = None
-        self.dtype = None
-        self.requires_grad = None
+        self.shape = self.dtype = self.requires_grad = None      # "nothing seen yet"
         if tensor is not None:
             self.fill_from_tensor(tensor)
 
     def fill_from_tensor(self, tensor):
-        self.shape = tensor.shape
-        self.dtype = tensor.dtype
-        self.requires_grad = tensor.requires_grad
+        self.shape, self.dtype, self.requires_grad = tensor.shape, tensor.dtype, tensor.requires_grad
 
     def _key(self):
         shape = None if self.shape is None else tuple(int(s) for s in self.shape)
