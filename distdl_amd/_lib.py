@@ -30,6 +30,8 @@ DDL_DT_F64 = 2
 DDL_DT_BF16 = 3
 DDL_DT_F16 = 4
 
+DDL_EMBEDDING_BACKWARD_STATIC_MAX_ELEMS = 1048576
+
 
 class ddl_box_t(ctypes.Structure):
     _fields_ = [
@@ -77,6 +79,8 @@ SIGNATURES = {
                                      c_void_p, c_void_p]),
     "ddl_embedding_backward": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64,
                                        c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
+    "ddl_embedding_backward_static": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64,
+                                              c_int64, c_void_p, c_int64, c_void_p]),
     "ddl_linear_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                 c_int64, c_void_p]),
     "ddl_transpose_2d": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),

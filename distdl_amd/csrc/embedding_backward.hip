@@ -19,6 +19,14 @@
 //   emb_bwd_reduce   sort each bucket (it is short), sum, convert, store
 #include "ddl_common.h"
 
+#include <mutex>
+
+// Workspace of ddl_embedding_backward_static: the counters, bucket starts and
+// token buckets of one call, for callers that cannot hand over (or allocate)
+// device memory.  Every GPU the library runs on holds its own 4 MiB copy until
+// the process ends; its device address is looked up once per device.
+static __device__ __align__(256) int32_t scratch[DDL_EMBEDDING_BACKWARD_STATIC_MAX_ELEMS];
+
 namespace ddl {
 namespace {
 
@@ -284,8 +292,51 @@ int run(const void* dy, int dtype, int64_t dim, int64_t ld_dy, const IdT* ids, i
     return check_launch("embedding backward");
 }
 
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+int32_t* scratch_address[kMaxDevices] = {};   // device address of `scratch` on each GPU, filled on first use
+
+// The device address of `scratch` on the current GPU.  In host code the name
+// `scratch` is only a handle for the runtime, never a pointer a kernel may use.
+int scratch_on_current_device(int32_t** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(static_cast<int>(e), "embedding backward (static): hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(DDL_E_UNSUPP, "embedding backward (static): device index %d (at most %d devices)", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_address[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return fail(e != hipSuccess ? static_cast<int>(e) : DDL_E_ARG, "embedding backward (static): hipGetSymbolAddress: %s", hipGetErrorString(e));
+        scratch_address[dev] = static_cast<int32_t*>(p);
+    }
+    *out = scratch_address[dev];
+    return 0;
+}
+
 }  // namespace
 }  // namespace ddl
+
+extern "C" int ddl_embedding_backward_static(const void* dy, int dtype, int64_t dim, int64_t ld_dy, const void* ids, int ids_is_i64,
+                                             int64_t n_ids, int64_t lo, int64_t hi, int64_t padding_idx, void* dweight,
+                                             int64_t ld_dw, void* stream) {
+    using namespace ddl;
+    if (n_ids < 0 || hi < lo) return fail(DDL_E_ARG, "embedding backward (static): n_ids=%lld window=[%lld,%lld)", (long long)n_ids, (long long)lo, (long long)hi);
+    const int64_t rows = hi - lo;
+    // compared without forming 2 rows + 1 + n_ids, which could overflow
+    if (rows > DDL_EMBEDDING_BACKWARD_STATIC_MAX_ELEMS || n_ids > DDL_EMBEDDING_BACKWARD_STATIC_MAX_ELEMS ||
+        2 * rows + 1 + n_ids > DDL_EMBEDDING_BACKWARD_STATIC_MAX_ELEMS)
+        return fail(DDL_E_UNSUPP,
+                    "embedding backward (static): 2 * %lld rows + 1 + %lld tokens exceeds the built-in workspace of %lld int32; "
+                    "use ddl_embedding_backward with a workspace of your own", (long long)rows, (long long)n_ids,
+                    (long long)DDL_EMBEDDING_BACKWARD_STATIC_MAX_ELEMS);
+    int32_t* ws = nullptr;
+    const int rc = scratch_on_current_device(&ws);
+    if (rc) return rc;
+    return ddl_embedding_backward(dy, dtype, dim, ld_dy, ids, ids_is_i64, n_ids, lo, hi, padding_idx, dweight, ld_dw, ws,
+                                  DDL_EMBEDDING_BACKWARD_STATIC_MAX_ELEMS, stream);
+}
 
 extern "C" int ddl_embedding_backward(const void* dy, int dtype, int64_t dim, int64_t ld_dy, const void* ids, int ids_is_i64,
                                       int64_t n_ids, int64_t lo, int64_t hi, int64_t padding_idx, void* dweight,

@@ -284,6 +284,24 @@ int ddl_embedding_backward(const void* dy, int dtype, int64_t dim, int64_t ld_dy
                            void* dweight, int64_t ld_dw, int32_t* workspace,
                            int64_t workspace_elems, void* stream);
 
+/* ddl_embedding_backward without the workspace argument, for callers that
+ * cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid allocation).  No counterpart in the reference.
+ * The counters and buckets live in a 4 MiB device array built into the library
+ * (one copy per GPU, held until the process ends); the call allocates nothing
+ * and frees nothing.  It fails with DDL_E_UNSUPP when
+ *   2 (hi - lo) + 1 + n_ids > DDL_EMBEDDING_BACKWARD_STATIC_MAX_ELEMS.
+ * All calls on one GPU share that array: calls that overlap in time on one GPU
+ * (different streams or threads) race; calls on one stream are safe.  The
+ * array's device address is looked up the first time a GPU is used, so make
+ * that first call outside any stream capture.  Results are those of
+ * ddl_embedding_backward. */
+#define DDL_EMBEDDING_BACKWARD_STATIC_MAX_ELEMS 1048576
+int ddl_embedding_backward_static(const void* dy, int dtype, int64_t dim, int64_t ld_dy,
+                                  const void* ids, int ids_is_i64, int64_t n_ids,
+                                  int64_t lo, int64_t hi, int64_t padding_idx,
+                                  void* dweight, int64_t ld_dw, void* stream);
+
 /* ------------------------------------------------------------------------ *
  * DistributedLinear shard GEMM (bf16 in, fp32 accumulate, bf16 out)
  * ------------------------------------------------------------------------ */
