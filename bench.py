@@ -314,7 +314,7 @@ def build_halo(torch, lib, _lib, nsets):
                 gptr.append(None if g is None else g.data_ptr())
                 bptr.append(None if b is None else b.data_ptr())
         args = (x.data_ptr(), out.data_ptr(), plan.shape_arr, 5, 4, plan.pad_arr, plan.recv_arr, plan.send_arr,
-                _lib.ptr_array(gptr), _lib.ptr_array(bptr))
+                _lib.ptr_array(gptr), _lib.ptr_array(bptr), _lib.DDL_HALO_AUTO)
         keep.append((x, out, bufs, args))
 
         def fused(a=args):
@@ -384,7 +384,7 @@ def build_embedding_bwd(torch, lib, _lib, nsets):
         dw = torch.empty(16032, 4096, dtype=torch.bfloat16, device="cuda")
         work = torch.empty(2 * 16032 + 1 + ids.numel(), dtype=torch.int32, device="cuda")
         keep.append((ids, dw, work))
-        args = (dy.data_ptr(), _lib.DDL_DT_BF16, 4096, 4096, ids.data_ptr(), 1, ids.numel(), 0, 16032, -1, dw.data_ptr(),
+        args = (dy.data_ptr(), _lib.DDL_DT_BF16, 4096, 4096, ids.data_ptr(), 1, ids.numel(), 0, 16032, -1, 0, dw.data_ptr(),
                 4096, work.data_ptr(), work.numel())
         steps.append([_call(lib, _lib, "ddl_embedding_backward", args)])
     return steps, keep, sum(nbytes) / len(nbytes)

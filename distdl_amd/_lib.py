@@ -30,6 +30,10 @@ DDL_DT_F64 = 2
 DDL_DT_BF16 = 3
 DDL_DT_F16 = 4
 
+DDL_HALO_AUTO = 0
+DDL_HALO_ROWS = 1
+DDL_HALO_LINES = 2
+
 DDL_EMBEDDING_BACKWARD_STATIC_MAX_ELEMS = 1048576
 
 
@@ -58,8 +62,7 @@ SIGNATURES = {
                                POINTER(c_int64), POINTER(c_int64), c_void_p]),
     "ddl_halo_pad_exchange": (c_int, [c_void_p, c_void_p, POINTER(c_int64), c_int, c_int, POINTER(c_int64),
                                       POINTER(c_int64), POINTER(c_int64), POINTER(c_void_p), POINTER(c_void_p),
-                                      c_void_p]),
-    "ddl_halo_set_flat_min_row": (c_int, [c_int64]),
+                                      c_int, c_void_p]),
     "ddl_ln_partial_stats_f32": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "ddl_ln_normalize_affine_f32": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int, POINTER(c_int64),
                                             c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_void_p,
@@ -78,9 +81,9 @@ SIGNATURES = {
     "ddl_embedding_gather": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_int, c_int64, c_int64, c_int64,
                                      c_void_p, c_void_p]),
     "ddl_embedding_backward": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64,
-                                       c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
+                                       c_int, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "ddl_embedding_backward_static": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64,
-                                              c_int64, c_void_p, c_int64, c_void_p]),
+                                              c_int64, c_int, c_void_p, c_int64, c_void_p]),
     "ddl_linear_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                 c_int64, c_void_p]),
     "ddl_transpose_2d": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),

@@ -18,6 +18,12 @@ PRE_HOOK_CHECK_INPUT_CHANGED_ENV = "DISTDL_CHECK_INPUT_CHANGED"
 
 check_input_changed = True
 
+# Debug aid of DistributedEmbedding (no counterpart in the reference, whose
+# torch lookup raises by itself): check every forward's ids against
+# [0, num_embeddings) on the host before the gather kernel runs.
+CHECK_EMBEDDING_IDS_ENV = "DISTDL_CHECK_EMBEDDING_IDS"
+check_embedding_ids = os.environ.get(CHECK_EMBEDDING_IDS_ENV, "0") in ("1", "True")
+
 
 def get_default_comm():
     return os.environ.get(BACKEND_COMM_ENV, "stub")

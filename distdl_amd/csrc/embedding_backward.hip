@@ -16,7 +16,11 @@
 //   emb_bwd_count    count[row]++ per token in the window
 //   emb_bwd_scan     start[row] = exclusive prefix sum of count (one workgroup)
 //   emb_bwd_fill     bucket[start[row]++] = t, which leaves start[row] at the bucket's end
-//   emb_bwd_reduce   sort each bucket (it is short), sum, convert, store
+//   emb_bwd_sort     buckets longer than a wavefront: ascending token order (bitonic network)
+//   emb_bwd_reduce   order the short buckets in registers, sum, scale, convert, store
+//
+// The order in which the fill kernel's atomics hand out bucket slots varies
+// from run to run; both sorts exist so that the fp32 sums do not.
 #include "ddl_common.h"
 
 #include <mutex>
@@ -127,6 +131,79 @@ __global__ __launch_bounds__(kBlock) void emb_bwd_fill(const IdT* __restrict__ i
     if (r >= 0) bucket[atomicAdd(&start[r], 1)] = static_cast<int32_t>(t);   // start[r] ends as the end of bucket r
 }
 
+// Buckets of more than 64 tokens, sorted ascending in place.  Thread t of a
+// workgroup looks at row blockIdx.x * kBlock + t; the rows of the workgroup
+// that need sorting (few: tokens looked up that often are rare) are then taken
+// one after the other by the whole workgroup.  The network is the bitonic sort
+// in the form whose exchanges all put the smaller key first: partner of i is
+// its mirror image inside blocks of k in the first pass of a merge, i + j in
+// the others.  Keys beyond the end of the bucket count as +infinity and never
+// move, so any length works.  Buckets of up to kSortLds tokens are sorted in
+// LDS, longer ones where they lie (a workgroup's stores are visible to its own
+// later loads once the barrier between the passes has been passed; the loads
+// are volatile so that none is served from a stale cache line).
+constexpr int kSortLds = 8192;
+
+template <typename P>
+__device__ inline void bitonic_passes(P a, int32_t n) {
+    int32_t pow2 = 1;
+    while (pow2 < n) pow2 <<= 1;
+    for (int32_t k = 2; k <= pow2; k <<= 1) {
+        for (int32_t j = k >> 1; j > 0; j >>= 1) {
+            const bool mirror = j == (k >> 1);
+            for (int32_t t = threadIdx.x; t < (pow2 >> 1); t += kBlock) {
+                int32_t i, l;
+                if (mirror) {
+                    const int32_t blk = t / j, off = t - blk * j;
+                    i = blk * k + off;
+                    l = blk * k + k - 1 - off;
+                } else {
+                    const int32_t blk = t / j, off = t - blk * j;
+                    i = blk * 2 * j + off;
+                    l = i + j;
+                }
+                if (l < n) {
+                    const int32_t lo = a[i], hi = a[l];
+                    if (lo > hi) {
+                        a[i] = hi;
+                        a[l] = lo;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void emb_bwd_sort_long(const int32_t* __restrict__ start, int32_t* bucket, int64_t rows) {
+    __shared__ int32_t stage[kSortLds];
+    __shared__ int32_t todo[kBlock];
+    __shared__ int32_t n_todo;
+    if (threadIdx.x == 0) n_todo = 0;
+    __syncthreads();
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (r < rows) {
+        const int32_t b0 = r ? start[r - 1] : 0;
+        if (start[r] - b0 > kWave) todo[atomicAdd(&n_todo, 1)] = static_cast<int32_t>(threadIdx.x);
+    }
+    __syncthreads();
+    const int32_t cnt = n_todo;
+    for (int32_t q = 0; q < cnt; ++q) {
+        const int64_t row = static_cast<int64_t>(blockIdx.x) * kBlock + todo[q];
+        const int32_t b0 = row ? start[row - 1] : 0, n = start[row] - b0;
+        if (n <= kSortLds) {
+            for (int32_t i = threadIdx.x; i < n; i += kBlock) stage[i] = bucket[b0 + i];
+            __syncthreads();
+            bitonic_passes(stage, n);
+            for (int32_t i = threadIdx.x; i < n; i += kBlock) bucket[b0 + i] = stage[i];
+            __syncthreads();   // stage is refilled for the next row
+        } else {
+            __syncthreads();
+            bitonic_passes(static_cast<volatile int32_t*>(bucket + b0), n);
+        }
+    }
+}
+
 __device__ inline float load_as_f32(const uint16_t* p) { return __uint_as_float(static_cast<uint32_t>(*p) << 16); }
 __device__ inline float load_as_f32(const float* p) { return *p; }
 
@@ -144,8 +221,8 @@ __device__ inline void store_from_f32(float* p, float f) { *p = f; }
 // Order of the tokens of a bucket of at most 64: lane i holds one token and
 // counts the smaller ones (its rank), then every lane picks the token whose
 // rank is its own lane number.  Ascending token order makes the sums
-// independent of how the fill kernel's atomics interleaved; longer buckets are
-// taken as they are.
+// independent of how the fill kernel's atomics interleaved; longer buckets have
+// been put in order by emb_bwd_sort_long.
 __device__ inline int32_t sort_bucket(int32_t mine, int32_t m, int lane) {
     int32_t rank = 0;
     for (int k = 0; k < m; ++k) rank += __shfl(mine, k, kWave) < mine ? 1 : 0;
@@ -160,8 +237,9 @@ __device__ inline int32_t sort_bucket(int32_t mine, int32_t m, int lane) {
 // Wavefront (row, chunk): columns chunk * kChunk + lane + 64 j, j = 0..7.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void emb_bwd_reduce(const T* __restrict__ dy, int64_t dim, int64_t ld_dy,
-                                                         const int32_t* __restrict__ start, int32_t* __restrict__ bucket,
-                                                         int64_t rows, int chunks, T* __restrict__ dw, int64_t ld_dw) {
+                                                         const int32_t* __restrict__ start, const int32_t* __restrict__ bucket,
+                                                         int64_t rows, int chunks, T* __restrict__ dw, int64_t ld_dw,
+                                                         int scale_by_freq) {
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t w = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + threadIdx.x / kWave;
     const int64_t row = w / chunks;
@@ -185,10 +263,11 @@ __global__ __launch_bounds__(kBlock) void emb_bwd_reduce(const T* __restrict__ d
         }
     }
     T* dst = dw + row * ld_dw;
+    const float scale = (scale_by_freq && n > 1) ? 1.0f / static_cast<float>(n) : 1.0f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const int64_t c = c0 + 64 * j;
-        if (c < dim) store_from_f32(dst + c, acc[j]);
+        if (c < dim) store_from_f32(dst + c, acc[j] * scale);
     }
 }
 
@@ -199,8 +278,9 @@ __global__ __launch_bounds__(kBlock) void emb_bwd_reduce(const T* __restrict__ d
 // start and bucket is paid once for all of them.
 template <int CPW>
 __global__ __launch_bounds__(kBlock) void emb_bwd_reduce_bf16x8(const uint16_t* __restrict__ dy, int64_t dim, int64_t ld_dy,
-                                                                const int32_t* __restrict__ start, int32_t* __restrict__ bucket,
-                                                                int64_t rows, int groups, uint16_t* __restrict__ dw, int64_t ld_dw) {
+                                                                const int32_t* __restrict__ start, const int32_t* __restrict__ bucket,
+                                                                int64_t rows, int groups, uint16_t* __restrict__ dw, int64_t ld_dw,
+                                                                int scale_by_freq) {
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t w = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + threadIdx.x / kWave;
     const int64_t row = w / groups;
@@ -235,12 +315,13 @@ __global__ __launch_bounds__(kBlock) void emb_bwd_reduce_bf16x8(const uint16_t* 
         }
     }
     uint16_t* dst = dw + row * ld_dw + c0;
+    const float scale = (scale_by_freq && n > 1) ? 1.0f / static_cast<float>(n) : 1.0f;
 #pragma unroll
     for (int j = 0; j < CPW; ++j) {
         if (c0 + j * kChunk >= dim) continue;
         uint16_t o[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) store_from_f32(&o[e], acc[j][e]);
+        for (int e = 0; e < 8; ++e) store_from_f32(&o[e], acc[j][e] * scale);
         uint4 q;
         q.x = o[0] | (static_cast<uint32_t>(o[1]) << 16);
         q.y = o[2] | (static_cast<uint32_t>(o[3]) << 16);
@@ -254,18 +335,18 @@ __global__ __launch_bounds__(kBlock) void emb_bwd_reduce_bf16x8(const uint16_t* 
 }
 
 template <int CPW>
-void launch_reduce_x8(const void* dy, int64_t dim, int64_t ld_dy, const int32_t* start, int32_t* bucket, int64_t rows, int chunks,
-                      void* dw, int64_t ld_dw, hipStream_t s) {
+void launch_reduce_x8(const void* dy, int64_t dim, int64_t ld_dy, const int32_t* start, const int32_t* bucket, int64_t rows, int chunks,
+                      void* dw, int64_t ld_dw, int scale_by_freq, hipStream_t s) {
     const int groups = (chunks + CPW - 1) / CPW;
     const int64_t waves = rows * groups;
     hipLaunchKernelGGL((emb_bwd_reduce_bf16x8<CPW>), dim3(static_cast<uint32_t>((waves + kWavesPerBlock - 1) / kWavesPerBlock)),
                        dim3(kBlock), 0, s, static_cast<const uint16_t*>(dy), dim, ld_dy, start, bucket, rows, groups,
-                       static_cast<uint16_t*>(dw), ld_dw);
+                       static_cast<uint16_t*>(dw), ld_dw, scale_by_freq);
 }
 
 template <typename IdT>
 int run(const void* dy, int dtype, int64_t dim, int64_t ld_dy, const IdT* ids, int64_t n_ids, int64_t lo, int64_t hi,
-        int64_t padding_idx, void* dw, int64_t ld_dw, int32_t* ws, hipStream_t s) {
+        int64_t padding_idx, int scale_by_freq, void* dw, int64_t ld_dw, int32_t* ws, hipStream_t s) {
     const int64_t rows = hi - lo;
     int32_t* count = ws;                 // [rows]
     int32_t* start = ws + rows;          // [rows + 1]: begin of each bucket, advanced to its end by the fill pass
@@ -276,19 +357,20 @@ int run(const void* dy, int dtype, int64_t dim, int64_t ld_dy, const IdT* ids, i
     hipLaunchKernelGGL(emb_bwd_scan, dim3(1), dim3(kScanBlock), 0, s, count, rows, start);
     if (n_ids > 0)
         hipLaunchKernelGGL((emb_bwd_fill<IdT>), grid(n_ids), dim3(kBlock), 0, s, ids, n_ids, lo, hi, padding_idx, start, bucket);
+    if (n_ids > kWave) hipLaunchKernelGGL(emb_bwd_sort_long, grid(rows), dim3(kBlock), 0, s, start, bucket, rows);
     const int chunks = static_cast<int>((dim + kChunk - 1) / kChunk);
     const int64_t waves = rows * chunks;
     const dim3 rgrid(static_cast<uint32_t>((waves + kWavesPerBlock - 1) / kWavesPerBlock));
     const bool vec = dtype == DDL_DT_BF16 && dim % 8 == 0 && ld_dy % 8 == 0 && ld_dw % 8 == 0 && aligned_to(dy, 16) && aligned_to(dw, 16);
     if (vec) {
-        if (chunks >= 2) launch_reduce_x8<2>(dy, dim, ld_dy, start, bucket, rows, chunks, dw, ld_dw, s);
-        else launch_reduce_x8<1>(dy, dim, ld_dy, start, bucket, rows, chunks, dw, ld_dw, s);
+        if (chunks >= 2) launch_reduce_x8<2>(dy, dim, ld_dy, start, bucket, rows, chunks, dw, ld_dw, scale_by_freq, s);
+        else launch_reduce_x8<1>(dy, dim, ld_dy, start, bucket, rows, chunks, dw, ld_dw, scale_by_freq, s);
     } else if (dtype == DDL_DT_BF16)
         hipLaunchKernelGGL((emb_bwd_reduce<uint16_t>), rgrid, dim3(kBlock), 0, s, static_cast<const uint16_t*>(dy), dim, ld_dy,
-                           start, bucket, rows, chunks, static_cast<uint16_t*>(dw), ld_dw);
+                           start, bucket, rows, chunks, static_cast<uint16_t*>(dw), ld_dw, scale_by_freq);
     else
         hipLaunchKernelGGL((emb_bwd_reduce<float>), rgrid, dim3(kBlock), 0, s, static_cast<const float*>(dy), dim, ld_dy, start,
-                           bucket, rows, chunks, static_cast<float*>(dw), ld_dw);
+                           bucket, rows, chunks, static_cast<float*>(dw), ld_dw, scale_by_freq);
     return check_launch("embedding backward");
 }
 
@@ -319,8 +401,8 @@ int scratch_on_current_device(int32_t** out) {
 }  // namespace ddl
 
 extern "C" int ddl_embedding_backward_static(const void* dy, int dtype, int64_t dim, int64_t ld_dy, const void* ids, int ids_is_i64,
-                                             int64_t n_ids, int64_t lo, int64_t hi, int64_t padding_idx, void* dweight,
-                                             int64_t ld_dw, void* stream) {
+                                             int64_t n_ids, int64_t lo, int64_t hi, int64_t padding_idx, int scale_grad_by_freq,
+                                             void* dweight, int64_t ld_dw, void* stream) {
     using namespace ddl;
     if (n_ids < 0 || hi < lo) return fail(DDL_E_ARG, "embedding backward (static): n_ids=%lld window=[%lld,%lld)", (long long)n_ids, (long long)lo, (long long)hi);
     const int64_t rows = hi - lo;
@@ -334,13 +416,13 @@ extern "C" int ddl_embedding_backward_static(const void* dy, int dtype, int64_t 
     int32_t* ws = nullptr;
     const int rc = scratch_on_current_device(&ws);
     if (rc) return rc;
-    return ddl_embedding_backward(dy, dtype, dim, ld_dy, ids, ids_is_i64, n_ids, lo, hi, padding_idx, dweight, ld_dw, ws,
-                                  DDL_EMBEDDING_BACKWARD_STATIC_MAX_ELEMS, stream);
+    return ddl_embedding_backward(dy, dtype, dim, ld_dy, ids, ids_is_i64, n_ids, lo, hi, padding_idx, scale_grad_by_freq, dweight,
+                                  ld_dw, ws, DDL_EMBEDDING_BACKWARD_STATIC_MAX_ELEMS, stream);
 }
 
 extern "C" int ddl_embedding_backward(const void* dy, int dtype, int64_t dim, int64_t ld_dy, const void* ids, int ids_is_i64,
-                                      int64_t n_ids, int64_t lo, int64_t hi, int64_t padding_idx, void* dweight,
-                                      int64_t ld_dw, int32_t* workspace, int64_t workspace_elems, void* stream) {
+                                      int64_t n_ids, int64_t lo, int64_t hi, int64_t padding_idx, int scale_grad_by_freq,
+                                      void* dweight, int64_t ld_dw, int32_t* workspace, int64_t workspace_elems, void* stream) {
     using namespace ddl;
     if (dim < 0 || ld_dy < dim || ld_dw < dim || n_ids < 0 || hi < lo)
         return fail(DDL_E_ARG, "embedding backward: dim=%lld ld_dy=%lld ld_dw=%lld n_ids=%lld window=[%lld,%lld)", (long long)dim,
@@ -361,6 +443,8 @@ extern "C" int ddl_embedding_backward(const void* dy, int dtype, int64_t dim, in
     if (rows * chunks / kWavesPerBlock >= 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "embedding backward: too many workgroups");
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (ids_is_i64)
-        return run(dy, dtype, dim, ld_dy, static_cast<const int64_t*>(ids), n_ids, lo, hi, padding_idx, dweight, ld_dw, workspace, s);
-    return run(dy, dtype, dim, ld_dy, static_cast<const int32_t*>(ids), n_ids, lo, hi, padding_idx, dweight, ld_dw, workspace, s);
+        return run(dy, dtype, dim, ld_dy, static_cast<const int64_t*>(ids), n_ids, lo, hi, padding_idx, scale_grad_by_freq != 0, dweight,
+                   ld_dw, workspace, s);
+    return run(dy, dtype, dim, ld_dy, static_cast<const int32_t*>(ids), n_ids, lo, hi, padding_idx, scale_grad_by_freq != 0, dweight, ld_dw,
+               workspace, s);
 }

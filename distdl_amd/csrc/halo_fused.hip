@@ -817,8 +817,9 @@ __global__ __launch_bounds__(kBlock) void halo_flat_kernel(const HaloArgs args_b
     }
 }
 
-// Rows at least this long (shard elements) take halo_flat_kernel.
-int g_flat_min_row = 32;
+// Rows at least this long (shard elements) take halo_flat_kernel when the
+// caller leaves the choice to the library.
+constexpr int64_t kFlatMinRow = 32;
 
 template <typename T>
 int launch_halo(const HaloArgs& a, uint32_t lpr, hipStream_t s) {
@@ -835,17 +836,15 @@ int launch_halo(const HaloArgs& a, uint32_t lpr, hipStream_t s) {
 }  // namespace
 }  // namespace ddl
 
-extern "C" int ddl_halo_set_flat_min_row(int64_t elements) {
-    if (elements < 1) return ddl::fail(DDL_E_ARG, "halo: row threshold %lld below 1", (long long)elements);
-    ddl::g_flat_min_row = elements > 0x7FFFFFFFll ? 0x7FFFFFFF : static_cast<int>(elements);
-    return 0;
-}
-
 extern "C" int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x_shape, int ndim, int elem_size,
                                      const int64_t* pad, const int64_t* recv, const int64_t* send,
-                                     const void* const* ghost_bufs, void* const* bulk_bufs, void* stream) {
+                                     const void* const* ghost_bufs, void* const* bulk_bufs, int kernel, void* stream) {
     using namespace ddl;
     if (ndim < 1 || ndim > DDL_MAX_DIMS) return fail(DDL_E_DIMS, "halo: ndim %d outside [1,%d]", ndim, DDL_MAX_DIMS);
+    if (kernel != DDL_HALO_AUTO && kernel != DDL_HALO_ROWS && kernel != DDL_HALO_LINES)
+        return fail(DDL_E_ARG, "halo: kernel choice %d is not DDL_HALO_AUTO, _ROWS or _LINES", kernel);
+    // shortest shard row the whole-line kernel takes under this choice
+    const int64_t flat_min_row = kernel == DDL_HALO_ROWS ? INT64_MAX : kernel == DDL_HALO_LINES ? 1 : kFlatMinRow;
     if (!x_shape || !pad || !recv || !send) return fail(DDL_E_ARG, "halo: null geometry argument");
     if (elem_size != 1 && elem_size != 2 && elem_size != 4 && elem_size != 8)
         return fail(DDL_E_ARG, "halo: element size %d not in {1,2,4,8}", elem_size);
@@ -978,7 +977,7 @@ extern "C" int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x
     if (nplanes * static_cast<int64_t>(a.row_chunks) >= (1ll << 31)) return fail(DDL_E_UNSUPP, "halo: too many workgroups");
     a.nplanes = static_cast<uint32_t>(nplanes);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if ((es == 4 || es == 2) && total < (1ll << 31) && xs[L] >= g_flat_min_row && ps[L] >= kFlatMinPitch && aligned_to(xpad, 16)) {
+    if ((es == 4 || es == 2) && total < (1ll << 31) && xs[L] >= flat_min_row && ps[L] >= kFlatMinPitch && aligned_to(xpad, 16)) {
         const int64_t nstages = (total + kStage - 1) / kStage;
         FlatTop& t = a.top;
         t.x = a.x;

@@ -207,8 +207,10 @@ class HaloPadPlan:
                 shape.append(self.padded_shape[j] - self.recv[j][0] - self.recv[j][1])
         return tuple(shape)
 
-    def run(self, x, ghost_bufs, bulk_bufs, out=None):
-        """ghost_bufs / bulk_bufs: ``[ndim][2]`` nested lists of tensors or None."""
+    def run(self, x, ghost_bufs, bulk_bufs, out=None, kernel=_lib.DDL_HALO_AUTO):
+        """ghost_bufs / bulk_bufs: ``[ndim][2]`` nested lists of tensors or None.
+        ``kernel``: ``DDL_HALO_AUTO`` (library's choice), ``DDL_HALO_ROWS`` or
+        ``DDL_HALO_LINES``; the results are identical."""
         _require_gpu(x)
         if tuple(x.shape) != self.x_shape or not x.is_contiguous():
             raise ValueError("halo_pad_exchange: input must be contiguous with the planned shape")
@@ -232,16 +234,9 @@ class HaloPadPlan:
                     ptrs.append(buf.data_ptr())
         rc = _lib.load().ddl_halo_pad_exchange(x.data_ptr(), out.data_ptr(), self.shape_arr, self.ndim,
                                                x.element_size(), self.pad_arr, self.recv_arr, self.send_arr,
-                                               _lib.ptr_array(gptr), _lib.ptr_array(bptr), _stream())
+                                               _lib.ptr_array(gptr), _lib.ptr_array(bptr), int(kernel), _stream())
         _lib.check(rc, "ddl_halo_pad_exchange")
         return out
-
-
-def halo_set_flat_min_row(elements):
-    """Shard rows of at least ``elements`` 4-byte elements take the whole-line
-    kernel of ``ddl_halo_pad_exchange`` (library default 32); shorter rows are
-    written row by row.  Results are identical either way."""
-    _lib.check(_lib.load().ddl_halo_set_flat_min_row(int(elements)), "ddl_halo_set_flat_min_row")
 
 
 def ln_partial_stats(x2d, out=None):
@@ -398,8 +393,10 @@ def embedding_gather(weight, ids, lo, hi, out=None):
     return out
 
 
-def embedding_backward(grad_output, ids, lo, hi, padding_idx=None):
-    """Gradient of :func:`embedding_gather` with respect to the ``[hi-lo, dim]`` table."""
+def embedding_backward(grad_output, ids, lo, hi, padding_idx=None, scale_grad_by_freq=False):
+    """Gradient of :func:`embedding_gather` with respect to the ``[hi-lo, dim]``
+    table; with ``scale_grad_by_freq`` every row's sum is divided by the number
+    of tokens that looked the row up."""
     _require_gpu(grad_output, ids)
     if grad_output.dtype not in (torch.bfloat16, torch.float32):
         raise ValueError("embedding_backward: bfloat16 or float32 gradients only")
@@ -418,8 +415,8 @@ def embedding_backward(grad_output, ids, lo, hi, padding_idx=None):
     dt = _lib.DDL_DT_BF16 if grad_output.dtype == torch.bfloat16 else _lib.DDL_DT_F32
     rc = _lib.load().ddl_embedding_backward(dy.data_ptr(), dt, dim, dy.stride(0) if n_ids > 1 else dim, ids_c.data_ptr(),
                                             1 if ids.dtype == torch.int64 else 0, n_ids, int(lo), int(hi),
-                                            -1 if padding_idx is None else int(padding_idx), dw.data_ptr(), dim,
-                                            work.data_ptr(), work.numel(), _stream())
+                                            -1 if padding_idx is None else int(padding_idx), 1 if scale_grad_by_freq else 0,
+                                            dw.data_ptr(), dim, work.data_ptr(), work.numel(), _stream())
     _lib.check(rc, "ddl_embedding_backward")
     return dw
 

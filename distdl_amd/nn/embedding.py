@@ -9,6 +9,7 @@ extension for vocabulary-sharded tables: the local table then holds rows
 
 import torch
 
+from .. import config
 from .. import hip_ops
 from ..utilities.slicing import compute_subshape
 from ..utilities.slicing import worker_layout
@@ -23,26 +24,33 @@ class _EmbeddingShard(torch.autograd.Function):
     looked-up table row, the ``padding_idx`` row left at zero)."""
 
     @staticmethod
-    def forward(ctx, weight, ids, lo, hi, padding_idx=None):
+    def forward(ctx, weight, ids, lo, hi, padding_idx=None, scale_grad_by_freq=False):
         ctx.save_for_backward(ids)
-        ctx.window = (lo, hi, padding_idx)
+        ctx.window = (lo, hi, padding_idx, scale_grad_by_freq)
         return hip_ops.embedding_gather(weight.detach(), ids, lo, hi)
 
     @staticmethod
     def backward(ctx, grad_output):
         (ids,) = ctx.saved_tensors
-        lo, hi, padding_idx = ctx.window
-        dw = hip_ops.embedding_backward(grad_output.detach(), ids, lo, hi, padding_idx)
-        return dw, None, None, None, None
+        lo, hi, padding_idx, scale_grad_by_freq = ctx.window
+        dw = hip_ops.embedding_backward(grad_output.detach(), ids, lo, hi, padding_idx, scale_grad_by_freq)
+        return dw, None, None, None, None, None
 
 
 class DistributedEmbedding(Module):
     r"""Lookup table of ``num_embeddings`` vectors of size ``embedding_dim``
     whose last dimension is partitioned by the last dimension of ``P_x``.
 
-    Signature of the reference; ``max_norm`` (in-place renormalisation of the
-    table during the lookup) is refused, ``padding_idx``, ``scale_grad_by_freq``
-    and ``sparse`` only concern gradients and are stored.
+    Signature of the reference.  ``padding_idx`` and ``scale_grad_by_freq``
+    act on the gradient as they do in ``torch.nn.functional.embedding``;
+    ``max_norm`` (in-place renormalisation of the table during the lookup) and
+    ``sparse=True`` (a sparse gradient tensor) are refused.
+
+    Without ``vocab_shard`` every id must lie in ``[0, num_embeddings)``; the
+    kernel does not look (an id outside yields a zero row and no gradient).
+    ``distdl_amd.config.check_embedding_ids = True`` (environment
+    ``DISTDL_CHECK_EMBEDDING_IDS=1``) makes ``forward`` check the ids first and
+    raise ``IndexError``, at the price of a device synchronisation per call.
     """
 
     def __init__(self, P_x, num_embeddings, embedding_dim, padding_idx=None,
@@ -62,6 +70,9 @@ class DistributedEmbedding(Module):
             raise NotImplementedError("max_norm renormalises the table in place; not part of this build")
         if collect_state:
             raise NotImplementedError("collect_state=True is not part of this build")
+        if sparse:
+            raise NotImplementedError("sparse=True (a sparse gradient tensor) is not part of this build; "
+                                      "the gradient of the table is dense")
         self.padding_idx = padding_idx
         self.max_norm = max_norm
         self.norm_type = norm_type
@@ -136,4 +147,9 @@ class DistributedEmbedding(Module):
         else:
             weight = self.weight_buffer
             self.weight_buffer = None
-        return _EmbeddingShard.apply(weight, input, self.vocab_lo, self.vocab_hi, self.padding_idx)
+        if config.check_embedding_ids and input.numel() > 0:
+            lo, hi = (int(v) for v in torch.aminmax(input))
+            if lo < 0 or hi >= self.num_embeddings:
+                raise IndexError(f"token ids span [{lo}, {hi}], outside the table's [0, {self.num_embeddings})")
+        return _EmbeddingShard.apply(weight, input, self.vocab_lo, self.vocab_hi, self.padding_idx,
+                                     bool(self.scale_grad_by_freq))

@@ -1,7 +1,9 @@
 """ReduceScatter layer (reference: nn/reduce_scatter.py): sums the tensors of
 the workers that differ along ``axes_reduce_scatter`` and leaves every worker
-its balanced slab of the sum.  Under the solo transport the layer keeps the live
-worker's slab of its own tensor (the absent workers contribute nothing)."""
+its balanced slab of the sum.  Under the solo transport the absent workers
+hold what the live one holds unless a gather provider supplies their tensors, so
+without one the result is the live worker's slab of its own tensor times the
+number of workers."""
 
 import numpy as np
 

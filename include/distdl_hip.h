@@ -140,22 +140,26 @@ int ddl_zero_boxes(void* tensor, const int64_t* tensor_shape,
  * several dimensions takes the slab of the highest such dimension, and a bulk
  * slab of dimension i sees the ghosts of dimensions < i.
  * Only when every ghost slab is available before the call (one-GPU stub
- * exchange, or `ghost_bufs` all NULL for phase 0 of a real exchange). */
+ * exchange, or `ghost_bufs` all NULL for phase 0 of a real exchange).
+ *
+ * `kernel` chooses between the library's two implementations, whose results
+ * are identical (no counterpart in the reference; tests run every case on
+ * both).  DDL_HALO_AUTO: tensors of 2-, 4- or 8-byte elements whose shard rows
+ * hold at least 32 elements (8-byte ones count as two) are assembled through
+ * LDS and stored in whole 128-byte lines, everything else is written row by
+ * row.  DDL_HALO_LINES lowers that row threshold to 1, DDL_HALO_ROWS always
+ * writes row by row.  Whatever the choice, 1-byte elements, padded rows shorter
+ * than 32 elements, outputs not aligned to 16 bytes and tensors of 2^31
+ * elements or more are written row by row. */
+#define DDL_HALO_AUTO  0
+#define DDL_HALO_ROWS  1
+#define DDL_HALO_LINES 2
 int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x_shape,
                           int ndim, int elem_size,
                           const int64_t* pad, const int64_t* recv,
                           const int64_t* send,
                           const void* const* ghost_bufs, void* const* bulk_bufs,
-                          void* stream);
-
-/* Tuning knob of ddl_halo_pad_exchange (no counterpart in the reference):
- * tensors of 2-, 4- or 8-byte elements whose shard rows hold at least
- * `elements` elements (8-byte ones count as two) and whose padded rows hold at
- * least 32 are assembled through LDS and stored in whole 128-byte lines;
- * shorter rows, 1-byte elements, outputs not aligned to 16 bytes and tensors of
- * 2^31 elements or more are written row by row.  Both ways give identical
- * results.  Default 32.  Process-wide; not synchronised with concurrent calls. */
-int ddl_halo_set_flat_min_row(int64_t elements);
+                          int kernel, void* stream);
 
 /* ------------------------------------------------------------------------ *
  * DistributedLayerNorm local shard (fp32)
@@ -275,12 +279,17 @@ int ddl_embedding_gather(const void* weight, int64_t dim, int64_t ldw,
  * (what autograd derives for torch.nn.functional.embedding,
  * nn/embedding.py:244-246; padding_idx < 0 = none).  dtype = DDL_DT_BF16 or
  * DDL_DT_F32 for dy and dweight alike; sums are accumulated in fp32 in
- * ascending token order.  Every element of dweight is written, so it needs no
- * clearing.  `workspace`: device memory for at least 2 (hi-lo) + 1 + n_ids
- * int32, contents on entry do not matter. */
+ * ascending token order whatever the length of a row's token list, so the
+ * result is the same on every run.  With scale_grad_by_freq != 0 each row's
+ * sum is divided by the number of tokens that contributed to it
+ * (torch.nn.functional.embedding's option of that name, nn/embedding.py:244-246).
+ * Every element of dweight is written, so it needs no clearing.  `workspace`:
+ * device memory for at least 2 (hi-lo) + 1 + n_ids int32, contents on entry do
+ * not matter. */
 int ddl_embedding_backward(const void* dy, int dtype, int64_t dim, int64_t ld_dy,
                            const void* ids, int ids_is_i64, int64_t n_ids,
                            int64_t lo, int64_t hi, int64_t padding_idx,
+                           int scale_grad_by_freq,
                            void* dweight, int64_t ld_dw, int32_t* workspace,
                            int64_t workspace_elems, void* stream);
 
@@ -300,6 +309,7 @@ int ddl_embedding_backward(const void* dy, int dtype, int64_t dim, int64_t ld_dy
 int ddl_embedding_backward_static(const void* dy, int dtype, int64_t dim, int64_t ld_dy,
                                   const void* ids, int ids_is_i64, int64_t n_ids,
                                   int64_t lo, int64_t hi, int64_t padding_idx,
+                                  int scale_grad_by_freq,
                                   void* dweight, int64_t ld_dw, void* stream);
 
 /* ------------------------------------------------------------------------ *

@@ -25,17 +25,23 @@ def gather(table, ids, lo=0, hi=None):
     return out
 
 
-def backward(dy, ids, lo, hi, padding_idx=None, dtype=np.float64):
+def backward(dy, ids, lo, hi, padding_idx=None, dtype=np.float64, scale_grad_by_freq=False):
     """Adjoint of ``gather`` with respect to the table: row r of the result is
     the sum of dy[t] over the tokens with ids[t] - lo == r (tokens outside the
     window and tokens equal to padding_idx add nothing) -- the dense gradient
     of torch.nn.functional.embedding (reference call site nn/embedding.py:244-246).
     ``dy`` holds values (not bit patterns); sums are exact in ``dtype``.
+    With ``scale_grad_by_freq`` a row's sum is divided by the number of tokens
+    that contributed to it (the option of that name of the same torch call).
     Pinned by torch autograd on CPU in tests/test_oracle_golden.py."""
     ids = np.asarray(ids).reshape(-1)
     dy = np.asarray(dy, dtype=dtype).reshape(ids.size, -1)
     out = np.zeros((hi - lo, dy.shape[1]), dtype=dtype)
+    count = np.zeros(hi - lo, dtype=np.int64)
     for t, i in enumerate(ids):
         if lo <= i < hi and (padding_idx is None or i != padding_idx):
             out[i - lo] += dy[t]
+            count[i - lo] += 1
+    if scale_grad_by_freq:
+        out /= np.maximum(count, 1)[:, None]
     return out

@@ -90,13 +90,58 @@ def halo_path(request, ops):
     """The fused kernel has two ways of writing fp32 tensors (row by row, or in
     whole 128-byte lines through LDS); every fused case runs on both and on the
     library's own choice."""
-    if request.param != "default":
-        ops.halo_set_flat_min_row(1 << 40 if request.param == "rows" else 1)
-    yield request.param
-    ops.halo_set_flat_min_row(32)
+    from distdl_amd import _lib
+    return {"rows": _lib.DDL_HALO_ROWS, "lines": _lib.DDL_HALO_LINES, "default": _lib.DDL_HALO_AUTO}[request.param]
 
 
-def _fused_case(ops, x_shape, pad, recv, send, dtype, seed):
+_INT_VIEW = {2: torch.int16, 4: torch.int32, 8: torch.int64}
+_NP_INT = {2: np.int16, 4: np.int32, 8: np.int64}
+
+
+def _random_bits(shape, dtype, gen):
+    """Random BIT patterns of the dtype: NaN payloads, subnormals, signed zeros."""
+    es = torch.empty((), dtype=dtype).element_size()
+    raw = torch.randint(0, 256, tuple(shape) + (es,), dtype=torch.uint8, generator=gen)
+    return raw.view(dtype).reshape(tuple(shape))
+
+
+def _np_bits(t):
+    """The tensor's elements as NumPy integers of the same width (NaN == NaN under this view)."""
+    return t.contiguous().view(_INT_VIEW[t.element_size()]).cpu().numpy()
+
+
+def _fused_case_bits(ops, x_shape, pad, recv, send, dtype, seed, kernel):
+    """The same comparison as ``_fused_case`` on raw bit patterns: shard, ghost
+    slabs and results are compared as integers, so NaN payloads, negative
+    zeros and subnormals must come through both kernels unchanged (the oracle
+    only moves elements, so it runs on the integer view)."""
+    gen = torch.Generator().manual_seed(seed)
+    x = _random_bits(x_shape, dtype, gen)
+    plan = ops.HaloPadPlan(x_shape, pad, recv, send)
+    nd = len(x_shape)
+    ghosts_np, ghosts, bulks = [], [], []
+    for d in range(nd):
+        grow_n, grow, brow = [], [], []
+        for s in range(2):
+            gs, bs = plan.slab_shape(d, s, "ghost"), plan.slab_shape(d, s, "bulk")
+            gc = None if gs is None else _random_bits(gs, dtype, gen)
+            grow_n.append(None if gc is None else _np_bits(gc))
+            grow.append(None if gc is None else gc.cuda())
+            brow.append(None if bs is None else torch.full(bs, 7, dtype=dtype, device="cuda"))
+        ghosts_np.append(grow_n)
+        ghosts.append(grow)
+        bulks.append(brow)
+    out = plan.run(x.cuda(), ghosts, bulks, kernel=kernel)
+    torch.cuda.synchronize()
+    want, want_bulks = o_halo.pad_exchange_single(_np_bits(x), pad, recv, send, ghosts_np)
+    assert np.array_equal(_np_bits(out), want)
+    for d in range(nd):
+        for s in range(2):
+            if bulks[d][s] is not None:
+                assert np.array_equal(_np_bits(bulks[d][s]), want_bulks[d][s]), (d, s)
+
+
+def _fused_case(ops, x_shape, pad, recv, send, dtype, seed, kernel=0):
     gen = torch.Generator().manual_seed(seed)
     x = torch.randn(x_shape, generator=gen).to(dtype)
     plan = ops.HaloPadPlan(x_shape, pad, recv, send)
@@ -113,7 +158,7 @@ def _fused_case(ops, x_shape, pad, recv, send, dtype, seed):
         ghosts_cpu.append(grow_c)
         ghosts.append(grow)
         bulks.append(brow)
-    out = plan.run(x.cuda(), ghosts, bulks)
+    out = plan.run(x.cuda(), ghosts, bulks, kernel=kernel)
     torch.cuda.synchronize()
     np_dtype = {torch.float32: np.float32, torch.float64: np.float64, torch.float16: np.float16}[dtype]
     want, want_bulks = o_halo.pad_exchange_single(
@@ -130,47 +175,47 @@ def _fused_case(ops, x_shape, pad, recv, send, dtype, seed):
 def test_fused_halo_interior_rank_3d(ops, dtype, halo_path):
     # every side has a ghost and a bulk strip, widths differ per side
     _fused_case(ops, (2, 3, 9, 10, 70), [[0, 0], [0, 0], [1, 2], [2, 1], [1, 3]],
-                [[0, 0], [0, 0], [1, 2], [2, 1], [1, 3]], [[0, 0], [0, 0], [2, 1], [1, 2], [3, 1]], dtype, 51)
+                [[0, 0], [0, 0], [1, 2], [2, 1], [1, 3]], [[0, 0], [0, 0], [2, 1], [1, 2], [3, 1]], dtype, 51, halo_path)
 
 
 def test_fused_halo_corner_rank_with_explicit_padding(ops, halo_path):
     # rank 0 of a 2x2x2 split, kernel 3 / padding 1: left sides are zero padding, right sides ghosts
     _fused_case(ops, (1, 4, 16, 16, 16), [[0, 0], [0, 0], [1, 1], [1, 1], [1, 1]],
-                [[0, 0], [0, 0], [0, 1], [0, 1], [0, 1]], [[0, 0], [0, 0], [0, 1], [0, 1], [0, 1]], torch.float32, 52)
+                [[0, 0], [0, 0], [0, 1], [0, 1], [0, 1]], [[0, 0], [0, 0], [0, 1], [0, 1], [0, 1]], torch.float32, 52, halo_path)
 
 
 def test_fused_halo_long_rows_and_other_ranks(ops, halo_path):
     _fused_case(ops, (3, 5, 300), [[0, 0], [2, 2], [4, 4]], [[0, 0], [2, 2], [4, 0]], [[0, 0], [1, 2], [0, 3]],
-                torch.float32, 53)
-    _fused_case(ops, (40,), [[3, 2]], [[3, 2]], [[2, 3]], torch.float32, 54)
-    _fused_case(ops, (6, 20), [[0, 0], [0, 0]], [[0, 0], [0, 0]], [[0, 0], [0, 0]], torch.float32, 55)   # plain copy
+                torch.float32, 53, halo_path)
+    _fused_case(ops, (40,), [[3, 2]], [[3, 2]], [[2, 3]], torch.float32, 54, halo_path)
+    _fused_case(ops, (6, 20), [[0, 0], [0, 0]], [[0, 0], [0, 0]], [[0, 0], [0, 0]], torch.float32, 55, halo_path)   # plain copy
     _fused_case(ops, (4, 6, 20), [[1, 0], [0, 2], [3, 3]], [[0, 0], [0, 0], [0, 0]], [[0, 0], [0, 0], [0, 0]],
-                torch.float32, 56)                                                                        # F.pad only
+                torch.float32, 56, halo_path)                                                                        # F.pad only
 
 
 def test_fused_halo_wide_rows_geometries(ops, halo_path):
     # rows longer than a 1024-element piece; pieces that begin and end inside a row
     _fused_case(ops, (2, 3, 2500), [[0, 0], [1, 1], [2, 3]], [[0, 0], [1, 1], [2, 3]], [[0, 0], [1, 1], [3, 2]],
-                torch.float32, 57)
+                torch.float32, 57, halo_path)
     # padding wider than the ghosts on every side, missing neighbours on some sides
     _fused_case(ops, (2, 7, 9, 100), [[0, 0], [3, 2], [2, 3], [4, 5]], [[0, 0], [1, 0], [0, 2], [2, 0]],
-                [[0, 0], [2, 0], [0, 1], [1, 0]], torch.float32, 58)
+                [[0, 0], [2, 0], [0, 1], [1, 0]], torch.float32, 58, halo_path)
     # four exchanged dimensions, output volume not a multiple of four elements
     _fused_case(ops, (3, 5, 6, 33), [[1, 1], [1, 1], [1, 1], [1, 1]], [[1, 1], [1, 1], [1, 1], [1, 1]],
-                [[1, 1], [1, 1], [1, 1], [1, 1]], torch.float32, 59)
+                [[1, 1], [1, 1], [1, 1], [1, 1]], torch.float32, 59, halo_path)
     # 2-D and 1-D tensors with long rows, int32 payload of the same element size
-    _fused_case(ops, (5, 1030), [[2, 2], [1, 1]], [[2, 2], [1, 1]], [[2, 2], [1, 1]], torch.float32, 60)
-    _fused_case(ops, (4099,), [[3, 2]], [[3, 2]], [[2, 3]], torch.float32, 61)
+    _fused_case(ops, (5, 1030), [[2, 2], [1, 1]], [[2, 2], [1, 1]], [[2, 2], [1, 1]], torch.float32, 60, halo_path)
+    _fused_case(ops, (4099,), [[3, 2]], [[3, 2]], [[2, 3]], torch.float32, 61, halo_path)
     # ghost strips without bulk strips and the reverse
     _fused_case(ops, (2, 6, 40, 64), [[0, 0], [2, 2], [1, 1], [2, 2]], [[0, 0], [2, 2], [1, 1], [2, 2]],
-                [[0, 0], [0, 0], [0, 0], [0, 0]], torch.float32, 62)
+                [[0, 0], [0, 0], [0, 0], [0, 0]], torch.float32, 62, halo_path)
     _fused_case(ops, (2, 6, 40, 64), [[0, 0], [2, 2], [1, 1], [2, 2]], [[0, 0], [0, 0], [0, 0], [0, 0]],
-                [[0, 0], [2, 1], [1, 1], [1, 2]], torch.float32, 63)
+                [[0, 0], [2, 1], [1, 1], [1, 2]], torch.float32, 63, halo_path)
     # 2-byte elements: odd widths, pieces of 1024 elements that end inside a row, a volume that is not a multiple of 8
     _fused_case(ops, (3, 9, 131), [[0, 0], [1, 1], [1, 1]], [[0, 0], [1, 1], [1, 1]], [[0, 0], [1, 1], [1, 1]],
-                torch.float16, 64)
+                torch.float16, 64, halo_path)
     _fused_case(ops, (2, 3, 2500), [[0, 0], [1, 1], [2, 3]], [[0, 0], [1, 1], [2, 3]], [[0, 0], [1, 1], [3, 2]],
-                torch.float16, 65)
+                torch.float16, 65, halo_path)
 
 
 def test_fused_halo_random_geometries(ops, halo_path):
@@ -192,7 +237,38 @@ def test_fused_halo_random_geometries(ops, halo_path):
             recv.append(r)
             send.append(s_)
         dtype = (torch.float32, torch.float16, torch.float64)[case % 3]
-        _fused_case(ops, tuple(x_shape), pad, recv, send, dtype, 1000 + case)
+        _fused_case(ops, tuple(x_shape), pad, recv, send, dtype, 1000 + case, halo_path)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.float64])
+def test_fused_halo_moves_bit_patterns_unchanged(ops, dtype, halo_path):
+    """Random bit patterns (NaN payloads, -0, subnormals) through both kernels:
+    the 2-byte whole-line path widens elements on the way into LDS and packs them
+    on the way out, the 8-byte path moves pairs of words; neither may alter a bit."""
+    # interior rank, rows longer than a wavefront's piece and rows that end inside one
+    _fused_case_bits(ops, (2, 3, 9, 10, 70), [[0, 0], [0, 0], [1, 2], [2, 1], [1, 3]],
+                     [[0, 0], [0, 0], [1, 2], [2, 1], [1, 3]], [[0, 0], [0, 0], [2, 1], [1, 2], [3, 1]], dtype, 71, halo_path)
+    _fused_case_bits(ops, (2, 3, 2500), [[0, 0], [1, 1], [2, 3]], [[0, 0], [1, 1], [2, 3]], [[0, 0], [1, 1], [3, 2]],
+                     dtype, 72, halo_path)
+    # corner rank with explicit zero padding on the left sides, odd row length
+    _fused_case_bits(ops, (1, 4, 16, 16, 131), [[0, 0], [0, 0], [1, 1], [1, 1], [1, 1]],
+                     [[0, 0], [0, 0], [0, 1], [0, 1], [0, 1]], [[0, 0], [0, 0], [0, 1], [0, 1], [0, 1]], dtype, 73, halo_path)
+    # short rows (row kernel under every choice) and a 1-D tensor
+    _fused_case_bits(ops, (3, 5, 6, 12), [[1, 1], [1, 1], [1, 1], [1, 1]], [[1, 1], [1, 1], [1, 1], [1, 1]],
+                     [[1, 1], [1, 1], [1, 1], [1, 1]], dtype, 74, halo_path)
+    _fused_case_bits(ops, (4099,), [[3, 2]], [[3, 2]], [[2, 3]], dtype, 75, halo_path)
+
+
+def test_fused_halo_config5_interior_rank_full_size(ops):
+    """The shard of configuration 5 as an interior rank of a partition at least
+    three wide in every spatial dimension: six ghost and six bulk slabs
+    ([1,32,1,128,128], [1,32,130,1,128], [1,32,130,130,1] per side), bit-exact
+    against the oracle at full size."""
+    w = [[0, 0], [0, 0], [1, 1], [1, 1], [1, 1]]
+    plan = ops.HaloPadPlan((1, 32, 128, 128, 128), w, w, w)
+    assert plan.slab_shape(2, 0, "ghost") == (1, 32, 1, 128, 128) and plan.slab_shape(3, 1, "bulk") == (1, 32, 130, 1, 128)
+    assert plan.slab_shape(4, 0, "bulk") == (1, 32, 130, 130, 1)
+    _fused_case(ops, (1, 32, 128, 128, 128), w, w, w, torch.float32, 1105)
 
 
 def test_fused_halo_config5_rank0_bit_exact(ops, halo_path):
@@ -210,7 +286,7 @@ def test_fused_halo_config5_rank0_bit_exact(ops, halo_path):
     assert halo == [[0, 0], [0, 0], [0, 1], [0, 1], [0, 1]] and send == halo
     total = [[a + c, b + e] for (a, b), (c, e) in zip(lpad, halo)]
     assert total == [[0, 0], [0, 0], [1, 1], [1, 1], [1, 1]]
-    _fused_case(ops, (1, 32, 128, 128, 128), total, recv, send, torch.float32, 1005)
+    _fused_case(ops, (1, 32, 128, 128, 128), total, recv, send, torch.float32, 1005, halo_path)
 
 
 # ------------------------------------------------------- conv, end to end --

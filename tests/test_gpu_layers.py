@@ -115,7 +115,14 @@ def test_layernorm_layer_matches_torch(golden):
     from distdl_amd.backends.stub_hip import SimWorld
     from distdl_amd.nn import DistributedLayerNorm
     torch.manual_seed(0)
-    for geom in golden("layer_geometries.json")["layernorm"]:
+    # the reference's geometries (all with equal shard widths), then geometries whose normalised dimensions do not
+    # divide evenly among the workers, which the reference never tests
+    uneven = [{"P_x_shape": [1, 1, 3], "input_shape": [2, 5, 10], "normalized_shape": [10]},
+              {"P_x_shape": [2, 1, 2], "input_shape": [5, 3, 7], "normalized_shape": [3, 7]},
+              {"P_x_shape": [1, 2, 2], "input_shape": [3, 5, 9], "normalized_shape": [5, 9]},
+              {"P_x_shape": [2, 3], "input_shape": [6, 301], "normalized_shape": [301]}]
+    seen_uneven = 0
+    for geom in golden("layer_geometries.json")["layernorm"] + uneven:
         P, shape, norm = geom["P_x_shape"], geom["input_shape"], geom["normalized_shape"]
         nn_ = len(norm)
         x = torch.rand(shape)
@@ -147,11 +154,22 @@ def test_layernorm_layer_matches_torch(golden):
             want = F.layer_norm(x, tuple(norm), gamma, beta, 1e-5).numpy()
             parts = o_rep.scatter(want, P)
         else:
-            # unequal widths: the reference is the mean of local statistics, restated by the oracle
-            parts = None
-        if parts is not None:
-            for got, part in zip(outs, parts):
-                assert np.allclose(got, part, rtol=1e-4, atol=1e-5), geom     # reference tolerance is atol sqrt(1e-7)
+            # unequal widths: the reference is the mean of local statistics (not the layer norm of the whole
+            # row), restated by the oracle over each group of workers that share rows
+            seen_uneven += 1
+            parts = [None] * n
+            lead_shape, red_shape = tuple(P[:len(P) - nn_]), tuple(P[-nn_:])
+            n_red = int(np.prod(red_shape))
+            for lead in np.ndindex(*lead_shape) if lead_shape else [()]:
+                group = [int(np.ravel_multi_index(tuple(lead) + tuple(r), tuple(P))) for r in np.ndindex(*red_shape)]
+                res = o_ln.forward_shards([xs[r] for r in group], [gs[k] for k in range(n_red)],
+                                          [bs[k] for k in range(n_red)], 1e-5, num_norm_dims=nn_, dtype=np.float64)
+                for r, y in zip(group, res):
+                    parts[r] = y
+        for got, part in zip(outs, parts):
+            assert got.shape == part.shape, geom
+            assert np.allclose(got, part, rtol=1e-4, atol=1e-5), geom     # reference tolerance is atol sqrt(1e-7)
+    assert seen_uneven == len(uneven)
 
 
 @pytest.mark.parametrize("cols", [[256, 256, 256, 256], [64, 64], [300, 212], [7, 9], [2048], [5000, 40], [4] * 70])
@@ -388,6 +406,85 @@ def test_embedding_backward_matches_torch_autograd_on_random_data(ops):
     tw = table.float().requires_grad_(True)
     F.embedding(ids, tw).backward(dy.float())
     assert np.allclose(got, tw.grad.double().numpy(), rtol=2.0 ** -7, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_embedding_backward_long_buckets_are_summed_in_token_order(ops, dtype):
+    """Rows looked up 65 to several thousand times with random float gradients:
+    the sums run in ascending token order whatever order the bucket fill
+    produced, so the result equals a sequential fp32 sum in token order bit for
+    bit, and is the same on every run.  One row exceeds what the sort holds in
+    LDS (8192 tokens) and is sorted in global memory."""
+    gen = torch.Generator().manual_seed(31)
+    rows, dim, tokens = 12, 72, 30000
+    # row 0: about 12000 tokens, row 1: about 6000, rows 2..: 65 and more, row 11: rare
+    weights = torch.tensor([12000, 6000, 3000, 2000, 1500, 1200, 1000, 800, 600, 500, 300, 5], dtype=torch.float)
+    ids = torch.multinomial(weights, tokens, replacement=True, generator=gen) + 4
+    dy = torch.randn(tokens, dim, generator=gen).to(dtype)
+    counts = torch.bincount(ids - 4, minlength=rows)
+    assert int(counts[0]) > 8192 and int((counts > 64).sum()) >= 10
+    first = ops.embedding_backward(dy.cuda(), ids.cuda(), 4, 4 + rows).cpu()
+    want = torch.zeros(rows, dim, dtype=torch.float32)
+    dy32 = dy.float()
+    for r in range(rows):
+        acc = torch.zeros(dim, dtype=torch.float32)
+        for t in torch.nonzero(ids == r + 4).flatten().tolist():       # ascending token order, fp32, one add at a time
+            acc += dy32[t]
+        want[r] = acc
+    assert torch.equal(first, want.to(dtype))
+    for _ in range(3):
+        again = ops.embedding_backward(dy.cuda(), ids.cuda(), 4, 4 + rows).cpu()
+        assert torch.equal(again.view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                           first.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_embedding_backward_scale_grad_by_freq(ops, dtype):
+    """Each row's sum divided by its number of contributing tokens, against the
+    oracle (pinned to torch autograd) and through the layer's autograd path."""
+    from distdl_amd.nn.embedding import _EmbeddingShard
+    gen = torch.Generator().manual_seed(32)
+    ids = torch.randint(0, 40, (6, 50), generator=gen)
+    dy = torch.randn(6, 50, 96, generator=gen).to(dtype)
+    got = ops.embedding_backward(dy.cuda(), ids.cuda(), 5, 30, padding_idx=7, scale_grad_by_freq=True)
+    want = o_emb.backward(dy.double().numpy(), ids.numpy(), 5, 30, padding_idx=7, scale_grad_by_freq=True)
+    tol = 2.0 ** -7 if dtype == torch.bfloat16 else 1e-5
+    assert (np.abs(got.cpu().double().numpy() - want) <= tol * np.abs(want) + 1e-6).all()
+    w = torch.zeros(25, 96, dtype=dtype, device="cuda", requires_grad=True)
+    _EmbeddingShard.apply(w, ids.cuda(), 5, 30, 7, True).backward(dy.cuda())
+    assert torch.equal(w.grad, got)
+    plain = ops.embedding_backward(dy.cuda(), ids.cuda(), 5, 30, padding_idx=7)
+    assert not torch.equal(plain, got)
+
+
+def test_embedding_layer_options(ops):
+    """sparse=True is refused; the id check raises on ids outside the table when switched on."""
+    from distdl_amd import config
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedEmbedding
+
+    def body(P_world):
+        P_x = P_world.create_partition_inclusive([0]).create_cartesian_topology_partition([1, 1, 1])
+        with pytest.raises(NotImplementedError):
+            DistributedEmbedding(P_x, 10, 8, sparse=True)
+        layer = DistributedEmbedding(P_x, 10, 8, scale_grad_by_freq=True)
+        ids = torch.tensor([[1, 1, 1, 2]], device="cuda")
+        out = layer(ids)
+        out.sum().backward()
+        g = layer.weight.grad.cpu()
+        assert torch.allclose(g[1], torch.ones(8)) and torch.allclose(g[2], torch.ones(8)) and float(g[0].abs().sum()) == 0
+        bad = torch.tensor([[1, 10]], device="cuda")
+        assert float(layer(bad).detach()[0, 1].abs().sum()) == 0          # unchecked: a zero row
+        config.check_embedding_ids = True
+        try:
+            with pytest.raises(IndexError):
+                layer(bad)
+            layer(ids)
+        finally:
+            config.check_embedding_ids = False
+        return True
+
+    assert SimWorld(1).run(body) == [True]
 
 
 def test_embedding_backward_config3_rank0(ops):

@@ -411,3 +411,9 @@ def test_embedding_backward_oracle_matches_torch_autograd():
     # a window: exactly the rows [lo, hi) of the full gradient (padding row excluded as above)
     full = o_emb.backward(dy.numpy(), ids.numpy(), 0, 20)
     assert np.array_equal(o_emb.backward(dy.numpy(), ids.numpy(), 5, 12), full[5:12])
+    # scale_grad_by_freq: torch divides each row's gradient by the row's number of occurrences in the batch
+    table2 = table.detach().clone().requires_grad_(True)
+    F.embedding(ids, table2, padding_idx=3, scale_grad_by_freq=True).backward(dy)
+    got = o_emb.backward(dy.numpy(), ids.numpy(), 0, 20, padding_idx=3, scale_grad_by_freq=True)
+    assert np.allclose(got, table2.grad.numpy(), rtol=1e-13, atol=1e-13)
+    assert not np.allclose(got, table.grad.numpy())      # the option changes the answer on this input

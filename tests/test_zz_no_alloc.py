@@ -34,11 +34,11 @@ def _both(lib, dy, ids, lo, hi, padding_idx):
     work = torch.full((2 * rows + 1 + n,), -1, dtype=torch.int32, device="cuda")
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
-    rc = lib.ddl_embedding_backward_static(dy.data_ptr(), dt, dim, dim, ids.data_ptr(), i64, n, lo, hi, padding_idx,
+    rc = lib.ddl_embedding_backward_static(dy.data_ptr(), dt, dim, dim, ids.data_ptr(), i64, n, lo, hi, padding_idx, 0,
                                            got.data_ptr(), dim, _stream())
     _lib.check(rc, "ddl_embedding_backward_static")
     assert torch.cuda.memory_allocated() == before
-    rc = lib.ddl_embedding_backward(dy.data_ptr(), dt, dim, dim, ids.data_ptr(), i64, n, lo, hi, padding_idx,
+    rc = lib.ddl_embedding_backward(dy.data_ptr(), dt, dim, dim, ids.data_ptr(), i64, n, lo, hi, padding_idx, 0,
                                     ref.data_ptr(), dim, work.data_ptr(), work.numel(), _stream())
     _lib.check(rc, "ddl_embedding_backward")
     torch.cuda.synchronize()
@@ -88,11 +88,11 @@ def test_static_entry_rejects_sizes_beyond_the_built_in_workspace():
     ids = torch.zeros(8, dtype=torch.int64, device="cuda")
     dw = torch.zeros(8, 8, device="cuda")
     # the size test comes before any pointer is used: n_ids alone exceeds the capacity
-    rc = lib.ddl_embedding_backward_static(dy.data_ptr(), _lib.DDL_DT_F32, 8, 8, ids.data_ptr(), 1, cap, 0, 8, -1,
+    rc = lib.ddl_embedding_backward_static(dy.data_ptr(), _lib.DDL_DT_F32, 8, 8, ids.data_ptr(), 1, cap, 0, 8, -1, 0,
                                            dw.data_ptr(), 8, _stream())
     assert rc == -5
     assert b"exceeds the built-in workspace" in lib.ddl_last_error()
-    rc = lib.ddl_embedding_backward_static(dy.data_ptr(), _lib.DDL_DT_F32, 8, 8, ids.data_ptr(), 1, 8, 0, cap // 2, -1,
+    rc = lib.ddl_embedding_backward_static(dy.data_ptr(), _lib.DDL_DT_F32, 8, 8, ids.data_ptr(), 1, 8, 0, cap // 2, -1, 0,
                                            dw.data_ptr(), 8, _stream())
     assert rc == -5
     torch.cuda.synchronize()
