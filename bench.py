@@ -1,28 +1,40 @@
 """Benchmark of the per-rank hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--only NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--skip-layers] [--only NAMES]
 
 Headline workload (BASELINE.json configs[1]): Repartition pack + unpack of one
 rank, bf16 global tensor [8,4096,8192] moved from P_x=[1,8,1] to P_y=[1,1,8].
 One step = one pack launch (the [8,512,8192] shard into eight [8,512,1024]
 boxes) + one unpack launch (eight seeded boxes into the [8,4096,1024] output
-shard) = 268 435 456 algorithmic bytes.  Inputs are resident in HBM before the
-timed region; the step rotates over several buffer sets so that the 256 MB
-last-level cache cannot hold the working set.  The other hot-path kernels
-(LayerNorm, Embedding, Linear GEMM, fused halo staging) are measured the same
-way and reported under "workloads" of the same JSON line.
+shard) = 268 435 456 algorithmic bytes.  The box lists come from the product's
+own planner (distdl_amd.nn.Repartition's set-up on rank 0 of 8) and are
+asserted equal to the oracle's before anything is timed.  Inputs are resident
+in HBM before the timed region; a step rotates over several buffer sets so that
+the 256 MB last-level cache cannot hold the working set.  The other hot-path
+kernels (LayerNorm, Embedding, Linear GEMM, halo staging) are measured the same
+way and reported under "workloads" of the same JSON line, each with
+
+  roofline      algorithmic work / HIP-event time of the step's launches
+  layer         microseconds per forward call of the distdl_amd.nn module that
+                wraps the kernel (host path included), next to the kernel time
+  cpu_baseline  the oracle's CPU restatement of the reference path, timed on a
+                bounded sample in this same run
 
 Timing: the launches of the timed region are captured once into a HIP graph
 (no host work between kernels) and replayed; wall clock with a device
 synchronisation on both sides gives ms_per_step, HIP events on the launch
 stream give the per-launch kernel duration used for the roofline.  If graph
 capture is unavailable the same launches are issued directly on the stream.
+The headline runs exactly --steps steps; the other workloads run at least 100
+steps after at least 20 warm-ups, whatever --steps says, because the GEMM's
+clock needs that many samples to settle.
 """
 
 import argparse
 import ctypes
 import json
 import os
+import re
 import sys
 import time
 
@@ -32,21 +44,24 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+MIN_SECONDARY_STEPS, MIN_SECONDARY_WARMUP = 100, 20
 
-# HBM bytes per launch (read + write) from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs of these same workloads, each counter scaled by what it reads
-# for a plain 64 MiB device copy (FETCH_SIZE x1.9993, WRITE_SIZE x1.0000); the
-# summaries are profiles/*_hbm_traffic_pmc.txt.  layernorm is the mean of its two
-# kernels (stats 8 482 132 B, normalize 17 875 667 B), like its launch time;
-# linear is the sum of the two launches of a step (256-wide tiles 436 344 160 B,
-# 192-wide tiles 398 065 226 B).
-MEASURED_TRAFFIC_BYTES = {
-    "repartition": 134414634,
-    "layernorm": 13178900,
-    "embedding": 1210721771,
-    "linear": 834409386,
-    "halo": 568008812,
-}
+
+def profile_traffic(name, combine):
+    """HBM bytes per launch of a workload, as measured with rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE (each counter scaled by what it reads for a plain
+    copy of known size) and written down in profiles/<name>_hbm_traffic_pmc.txt:
+    one "traffic (read + write) = N B" line per kernel of a step.  These are not
+    measured by the run that prints them; None when there is no such summary."""
+    path = os.path.join(ROOT, "profiles", f"{name}_hbm_traffic_pmc.txt")
+    try:
+        with open(path) as f:
+            values = [int(v) for v in re.findall(r"traffic \(read \+ write\) = (\d+) B", f.read())]
+    except OSError:
+        return None
+    if not values:
+        return None
+    return sum(values) / len(values) if combine == "mean" else sum(values)
 
 
 def parse_args():
@@ -54,8 +69,9 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default=None, help="run only these workloads, comma-separated (repartition, layernorm, layernorm_long, embedding, linear, halo, layernorm_bwd, embedding_bwd, linear_bwd, calib)")
+    ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--skip-layers", action="store_true", help="skip the module-level (host path included) timings")
+    ap.add_argument("--only", default=None, help="run only these workloads, comma-separated; see WORKLOADS")
     ap.add_argument("--no-graph", action="store_true", help="launch on the stream instead of replaying a HIP graph")
     return ap.parse_args()
 
@@ -140,16 +156,78 @@ def measure(torch, name, step_fns, launches_per_step, steps, warmup, use_graph):
             "launch_s": ev / (n * launches_per_step)}
 
 
+def _call(lib, _lib, name, args):
+    def fn(a=args, f=getattr(lib, name), n=name):
+        rc = f(*a, STREAM[0])
+        if rc:
+            _lib.check(rc, n)
+    return fn
+
+
+def time_layer(torch, fn, calls=200, warm=10):
+    """Microseconds per call of a module's forward: the host loop alone, and
+    with the device drained at the end (the larger of the two is what a caller
+    sees per call in steady state)."""
+    with torch.no_grad():
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(calls):
+            fn()
+        t1 = time.perf_counter()
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+    return {"host_us_per_call": 1e6 * (t1 - t0) / calls, "us_per_call": 1e6 * (t2 - t0) / calls, "calls": calls}
+
+
+def timed_cpu(fn, budget_s):
+    """Runs fn() (one sample) until about budget_s seconds are spent; returns
+    (runs, seconds), after one untimed run."""
+    fn()
+    n, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        n += 1
+        dt = time.perf_counter() - t0
+        if dt >= budget_s:
+            return n, dt
+
+
 # ----------------------------------------------------------------------------
-# workloads
+# configuration 2: Repartition (headline)
 # ----------------------------------------------------------------------------
 
+def repartition_layer(torch):
+    """The product's Repartition for configuration 2 on rank 0 of 8, set up
+    for the [8,512,8192] bf16 shard: (layer, x)."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import Repartition
+    world = SimWorld(8)
+    base = world.partition(0).create_partition_inclusive(list(range(8)))
+    P_x = base.create_cartesian_topology_partition([1, 8, 1])
+    P_y = base.create_cartesian_topology_partition([1, 1, 8])
+    layer = Repartition(P_x, P_y)
+    gen = torch.Generator().manual_seed(1002)
+    x = (2 * torch.rand(8, 512, 8192, generator=gen) - 1).to(torch.bfloat16).cuda()
+    layer._distdl_forward_pre_hook(layer, (x,))       # what torch calls in front of forward
+    return layer, x
+
+
 def build_repartition(torch, lib, _lib, nsets):
-    """Config 2.  Returns (step closures per set, bytes per step, description)."""
+    """Config 2.  Box lists from the product's planner, checked against the oracle's."""
     from oracle import repartition as o_rep
-    send, recv, _, _ = o_rep.plan([8, 4096, 8192], [1, 8, 1], [1, 1, 8])
-    send0 = [sl for sl, sh, p in send[0]]
-    recv0 = [sl for sl, sh, p in recv[0]]
+    layer, x0 = repartition_layer(torch)
+    send0 = [tuple(sl) for sl, sh, p in layer.P_x_to_y_overlaps]
+    recv0 = [tuple(sl) for sl, sh, p in layer.P_y_to_x_overlaps]
+    o_send, o_recv, _, _ = o_rep.plan([8, 4096, 8192], [1, 8, 1], [1, 1, 8])
+
+    def norm(slices):
+        return [tuple((int(s.start), int(s.stop)) for s in sl) for sl in slices]
+    assert norm(send0) == norm([sl for sl, sh, p in o_send[0]]), "planner and oracle disagree on the send boxes"
+    assert norm(recv0) == norm([sl for sl, sh, p in o_recv[0]]), "planner and oracle disagree on the receive boxes"
+    assert tuple(layer.output_tensor_structure.shape) == (8, 4096, 1024)
+    del x0
     keep, steps = [], []
     for s in range(nsets):
         gen = torch.Generator().manual_seed(1002 + s)
@@ -167,52 +245,84 @@ def build_repartition(torch, lib, _lib, nsets):
                        _lib.i64_array([int(sl_d.stop - sl_d.start) for sl in recv0 for sl_d in sl]),
                        _lib.ptr_array([b.data_ptr() for b in rbufs]), 0, 0)
         keep.append((x, sbufs, rbufs, y, pack_args, unpack_args))
-
-        def pack(a=pack_args):
-            rc = lib.ddl_pack_boxes(*a, STREAM[0])
-            if rc:
-                _lib.check(rc, "ddl_pack_boxes")
-
-        def unpack(a=unpack_args):
-            rc = lib.ddl_unpack_boxes(*a, STREAM[0])
-            if rc:
-                _lib.check(rc, "ddl_unpack_boxes")
-        steps.append([pack, unpack])
+        steps.append([_call(lib, _lib, "ddl_pack_boxes", pack_args), _call(lib, _lib, "ddl_unpack_boxes", unpack_args)])
     return steps, keep, 268435456
 
 
-def build_layernorm(torch, lib, _lib, nsets):
-    """Config 1: rank 0's [16,512,256] fp32 shard; stats + normalize."""
+def layer_repartition(torch):
+    layer, x = repartition_layer(torch)
+    rec = time_layer(torch, lambda: layer(x))
+    rec["module"] = ("Repartition(P_x=[1,8,1], P_y=[1,1,8]).forward under no_grad, rank 0 of 8, solo transport "
+                     "(one launch for 7 packs + the self copy, one for 7 unpacks)")
+    return rec
+
+
+def cpu_repartition(budget_s=12.0):
+    """One rank's pack + unpack of config 2 with the oracle's NumPy code
+    (np.copyto per box, zero-filled output), single thread, uint16 views of the
+    bf16 payload."""
+    import numpy as np
+    from oracle import repartition as o_rep
+    send, recv, _, _ = o_rep.plan([8, 4096, 8192], [1, 8, 1], [1, 1, 8])
+    send0 = [(sl, sh, 99 if p == "self" else p) for sl, sh, p in send[0]]
+    recv0 = [(sl, sh, 99 if p == "self" else p) for sl, sh, p in recv[0]]
+    rng = np.random.default_rng(1002)
+    x = rng.integers(0, 2 ** 16, size=(8, 512, 8192), dtype=np.uint16)
+    rbufs = [rng.integers(0, 2 ** 16, size=(8, 512, 1024), dtype=np.uint16) for _ in range(8)]
+
+    def step():
+        o_rep.pack(x, send0)
+        o_rep.unpack(recv0, rbufs, (8, 4096, 1024), np.uint16)
+    n, dt = timed_cpu(step, budget_s)
+    return {"value": 268435456 * n / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{n} full steps of config 2 (pack 8 boxes + zero-filled unpack of 8 boxes), "
+                      f"NumPy np.copyto on uint16 views, one process standing in for rank 0, {dt:.1f} s"}
+
+
+# ----------------------------------------------------------------------------
+# configuration 1: LayerNorm
+# ----------------------------------------------------------------------------
+
+def _ln_steps(torch, lib, _lib, nsets, rows, cols, seed, peers_from_global):
     import numpy as np
     from oracle import layernorm as o_ln
-    rows, cols = 16 * 512, 256
     keep, steps = [], []
-    part_cols = _lib.i64_array([256] * 4)
+    part_cols = _lib.i64_array([cols] * 4)
     for s in range(nsets):
-        gen = torch.Generator().manual_seed(1001 + s)
-        xg = torch.randn(16, 512, 1024, generator=gen)
-        gamma = (1 + 0.1 * torch.randn(1024, generator=gen))[:256].contiguous().cuda()
-        beta = (0.1 * torch.randn(1024, generator=gen))[:256].contiguous().cuda()
-        x = xg[..., :256].contiguous().cuda()
-        gathered = torch.empty(4, rows, 2, device="cuda")
-        for p in range(1, 4):   # peers' partial statistics: seeded, computed on the CPU from the same global x
-            gathered[p] = torch.from_numpy(o_ln.partial_stats(xg[..., 256 * p:256 * (p + 1)].numpy()).astype(np.float32))
+        if peers_from_global:
+            gen = torch.Generator().manual_seed(seed + s)
+            xg = torch.randn(16, 512, 4 * cols, generator=gen)
+            gamma = (1 + 0.1 * torch.randn(4 * cols, generator=gen))[:cols].contiguous().cuda()
+            beta = (0.1 * torch.randn(4 * cols, generator=gen))[:cols].contiguous().cuda()
+            x = xg[..., :cols].contiguous().cuda().reshape(rows, cols)
+            gathered = torch.empty(4, rows, 2, device="cuda")
+            for p in range(1, 4):   # peers' partial statistics: seeded, computed on the CPU from the same global x
+                gathered[p] = torch.from_numpy(o_ln.partial_stats(xg[..., cols * p:cols * (p + 1)].numpy()).astype(np.float32))
+        else:
+            gen = torch.Generator(device="cuda").manual_seed(seed + s)
+            x = torch.randn(rows, cols, generator=gen, device="cuda")
+            gamma = 1 + 0.1 * torch.randn(cols, generator=gen, device="cuda")
+            beta = 0.1 * torch.randn(cols, generator=gen, device="cuda")
+            gathered = torch.zeros(4, rows, 2, device="cuda")
+            gathered[1:, :, 1] = float(cols)                             # peers: mean 0, M2 = n (unit variance)
         y = torch.empty_like(x)
         stats_args = (x.data_ptr(), rows, cols, cols, gathered.data_ptr())      # own partials land in slot 0
         norm_args = (x.data_ptr(), rows, cols, cols, gathered.data_ptr(), 4, part_cols, gamma.data_ptr(),
                      beta.data_ptr(), 1e-5, y.data_ptr(), cols, None, None)
         keep.append((x, gamma, beta, gathered, y, stats_args, norm_args))
+        steps.append([_call(lib, _lib, "ddl_ln_partial_stats_f32", stats_args),
+                      _call(lib, _lib, "ddl_ln_normalize_affine_f32", norm_args)])
+    return steps, keep
 
-        def stats(a=stats_args):
-            rc = lib.ddl_ln_partial_stats_f32(*a, STREAM[0])
-            if rc:
-                _lib.check(rc, "ddl_ln_partial_stats_f32")
 
-        def norm(a=norm_args):
-            rc = lib.ddl_ln_normalize_affine_f32(*a, STREAM[0])
-            if rc:
-                _lib.check(rc, "ddl_ln_normalize_affine_f32")
-        steps.append([stats, norm])
+def ln_bytes(rows, cols, nparts=4):
+    # x read by both kernels, y written once, gamma and beta, own statistics written and all nparts read back
+    return 3 * rows * cols * 4 + 2 * cols * 4 + rows * 8 + nparts * rows * 8
+
+
+def build_layernorm(torch, lib, _lib, nsets):
+    """Config 1: rank 0's [16,512,256] fp32 shard; stats + normalize."""
+    steps, keep = _ln_steps(torch, lib, _lib, nsets, 16 * 512, 256, 1001, True)
     return steps, keep, 25298944
 
 
@@ -220,34 +330,97 @@ def build_layernorm_long(torch, lib, _lib, nsets):
     """The kernels of config 1 on 32 times its rows ([262144, 256] fp32, 268 MB):
     the streaming rate of the same code once launch ramp and memory latency no
     longer dominate.  Not a BASELINE configuration; reported next to config 1."""
-    rows, cols = 32 * 16 * 512, 256
+    steps, keep = _ln_steps(torch, lib, _lib, nsets, 32 * 16 * 512, 256, 2001, False)
+    return steps, keep, 32 * 25298944 - 31 * 2 * 256 * 4
+
+
+def build_layernorm_wide(torch, lib, _lib, nsets):
+    """Rows longer than a wavefront keeps in registers: [4096, 8192] fp32
+    (128 MiB), one workgroup per row.  Not a BASELINE configuration."""
+    rows, cols = 4096, 8192
+    steps, keep = _ln_steps(torch, lib, _lib, nsets, rows, cols, 2101, False)
+    return steps, keep, ln_bytes(rows, cols)
+
+
+def build_layernorm_local(torch, lib, _lib, nsets):
+    """The single-launch kernel for rows one worker holds whole (the reference's
+    F.layer_norm branch): the global rows of config 1, [8192, 1024] fp32."""
+    rows, cols = 16 * 512, 1024
     keep, steps = [], []
-    part_cols = _lib.i64_array([256] * 4)
     for s in range(nsets):
-        gen = torch.Generator(device="cuda").manual_seed(2001 + s)
+        gen = torch.Generator(device="cuda").manual_seed(2201 + s)
         x = torch.randn(rows, cols, generator=gen, device="cuda")
         gamma = 1 + 0.1 * torch.randn(cols, generator=gen, device="cuda")
         beta = 0.1 * torch.randn(cols, generator=gen, device="cuda")
-        gathered = torch.zeros(4, rows, 2, device="cuda")
-        gathered[1:, :, 1] = 256.0                                   # peers: mean 0, M2 = n (unit variance)
         y = torch.empty_like(x)
-        stats_args = (x.data_ptr(), rows, cols, cols, gathered.data_ptr())
-        norm_args = (x.data_ptr(), rows, cols, cols, gathered.data_ptr(), 4, part_cols, gamma.data_ptr(),
-                     beta.data_ptr(), 1e-5, y.data_ptr(), cols, None, None)
-        keep.append((x, gamma, beta, gathered, y, stats_args, norm_args))
+        args = (x.data_ptr(), _lib.DDL_DT_F32, rows, cols, cols, gamma.data_ptr(), beta.data_ptr(), 1e-5, y.data_ptr(),
+                cols, None, None)
+        keep.append((x, gamma, beta, y, args))
+        steps.append([_call(lib, _lib, "ddl_layer_norm", args)])
+    return steps, keep, 2 * rows * cols * 4 + 2 * cols * 4
 
-        def stats(a=stats_args):
-            rc = lib.ddl_ln_partial_stats_f32(*a, STREAM[0])
-            if rc:
-                _lib.check(rc, "ddl_ln_partial_stats_f32")
 
-        def norm(a=norm_args):
-            rc = lib.ddl_ln_normalize_affine_f32(*a, STREAM[0])
-            if rc:
-                _lib.check(rc, "ddl_ln_normalize_affine_f32")
-        steps.append([stats, norm])
-    return steps, keep, 32 * 25298944 - 31 * 2 * 256 * 4
+def layer_layernorm(torch):
+    import numpy as np
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedLayerNorm
+    from distdl_amd.nn.layernorm import STATS_TAG
+    from oracle import layernorm as o_ln
+    world = SimWorld(4)
+    P_x = world.partition(0).create_partition_inclusive(list(range(4))).create_cartesian_topology_partition([1, 1, 4])
+    layer = DistributedLayerNorm(P_x, [1024])
+    gen = torch.Generator().manual_seed(1001)
+    xg = torch.randn(16, 512, 1024, generator=gen)
+    x = xg[..., :256].contiguous().cuda()
+    peers = [None] + [torch.from_numpy(o_ln.partial_stats(xg[..., 256 * p:256 * (p + 1)].numpy()).astype(np.float32)).cuda()
+                      for p in range(1, 4)]
+    world.transport.set_gather_provider(STATS_TAG, lambda P, t: list(peers))
+    rec = time_layer(torch, lambda: layer(x))
+    rec["module"] = "DistributedLayerNorm(P_x=[1,1,4], 1024).forward under no_grad, rank 0 of 4, peers' statistics seeded"
+    xr = x.clone().requires_grad_(True)
+    grad = time_layer_grad(torch, lambda: layer(xr))
+    rec["host_us_per_call_grad_mode"] = grad["host_us_per_call"]
+    rec["us_per_call_grad_mode"] = grad["us_per_call"]
+    return rec
 
+
+def time_layer_grad(torch, fn, calls=200, warm=10):
+    """time_layer with autograd recording (the forward of a training step)."""
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(calls):
+        fn()
+    t1 = time.perf_counter()
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    return {"host_us_per_call": 1e6 * (t1 - t0) / calls, "us_per_call": 1e6 * (t2 - t0) / calls, "calls": calls}
+
+
+def cpu_layernorm(budget_s=4.0):
+    """Rank 0's share of the reference's op sequence (local mean, all-reduce,
+    local mean of squared deviations, all-reduce, normalise, affine) in NumPy
+    fp32, the all-reduces replaced by adding the seeded sums of ranks 1-3."""
+    import numpy as np
+    from oracle import layernorm as o_ln
+    rng = np.random.default_rng(1001)
+    xg = rng.standard_normal((16, 512, 1024), dtype=np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(256)).astype(np.float32)
+    beta = (0.1 * rng.standard_normal(256)).astype(np.float32)
+    x = np.ascontiguousarray(xg[..., :256])
+    mean = xg.mean(axis=-1, keepdims=True)
+    peer_mean = sum(xg[..., 256 * p:256 * (p + 1)].mean(axis=-1, keepdims=True) for p in range(1, 4))
+    peer_var = sum(((xg[..., 256 * p:256 * (p + 1)] - mean) ** 2).mean(axis=-1, keepdims=True) for p in range(1, 4))
+    n, dt = timed_cpu(lambda: o_ln.forward_rank(x, peer_mean, peer_var, 4, gamma, beta, 1e-5), budget_s)
+    return {"value": 25298944 * n / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{n} full steps of config 1 on rank 0 ([16,512,256] fp32): the reference's op sequence in NumPy fp32, "
+                      f"all-reduces replaced by seeded sums of the three peers, {dt:.1f} s"}
+
+
+# ----------------------------------------------------------------------------
+# configuration 3: Embedding
+# ----------------------------------------------------------------------------
 
 def build_embedding(torch, lib, _lib, nsets):
     """Config 3: rank-0 vocabulary shard [16032,4096] bf16, ids [32,4096] int64."""
@@ -263,79 +436,267 @@ def build_embedding(torch, lib, _lib, nsets):
         out = torch.empty(32, 4096, 4096, dtype=torch.bfloat16, device="cuda")
         args = (table.data_ptr(), 4096, 4096, 2, ids.data_ptr(), 1, ids.numel(), 0, 16032, out.data_ptr())
         keep.append((ids, out, args))
-
-        def gather(a=args):
-            rc = lib.ddl_embedding_gather(*a, STREAM[0])
-            if rc:
-                _lib.check(rc, "ddl_embedding_gather")
-        steps.append([gather])
+        steps.append([_call(lib, _lib, "ddl_embedding_gather", args)])
     return steps, keep, sum(nbytes) / len(nbytes)
+
+
+def layer_embedding(torch):
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedEmbedding
+    world = SimWorld(1)
+    P_x = world.partition(0).create_partition_inclusive([0]).create_cartesian_topology_partition([1, 1, 1])
+    layer = DistributedEmbedding(P_x, 128256, 4096, dtype=torch.bfloat16, vocab_shard=(0, 16032))
+    ids = torch.randint(0, 128256, (32, 4096), generator=torch.Generator().manual_seed(2003)).cuda()
+    rec = time_layer(torch, lambda: layer(ids), calls=50, warm=5)
+    rec["module"] = "DistributedEmbedding(128256, 4096, bf16, vocab_shard=(0,16032)).forward under no_grad, ids [32,4096]"
+    return rec
+
+
+def cpu_embedding(budget_s=4.0):
+    """The oracle's gather (NumPy row indexing, zero rows outside the window) on
+    the first 4096 tokens of config 3 against the full rank-0 shard."""
+    import numpy as np
+    from oracle import embedding as o_emb
+    rng = np.random.default_rng(1003)
+    table = rng.integers(0, 2 ** 16, size=(16032, 4096), dtype=np.uint16)
+    ids = rng.integers(0, 128256, size=(4096,), dtype=np.int64)
+    n_hit = int((ids < 16032).sum())
+    nbytes = ids.size * 4096 * 2 + ids.size * 8 + n_hit * 8192
+    n, dt = timed_cpu(lambda: o_emb.gather(table, ids, 0, 16032), budget_s)
+    return {"value": nbytes * n / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{n} gathers of 4096 of config 3's 131072 tokens (1/32 of a step) from the [16032,4096] shard, "
+                      f"NumPy indexing on uint16 views, {dt:.1f} s"}
+
+
+# ----------------------------------------------------------------------------
+# configuration 4: Linear
+# ----------------------------------------------------------------------------
+
+def _linear_operands(torch, nsets):
+    gen = torch.Generator().manual_seed(1004)
+    w = (0.02 * torch.randn(3584, 8192, generator=gen)).to(torch.bfloat16).cuda()
+    b = (0.02 * torch.randn(3584, generator=gen)).to(torch.bfloat16).cuda()
+    xs = []
+    for s in range(nsets):
+        gen = torch.Generator().manual_seed(3004 + s)
+        xs.append(torch.randn(4, 2048, 8192, generator=gen).to(torch.bfloat16).cuda())
+    return w, b, xs
 
 
 def build_linear(torch, lib, _lib, nsets):
     """Config 4: M=8192 N=3584 K=8192 bf16, fp32 accumulate, bias."""
-    gen = torch.Generator().manual_seed(1004)
-    w = (0.02 * torch.randn(3584, 8192, generator=gen)).to(torch.bfloat16).cuda()
-    b = (0.02 * torch.randn(3584, generator=gen)).to(torch.bfloat16).cuda()
+    w, b, xs = _linear_operands(torch, nsets)
     keep, steps = [w, b], []
-    for s in range(nsets):
-        gen = torch.Generator().manual_seed(3004 + s)
-        x = torch.randn(4, 2048, 8192, generator=gen).to(torch.bfloat16).cuda()
+    for x in xs:
         y = torch.empty(4, 2048, 3584, dtype=torch.bfloat16, device="cuda")
         args = (x.data_ptr(), w.data_ptr(), b.data_ptr(), y.data_ptr(), 8192, 3584, 8192, 8192, 8192, 3584)
         keep.append((x, y, args))
+        steps.append([_call(lib, _lib, "ddl_linear_bf16", args)])
+    return steps, keep, 2 * 8192 * 3584 * 8192
 
-        def gemm(a=args):
-            rc = lib.ddl_linear_bf16(*a, STREAM[0])
-            if rc:
-                _lib.check(rc, "ddl_linear_bf16")
+
+def build_linear_library(torch, lib, _lib, nsets):
+    """The same product on the same operands through torch.nn.functional.linear
+    (the vendor GEMM library): the comparison figure for the hand-written
+    kernel, not a product path."""
+    w, b, xs = _linear_operands(torch, nsets)
+    keep, steps = [w, b], []
+    for x in xs:
+        keep.append(x)
+
+        def gemm(x=x):
+            torch.nn.functional.linear(x, w, b)     # result dropped: its block is reused by the next call
         steps.append([gemm])
     return steps, keep, 2 * 8192 * 3584 * 8192
 
 
-def build_halo(torch, lib, _lib, nsets):
-    """Config 5 (fused): rank 0 of a 2x2x2 split, [1,32,128^3] fp32 -> [1,32,130^3]."""
+def layer_linear(torch):
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedLinearAllGather
+    world = SimWorld(8)
+    P_y = world.partition(0).create_partition_inclusive(list(range(8))).create_cartesian_topology_partition([1, 1, 8])
+    layer = DistributedLinearAllGather(P_y, 8192, 28672, dtype=torch.bfloat16)
+    x = torch.randn(4, 2048, 8192, generator=torch.Generator().manual_seed(3004)).to(torch.bfloat16).cuda()
+    rec = time_layer(torch, lambda: layer(x), calls=50, warm=5)
+    rec["module"] = ("DistributedLinearAllGather(P_y=[1,1,8], 8192, 28672, bf16).forward under no_grad, rank 0 of 8, "
+                     "x [4,2048,8192] whole on every worker")
+    return rec
+
+
+def cpu_linear(budget_s=4.0):
+    """The oracle's product (NumPy matmul on fp32 operands converted from the
+    same bf16 bits beforehand, bias added) on 256 of config 4's 8192 rows."""
+    import numpy as np
+    from oracle import linear as o_lin
+    rng = np.random.default_rng(1004)
+    m = 256
+    x = o_lin.bf16_bits_to_f32(o_lin.f32_to_bf16_bits(rng.standard_normal((m, 8192), dtype=np.float32)))
+    w = o_lin.bf16_bits_to_f32(o_lin.f32_to_bf16_bits(0.02 * rng.standard_normal((3584, 8192), dtype=np.float32)))
+    b = o_lin.bf16_bits_to_f32(o_lin.f32_to_bf16_bits(0.02 * rng.standard_normal(3584, dtype=np.float32)))
+    n, dt = timed_cpu(lambda: o_lin.linear_values(x, w, b), budget_s)
+    threads = 1
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([int(p.get("num_threads", 1)) for p in threadpool_info() if p.get("user_api") == "blas"] or [1])
+    except Exception:
+        pass
+    return {"value": 2.0 * m * 3584 * 8192 * n / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"{n} products of 256 of config 4's 8192 rows (1/32 of a step) with the [3584,8192] weight shard, NumPy "
+                      f"fp32 matmul (BLAS, {threads} threads) on operands converted from bf16 beforehand, {dt:.1f} s"}
+
+
+# ----------------------------------------------------------------------------
+# configuration 5: halo
+# ----------------------------------------------------------------------------
+
+RANK0 = [[0, 0], [0, 0], [0, 1], [0, 1], [0, 1]]        # corner rank of 2x2x2: right-hand neighbours only
+INTERIOR = [[0, 0], [0, 0], [1, 1], [1, 1], [1, 1]]     # interior rank of a partition at least 3 wide
+PAD5 = [[0, 0], [0, 0], [1, 1], [1, 1], [1, 1]]
+
+
+def _halo_sets(torch, nsets, widths, seed, padded_input=False):
     from distdl_amd import hip_ops
-    pad = [[0, 0], [0, 0], [1, 1], [1, 1], [1, 1]]
-    rs = [[0, 0], [0, 0], [0, 1], [0, 1], [0, 1]]
-    plan = hip_ops.HaloPadPlan((1, 32, 128, 128, 128), pad, rs, rs)
-    keep, steps = [], []
+    plan = hip_ops.HaloPadPlan((1, 32, 128, 128, 128), PAD5, widths, widths)
+    sets = []
     for s in range(nsets):
-        gen = torch.Generator().manual_seed(1005 + s)
-        x = torch.randn(1, 32, 128, 128, 128, generator=gen).cuda()
-        out = torch.empty(plan.padded_shape, device="cuda")
-        gptr, bptr, bufs = [], [], []
+        gen = torch.Generator(device="cuda").manual_seed(seed + s)
+        shape = plan.padded_shape if padded_input else (1, 32, 128, 128, 128)
+        x = torch.randn(shape, generator=gen, device="cuda")
+        ghosts, bulks = [], []
         for d in range(5):
+            grow, brow = [], []
             for side in range(2):
                 gs, bs = plan.slab_shape(d, side, "ghost"), plan.slab_shape(d, side, "bulk")
-                g = None if gs is None else torch.randn(gs, generator=gen).cuda()
-                b = None if bs is None else torch.empty(bs, device="cuda")
-                bufs += [g, b]
-                gptr.append(None if g is None else g.data_ptr())
-                bptr.append(None if b is None else b.data_ptr())
+                grow.append(None if gs is None else torch.randn(gs, generator=gen, device="cuda"))
+                brow.append(None if bs is None else torch.empty(bs, device="cuda"))
+            ghosts.append(grow)
+            bulks.append(brow)
+        sets.append((x, ghosts, bulks))
+    return plan, sets
+
+
+def _slab_bytes(plan, kind):
+    total = 0
+    for d in range(5):
+        for side in range(2):
+            shape = plan.slab_shape(d, side, kind)
+            if shape is not None:
+                n = 4
+                for v in shape:
+                    n *= v
+                total += n
+    return total
+
+
+def _build_halo_fused(torch, lib, _lib, nsets, widths, seed):
+    plan, sets = _halo_sets(torch, nsets, widths, seed)
+    keep, steps = [], []
+    for x, ghosts, bulks in sets:
+        out = torch.empty(plan.padded_shape, device="cuda")
+        gptr = [None if g is None else g.data_ptr() for row in ghosts for g in row]
+        bptr = [None if b is None else b.data_ptr() for row in bulks for b in row]
         args = (x.data_ptr(), out.data_ptr(), plan.shape_arr, 5, 4, plan.pad_arr, plan.recv_arr, plan.send_arr,
                 _lib.ptr_array(gptr), _lib.ptr_array(bptr), _lib.DDL_HALO_AUTO)
-        keep.append((x, out, bufs, args))
+        keep.append((x, out, ghosts, bulks, args))
+        steps.append([_call(lib, _lib, "ddl_halo_pad_exchange", args)])
+    work = 268435456 + 281216000 + _slab_bytes(plan, "ghost") + _slab_bytes(plan, "bulk")
+    return steps, keep, work
 
-        def fused(a=args):
-            rc = lib.ddl_halo_pad_exchange(*a, STREAM[0])
-            if rc:
-                _lib.check(rc, "ddl_halo_pad_exchange")
-        steps.append([fused])
-    return steps, keep, 562531072
+
+def build_halo(torch, lib, _lib, nsets):
+    """Config 5 (fused): rank 0 of a 2x2x2 split, [1,32,128^3] fp32 -> [1,32,130^3], 3 + 3 slabs."""
+    steps, keep, work = _build_halo_fused(torch, lib, _lib, nsets, RANK0, 1005)
+    assert work == 562531072
+    return steps, keep, work
+
+
+def build_halo_interior(torch, lib, _lib, nsets):
+    """The same shard as an interior rank: 6 ghost + 6 bulk slabs in the same single pass."""
+    return _build_halo_fused(torch, lib, _lib, nsets, INTERIOR, 1205)
+
+
+def _build_halo_slabs(torch, lib, _lib, nsets, widths, seed):
+    """Slab-only exchange on an existing padded tensor, in the reference's
+    order: per exchanged dimension one pack launch (bulk slabs of both sides)
+    and one unpack launch (ghost slabs of both sides)."""
+    from oracle import halo as o_halo
+    plan, sets = _halo_sets(torch, nsets, widths, seed, padded_input=True)
+    slices = o_halo.slab_slices(plan.padded_shape, widths, widths)
+    keep, steps = [], []
+    launches = 0
+    for xp, ghosts, bulks in sets:
+        fns = []
+        shape_arr, stride_arr = _lib.i64_array(xp.shape), _lib.i64_array(xp.stride())
+        for d in range(5):
+            lbs, lgs, rbs, rgs = slices[d]
+            packs = [(sl, bulks[d][side]) for side, sl in ((0, lbs), (1, rbs)) if bulks[d][side] is not None]
+            unpacks = [(sl, ghosts[d][side]) for side, sl in ((0, lgs), (1, rgs)) if ghosts[d][side] is not None]
+            for name, boxes, extra in (("ddl_pack_boxes", packs, ()), ("ddl_unpack_boxes", unpacks, (0, 0))):
+                if not boxes:
+                    continue
+                starts = _lib.i64_array([int(s.start) for sl, _ in boxes for s in sl])
+                shapes = _lib.i64_array([int(s.stop - s.start) for sl, _ in boxes for s in sl])
+                ptrs = _lib.ptr_array([b.data_ptr() for _, b in boxes])
+                args = (xp.data_ptr(), shape_arr, stride_arr, 5, 4, len(boxes), starts, shapes, ptrs) + extra
+                keep.append(args)
+                fns.append(_call(lib, _lib, name, args))
+        keep.append((xp, ghosts, bulks))
+        launches = len(fns)
+        steps.append(fns)
+    work = 2 * (_slab_bytes(plan, "ghost") + _slab_bytes(plan, "bulk"))
+    return steps, keep, work, launches
+
+
+def build_halo_slabs(torch, lib, _lib, nsets):
+    """Config 5, slab-only part: 3 bulk slabs packed, 3 ghost slabs unpacked (25 759 232 B in six launches)."""
+    steps, keep, work, launches = _build_halo_slabs(torch, lib, _lib, nsets, RANK0, 1305)
+    assert work == 25759232 and launches == 6, (work, launches)
+    return steps, keep, work
+
+
+def build_halo_slabs_interior(torch, lib, _lib, nsets):
+    """Slab-only exchange of an interior rank: 6 + 6 slabs (51 122 176 B in six launches)."""
+    steps, keep, work, launches = _build_halo_slabs(torch, lib, _lib, nsets, INTERIOR, 1405)
+    assert work == 51122176 and launches == 6, (work, launches)
+    return steps, keep, work
+
+
+def layer_halo(torch):
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedConv3d
+    world = SimWorld(8)
+    P_x = world.partition(0).create_partition_inclusive(list(range(8))).create_cartesian_topology_partition([1, 1, 2, 2, 2])
+    layer = DistributedConv3d(P_x, in_channels=32, out_channels=4, kernel_size=3, padding=1, bias=False)
+    x = torch.randn(1, 32, 128, 128, 128, generator=torch.Generator(device="cuda").manual_seed(1005), device="cuda")
+    layer._distdl_forward_pre_hook(layer, (x,))
+    rec = time_layer(torch, lambda: layer.stage_input(x), calls=50, warm=5)
+    rec["module"] = ("DistributedConv3d(P_x=[1,1,2,2,2], kernel 3, padding 1).stage_input under no_grad, rank 0 of 8 "
+                     "(pad + exchange + crop in front of the stock convolution)")
+    return rec
+
+
+def cpu_halo(budget_s=4.0):
+    """The oracle's np.pad + per-dimension slab pack / ghost unpack on the full
+    rank-0 shard of config 5."""
+    import numpy as np
+    from oracle import halo as o_halo
+    rng = np.random.default_rng(1005)
+    x = rng.standard_normal((1, 32, 128, 128, 128), dtype=np.float32)
+    shape = [1, 32, 130, 130, 130]
+    slices = o_halo.slab_slices(shape, RANK0, RANK0)
+    ghosts = []
+    for d in range(5):
+        lbs, lgs, rbs, rgs = slices[d]
+        ghosts.append([None, rng.standard_normal([s.stop - s.start for s in rgs], dtype=np.float32) if RANK0[d][1] else None])
+    n, dt = timed_cpu(lambda: o_halo.pad_exchange_single(x, PAD5, RANK0, RANK0, ghosts), budget_s)
+    return {"value": 562531072 * n / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{n} full steps of config 5 on rank 0 ([1,32,128^3] fp32, 3 + 3 slabs): np.pad, then per dimension "
+                      f"pack the bulk slabs and unpack the ghost slabs, NumPy, {dt:.1f} s"}
 
 
 # ----------------------------------------------------------------------------
 # backward (adjoint) workloads: the same shapes as the forward configurations
 # ----------------------------------------------------------------------------
-
-def _call(lib, _lib, name, args):
-    def fn(a=args, f=getattr(lib, name), n=name):
-        rc = f(*a, STREAM[0])
-        if rc:
-            _lib.check(rc, n)
-    return fn
-
 
 def build_layernorm_bwd(torch, lib, _lib, nsets):
     """Backward of config 1 on rank 0 as the layer runs it when every gradient
@@ -420,6 +781,10 @@ def build_linear_bwd(torch, lib, _lib, nsets):
     return steps, keep, 2 * 2 * M * N * K
 
 
+# ----------------------------------------------------------------------------
+# measurement aids
+# ----------------------------------------------------------------------------
+
 def build_calib(torch, lib, _lib, nsets):
     """Counter calibration: a plain contiguous device-to-device copy of 64 MiB
     (torch's own copy kernel), so that FETCH_SIZE / WRITE_SIZE readings of the
@@ -437,38 +802,55 @@ def build_calib(torch, lib, _lib, nsets):
     return steps, keep, 2 * (64 << 20)
 
 
-# ----------------------------------------------------------------------------
-# CPU baseline (the oracle, i.e. a port of the reference's mpi_numpy path)
-# ----------------------------------------------------------------------------
-
-def cpu_baseline_repartition(budget_s=12.0):
-    """One rank's pack + unpack of config 2 with the oracle's NumPy code
-    (np.copyto per box, zero-filled output), single thread, int16 views of the
-    bf16 payload.  Runs whole steps until about `budget_s` seconds are spent."""
-    import numpy as np
-    from oracle import repartition as o_rep
-    send, recv, _, _ = o_rep.plan([8, 4096, 8192], [1, 8, 1], [1, 1, 8])
-    send0 = [(sl, sh, 99 if p == "self" else p) for sl, sh, p in send[0]]
-    recv0 = [(sl, sh, 99 if p == "self" else p) for sl, sh, p in recv[0]]
-    rng = np.random.default_rng(1002)
-    x = rng.integers(0, 2 ** 16, size=(8, 512, 8192), dtype=np.uint16)
-    rbufs = [rng.integers(0, 2 ** 16, size=(8, 512, 1024), dtype=np.uint16) for _ in range(8)]
-    o_rep.pack(x, send0)
-    o_rep.unpack(recv0, rbufs, (8, 4096, 1024), np.uint16)
-    n, t0 = 0, time.perf_counter()
-    while True:
-        o_rep.pack(x, send0)
-        o_rep.unpack(recv0, rbufs, (8, 4096, 1024), np.uint16)
-        n += 1
-        dt = time.perf_counter() - t0
-        if dt >= budget_s:
-            break
-    return {"value": 268435456 * n / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{n} full steps of config 2 (pack 8 boxes + zero-filled unpack of 8 boxes), "
-                      f"NumPy np.copyto on uint16 views, one process standing in for rank 0, {dt:.1f} s"}
+def build_launch_floor(torch, lib, _lib, nsets):
+    """A kernel that does nothing, launched with the grid of config 1's
+    LayerNorm kernels (2048 workgroups of 256 threads) and replayed from the
+    same kind of graph: the time a launch costs on its own.  `work` is zero
+    bytes; only the time per launch means anything."""
+    steps = [[_call(lib, _lib, "ddl_probe_launch", (2048, 256)), _call(lib, _lib, "ddl_probe_launch", (2048, 256))]
+             for _ in range(nsets)]
+    return steps, [], 0
 
 
-# ----------------------------------------------------------------------------
+# name -> (builder, buffer sets, launches per step, bound, rule for combining the traffic figures of a step's kernels,
+#          layer timer, cpu baseline, BASELINE.json configuration number)
+WORKLOADS = {
+    "repartition": (build_repartition, 8, 2, "hbm", "mean", layer_repartition, cpu_repartition, 2),
+    "layernorm": (build_layernorm, 64, 2, "hbm", "mean", layer_layernorm, cpu_layernorm, 1),
+    "layernorm_long": (build_layernorm_long, 3, 2, "hbm", None, None, None, None),
+    "layernorm_wide": (build_layernorm_wide, 4, 2, "hbm", None, None, None, None),
+    "layernorm_local": (build_layernorm_local, 16, 1, "hbm", None, None, None, None),
+    "embedding": (build_embedding, 4, 1, "hbm", "sum", layer_embedding, cpu_embedding, 3),
+    "linear": (build_linear, 4, 1, "mfma", "sum", layer_linear, cpu_linear, 4),
+    "halo": (build_halo, 4, 1, "hbm", "sum", layer_halo, cpu_halo, 5),
+    "halo_interior": (build_halo_interior, 4, 1, "hbm", None, None, None, None),
+    "halo_slabs": (build_halo_slabs, 8, 6, "hbm", None, None, None, None),
+    "halo_slabs_interior": (build_halo_slabs_interior, 8, 6, "hbm", None, None, None, None),
+    "layernorm_bwd": (build_layernorm_bwd, 32, 2, "hbm", None, None, None, None),
+    "embedding_bwd": (build_embedding_bwd, 4, 1, "hbm", None, None, None, None),
+    "linear_bwd": (build_linear_bwd, 2, 1, "mfma", None, None, None, None),
+    "launch_floor": (build_launch_floor, 8, 2, "hbm", None, None, None, None),
+    # only with --only:
+    "linear_library": (build_linear_library, 4, 1, "mfma", None, None, None, None),
+    "calib": (build_calib, 4, 1, "hbm", None, None, None, None),
+}
+ONLY_ON_REQUEST = ("linear_library", "calib")
+
+
+def cpu_host():
+    import torch
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"nproc": os.cpu_count(), "affinity": len(os.sched_getaffinity(0)), "torch_threads": torch.get_num_threads(),
+            "cpu_model": model, "launch": "single process standing in for rank 0 (no mpirun: mpi4py is not installed)"}
+
 
 def main():
     args = parse_args()
@@ -487,28 +869,19 @@ def main():
     lib = _lib.load()
     use_graph = not args.no_graph
 
-    builders = {
-        "repartition": (build_repartition, 8, 2, "hbm"),
-        "layernorm": (build_layernorm, 64, 2, "hbm"),
-        "layernorm_long": (build_layernorm_long, 3, 2, "hbm"),
-        "embedding": (build_embedding, 4, 1, "hbm"),
-        "linear": (build_linear, 4, 1, "mfma"),
-        "halo": (build_halo, 4, 1, "hbm"),
-        "layernorm_bwd": (build_layernorm_bwd, 32, 2, "hbm"),
-        "embedding_bwd": (build_embedding_bwd, 4, 1, "hbm"),
-        "linear_bwd": (build_linear_bwd, 2, 1, "mfma"),
-        "calib": (build_calib, 4, 1, "hbm"),     # only with --only calib
-    }
-    names = [n.strip() for n in args.only.split(",")] if args.only else [n for n in builders if n != "calib"]
+    names = [n.strip() for n in args.only.split(",")] if args.only else [n for n in WORKLOADS if n not in ONLY_ON_REQUEST]
     for n in names:
-        if n not in builders:
-            raise SystemExit(f"bench.py: unknown workload {n!r}; choose from {', '.join(builders)}")
+        if n not in WORKLOADS:
+            raise SystemExit(f"bench.py: unknown workload {n!r}; choose from {', '.join(WORKLOADS)}")
+    head_name = "repartition" if "repartition" in names else names[0]
     results = {}
     for name in names:
-        build, nsets, launches, bound = builders[name]
+        build, nsets, launches, bound, combine, layer_fn, cpu_fn, config = WORKLOADS[name]
         step_fns, keep, work = build(torch, lib, _lib, nsets)
-        steps = args.steps if name in ("repartition", "layernorm") else max(8, args.steps // 4)
-        warm = args.warmup if name in ("repartition", "layernorm") else max(4, args.warmup // 4)
+        if name == head_name:
+            steps, warm = args.steps, args.warmup
+        else:
+            steps, warm = max(args.steps, MIN_SECONDARY_STEPS), max(args.warmup, MIN_SECONDARY_WARMUP)
         m = measure(torch, name, step_fns, launches, steps, warm, use_graph)
         per_launch = work / launches
         if bound == "hbm":
@@ -517,32 +890,45 @@ def main():
         else:
             achieved, peak, unit = per_launch / m["launch_s"] / 1e12, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
             value = work * m["steps"] / m["wall_s"] / 1e12
+        traffic = profile_traffic(name, combine) if combine else None
         results[name] = {
-            "value": value, "unit": unit, "steps": m["steps"], "ms_per_step": 1e3 * m["wall_s"] / m["steps"],
-            "mode": m["mode"], "work_per_step": work,
+            "value": value, "unit": unit, "steps": m["steps"], "warmup": warm, "ms_per_step": 1e3 * m["wall_s"] / m["steps"],
+            "mode": m["mode"], "work_per_step": work, "launches_per_step": launches, "us_per_launch": 1e6 * m["launch_s"],
+            "baseline_config": config,
             "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
-                         "traffic": MEASURED_TRAFFIC_BYTES.get(name)},
+                         "traffic": traffic,
+                         "traffic_source": f"profiles/{name}_hbm_traffic_pmc.txt (earlier rocprofv3 --pmc runs, not this run)"
+                         if traffic is not None else None},
         }
         del step_fns, keep
         torch.cuda.empty_cache()
+        if layer_fn is not None and not args.skip_layers:
+            rec = layer_fn(torch)
+            rec["kernel_us_per_step"] = 1e6 * m["launch_s"] * launches
+            results[name]["layer"] = rec
+            torch.cuda.empty_cache()
+        if cpu_fn is not None and not args.skip_cpu:
+            results[name]["cpu_baseline"] = cpu_fn()
 
-    head_name = "repartition" if "repartition" in results else names[0]
     head = results[head_name]
     line = {
         "metric": "Repartition pack+unpack GB/s (rank 0, bf16 [8,4096,8192], P_x=[1,8,1] -> P_y=[1,1,8])"
         if head_name == "repartition" else head_name,
-        "value": head["value"], "unit": head["unit"], "n_gpus": 1, "steps": head["steps"], "warmup": args.warmup,
+        "value": head["value"], "unit": head["unit"], "n_gpus": 1, "steps": head["steps"], "warmup": head["warmup"],
         "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u16" if head_name == "repartition" else "mixed", "data": "synthetic",
         "config": {"workload": "BASELINE.json configs[1]: Repartition pack/unpack bf16, rank 0 of 8, "
                                "pack [8,512,8192] -> 8x[8,512,1024], unpack 8x[8,512,1024] -> [8,4096,1024]"
                    if head_name == "repartition" else head_name,
-                   "launch_mode": head["mode"], "buffer_sets": builders[head_name][1]},
+                   "launch_mode": head["mode"], "buffer_sets": WORKLOADS[head_name][1],
+                   "box_lists": "distdl_amd.nn.Repartition set-up (rank 0 of 8), asserted equal to the oracle's plan"},
         "roofline": head["roofline"],
         "workloads": results,
     }
+    if "cpu_baseline" in head:
+        line["cpu_baseline"] = head["cpu_baseline"]
     if not args.skip_cpu:
-        line["cpu_baseline"] = cpu_baseline_repartition()
+        line["cpu_host"] = cpu_host()
     print(json.dumps(line))
 
 

@@ -14,6 +14,15 @@ import torch
 from . import device as _device
 
 
+# Number of times any buffer has been reallocated.  Whoever caches device
+# addresses of buffer views compares this against the value it saw.
+_reallocations = 0
+
+
+def reallocations():
+    return _reallocations
+
+
 class ExpandableBuffer:
 
     def __init__(self, dtype, initial_capacity=0, device=None):
@@ -27,7 +36,9 @@ class ExpandableBuffer:
         new_capacity = int(new_capacity)
         if new_capacity <= self.capacity:
             return
-        grown = torch.empty(new_capacity, dtype=self.dtype, device=self.device)
+        global _reallocations
+        _reallocations += 1
+        grown = torch.zeros(new_capacity, dtype=self.dtype, device=self.device)
         grown[:self.capacity].copy_(self.raw_buffer)
         self.raw_buffer = grown
         self.capacity = new_capacity

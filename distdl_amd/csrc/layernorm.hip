@@ -1,15 +1,26 @@
-// DistributedLayerNorm, local shard, fp32 (reference: nn/layernorm.py:218-247,
-// 295-309).  Two kernels with the cross-worker exchange between them:
+// DistributedLayerNorm, local shard (reference: nn/layernorm.py:218-247,
+// 295-321).  Elements are fp32, bf16 or fp16; every sum is fp32.
 //
 //   ln_stats     x[rows, cols] -> {mean_r, M2_r} per row     (one read of x)
 //   ln_normalize gathered {mean_p, M2_p} of the P workers sharing a row
 //                -> combined mean / var -> y = (x-mean)*rstd*gamma+beta
+//   ln_fused     both in one launch, for rows that one worker holds whole
+//                (the reference's torch.nn.functional.layer_norm branch, :310-319)
 //
-// Rows of up to 2048 columns live in registers: one wavefront owns a row, each
-// lane holds float4 pieces, sums go through DPP/shuffle butterflies; a long
-// input keeps two rows per wavefront in flight.  Longer (or unaligned)
-// rows are staged once in LDS by a 256-thread workgroup and reduced from there.
+// Three ways of holding a row, chosen by its length:
+//   wavefront rows  up to 2048 columns: one wavefront owns a row, each lane
+//                   holds pieces of four elements, sums go through shuffle
+//                   butterflies; a long input keeps two rows per wavefront in
+//                   flight
+//   workgroup rows  up to 16384 columns: a 256-thread workgroup owns a row, still
+//                   in registers (up to 16 pieces of four per thread), sums go
+//                   through the wavefronts and four words of LDS
+//   streamed rows   anything longer, or rows whose length, pitch or address
+//                   rule out four-element accesses: a workgroup walks the row
+//                   once per reduction
 #include "ddl_common.h"
+
+#include <hip/hip_fp16.h>
 
 namespace ddl {
 namespace {
@@ -18,11 +29,79 @@ constexpr int kWave = 64;
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr int kMaxParts = 256;
-constexpr int kLdsFloats = 16384;  // 64 KiB of staged row
+constexpr int kWaveRowCols = 2048;     // longest row a wavefront keeps in registers
+constexpr int kBlockRowCols = 16384;   // longest row a workgroup keeps in registers
 
 struct PartCounts {
     float inv_n[kMaxParts];  // 1 / columns held by worker p
 };
+
+// ------------------------------------------------------------ element I/O --
+
+struct bf16_t {
+    uint16_t bits;
+};
+
+__device__ inline float bf16_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+__device__ inline uint32_t f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if (f != f) return 0x7FC0u;
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+
+// Four consecutive elements as floats; y is never read again by these kernels,
+// so it leaves with streaming stores.
+__device__ inline float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ inline float4 load4(const bf16_t* p) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p);
+    return make_float4(bf16_to_f32(w.x & 0xFFFFu), bf16_to_f32(w.x >> 16), bf16_to_f32(w.y & 0xFFFFu), bf16_to_f32(w.y >> 16));
+}
+__device__ inline float4 load4(const __half* p) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p);
+    const __half2 a = *reinterpret_cast<const __half2*>(&w.x), b = *reinterpret_cast<const __half2*>(&w.y);
+    const float2 fa = __half22float2(a), fb = __half22float2(b);
+    return make_float4(fa.x, fa.y, fb.x, fb.y);
+}
+__device__ inline void store4(float* p, float4 v) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    f32x4 o;
+    o[0] = v.x, o[1] = v.y, o[2] = v.z, o[3] = v.w;
+    __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(p));
+}
+__device__ inline void store4(bf16_t* p, float4 v) {
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    u32x2 o;
+    o[0] = f32_to_bf16(v.x) | (f32_to_bf16(v.y) << 16);
+    o[1] = f32_to_bf16(v.z) | (f32_to_bf16(v.w) << 16);
+    __builtin_nontemporal_store(o, reinterpret_cast<u32x2*>(p));
+}
+__device__ inline void store4(__half* p, float4 v) {
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const __half2 a = __floats2half2_rn(v.x, v.y), b = __floats2half2_rn(v.z, v.w);
+    u32x2 o;
+    o[0] = *reinterpret_cast<const uint32_t*>(&a);
+    o[1] = *reinterpret_cast<const uint32_t*>(&b);
+    __builtin_nontemporal_store(o, reinterpret_cast<u32x2*>(p));
+}
+__device__ inline float load1(const float* p) { return *p; }
+__device__ inline float load1(const bf16_t* p) { return bf16_to_f32(p->bits); }
+__device__ inline float load1(const __half* p) { return __half2float(*p); }
+__device__ inline void store1(float* p, float v) { *p = v; }
+__device__ inline void store1(bf16_t* p, float v) { p->bits = static_cast<uint16_t>(f32_to_bf16(v)); }
+__device__ inline void store1(__half* p, float v) { *p = __float2half_rn(v); }
+
+__device__ inline float sum4(float4 v) { return (v.x + v.y) + (v.z + v.w); }
+__device__ inline float sq4(float4 v, float m) {
+    const float a = v.x - m, b = v.y - m, c = v.z - m, d = v.w - m;
+    return (a * a + b * b) + (c * c + d * d);
+}
+__device__ inline float4 norm4(float4 v, float mean, float rstd) {
+    return make_float4((v.x - mean) * rstd, (v.y - mean) * rstd, (v.z - mean) * rstd, (v.w - mean) * rstd);
+}
+__device__ inline float4 affine4(float4 g, float4 o, float4 b) {
+    return make_float4(g.x * o.x + b.x, g.y * o.y + b.y, g.z * o.z + b.z, g.w * o.w + b.w);
+}
 
 __device__ inline float wave_sum(float v) {
 #pragma unroll
@@ -30,6 +109,8 @@ __device__ inline float wave_sum(float v) {
     return v;
 }
 
+// Sum over the workgroup, the same value in every thread.  `scratch` holds one
+// float per wavefront; the leading barrier lets it be reused call after call.
 __device__ inline float block_sum(float v, float* scratch) {
     v = wave_sum(v);
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
@@ -73,67 +154,49 @@ __device__ inline void combine_parts(const float* __restrict__ part_stats, int64
     *rstd_out = 1.0f / sqrtf(var + eps);
 }
 
-// ------------------------------------------------------ register-row path --
+// What the three kernels of a family do with a row once its statistics exist.
+enum Mode {
+    kStats = 0,   // emit {mean, M2} of the local columns
+    kNorm = 1,    // statistics come from the gathered pairs
+    kFused = 2,   // statistics of the local columns are the row's statistics
+};
 
-// One wavefront per row, NV float4 per lane (cols <= 256*NV, cols % 4 == 0),
-// RPW rows of a wavefront in flight at once.
-template <int NV, int RPW>
-__global__ __launch_bounds__(kBlock) void ln_stats_rows(const float* __restrict__ x, int64_t rows, int cols, int64_t ld,
-                                                        float* __restrict__ stats) {
+struct LnArgs {
+    const void* x;
+    void* y;
+    const void* gamma;
+    const void* beta;
+    const float* part_stats;
+    float* stats;
+    float* mean_out;
+    float* rstd_out;
+    int64_t rows, ld, ldy;
+    int cols;
+    int nparts;
+    float eps;
+};
+
+// --------------------------------------------------------- wavefront rows --
+
+// One wavefront per row, NV pieces of four per lane (cols <= 256 NV, cols % 4
+// == 0), RPW rows of a wavefront in flight at once.
+template <typename T, int NV, int RPW, int MODE, bool AFFINE>
+__global__ __launch_bounds__(kBlock) void ln_wave_rows(const LnArgs a, const PartCounts pc) {
+    const T* __restrict__ x = static_cast<const T*>(a.x);
+    T* __restrict__ y = static_cast<T*>(a.y);
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t wave = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + threadIdx.x / kWave;
     const int64_t r0 = wave * RPW;
-    const int nv = cols >> 2;
-    float4 v[RPW][NV];
-#pragma unroll
-    for (int i = 0; i < RPW; ++i) {
-        const int64_t r = r0 + i;
-#pragma unroll
-        for (int k = 0; k < NV; ++k) {
-            const int c = lane + k * kWave;
-            v[i][k] = (r < rows && c < nv) ? reinterpret_cast<const float4*>(x + r * ld)[c] : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-    }
-    const float inv = 1.0f / static_cast<float>(cols);
-#pragma unroll
-    for (int i = 0; i < RPW; ++i) {
-        const int64_t r = r0 + i;
-        float s = 0.f;
-#pragma unroll
-        for (int k = 0; k < NV; ++k) s += (v[i][k].x + v[i][k].y) + (v[i][k].z + v[i][k].w);
-        const float mean = wave_sum(s) * inv;
-        float q = 0.f;
-#pragma unroll
-        for (int k = 0; k < NV; ++k) {
-            if (lane + k * kWave < nv) {
-                const float a = v[i][k].x - mean, b = v[i][k].y - mean, c = v[i][k].z - mean, d = v[i][k].w - mean;
-                q += (a * a + b * b) + (c * c + d * d);
-            }
-        }
-        q = wave_sum(q);
-        if (lane == 0 && r < rows) reinterpret_cast<float2*>(stats)[r] = make_float2(mean, q);
-    }
-}
-
-template <int NV, int RPW, bool AFFINE>
-__global__ __launch_bounds__(kBlock) void ln_norm_rows(const float* __restrict__ x, int64_t rows, int cols, int64_t ld,
-                                                       const float* __restrict__ part_stats, int nparts,
-                                                       const PartCounts pc, const float* __restrict__ gamma,
-                                                       const float* __restrict__ beta, float eps, float* __restrict__ y,
-                                                       int64_t ldy, float* __restrict__ mean_out,
-                                                       float* __restrict__ rstd_out) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const int64_t wave = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + threadIdx.x / kWave;
-    const int64_t r0 = wave * RPW;
-    const int nv = cols >> 2;
+    const int64_t rows = a.rows;
+    const int nv = a.cols >> 2;
     float4 g[NV], b[NV];
-    if (AFFINE) {
+    if (MODE != kStats && AFFINE) {
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const int c = lane + k * kWave;
             if (c < nv) {
-                g[k] = reinterpret_cast<const float4*>(gamma)[c];
-                b[k] = reinterpret_cast<const float4*>(beta)[c];
+                g[k] = load4(static_cast<const T*>(a.gamma) + 4 * c);
+                b[k] = load4(static_cast<const T*>(a.beta) + 4 * c);
             }
         }
     }
@@ -141,11 +204,14 @@ __global__ __launch_bounds__(kBlock) void ln_norm_rows(const float* __restrict__
     // the gathered statistics of its rows (lane p fetches worker p's pair) and
     // the rows themselves.
     float2 ps[RPW];
-    const float inv_n = lane < nparts ? pc.inv_n[lane] : 0.f;
+    float inv_n = 0.f;
+    if (MODE == kNorm) {
+        inv_n = lane < a.nparts ? pc.inv_n[lane] : 0.f;
 #pragma unroll
-    for (int i = 0; i < RPW; ++i) {
-        const int64_t r = r0 + i;
-        ps[i] = (r < rows && lane < nparts) ? load_part(part_stats, rows, r, lane) : make_float2(0.f, 0.f);
+        for (int i = 0; i < RPW; ++i) {
+            const int64_t r = r0 + i;
+            ps[i] = (r < rows && lane < a.nparts) ? load_part(a.part_stats, rows, r, lane) : make_float2(0.f, 0.f);
+        }
     }
     float4 v[RPW][NV];
 #pragma unroll
@@ -154,142 +220,249 @@ __global__ __launch_bounds__(kBlock) void ln_norm_rows(const float* __restrict__
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const int c = lane + k * kWave;
-            if (r < rows && c < nv) v[i][k] = reinterpret_cast<const float4*>(x + r * ld)[c];
+            v[i][k] = (r < rows && c < nv) ? load4(x + r * a.ld + 4 * c) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     }
+    const float inv = 1.0f / static_cast<float>(a.cols);
 #pragma unroll
     for (int i = 0; i < RPW; ++i) {
         const int64_t r = r0 + i;
-        if (r >= rows) continue;
+        if (r >= rows) continue;   // the whole wavefront takes the same branch
         float mean, rstd;
-        combine_parts(part_stats, rows, r, nparts, pc, eps, lane, ps[i], inv_n, &mean, &rstd);
+        if (MODE == kNorm) {
+            combine_parts(a.part_stats, rows, r, a.nparts, pc, a.eps, lane, ps[i], inv_n, &mean, &rstd);
+        } else {
+            float s = 0.f;
+#pragma unroll
+            for (int k = 0; k < NV; ++k) s += sum4(v[i][k]);
+            mean = wave_sum(s) * inv;
+            float q = 0.f;
+#pragma unroll
+            for (int k = 0; k < NV; ++k)
+                if (lane + k * kWave < nv) q += sq4(v[i][k], mean);
+            q = wave_sum(q);
+            if (MODE == kStats) {
+                if (lane == 0) reinterpret_cast<float2*>(a.stats)[r] = make_float2(mean, q);
+                continue;
+            }
+            rstd = 1.0f / sqrtf(q * inv + a.eps);
+        }
         if (lane == 0) {
-            if (mean_out) mean_out[r] = mean;
-            if (rstd_out) rstd_out[r] = rstd;
+            if (a.mean_out) a.mean_out[r] = mean;
+            if (a.rstd_out) a.rstd_out[r] = rstd;
         }
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             const int c = lane + k * kWave;
             if (c < nv) {
-                float4 o;
-                o.x = (v[i][k].x - mean) * rstd;
-                o.y = (v[i][k].y - mean) * rstd;
-                o.z = (v[i][k].z - mean) * rstd;
-                o.w = (v[i][k].w - mean) * rstd;
-                if (AFFINE) {
-                    o.x = g[k].x * o.x + b[k].x;
-                    o.y = g[k].y * o.y + b[k].y;
-                    o.z = g[k].z * o.z + b[k].z;
-                    o.w = g[k].w * o.w + b[k].w;
-                }
-                // y is not read again by this kernel: streaming store
-                typedef float f32x4 __attribute__((ext_vector_type(4)));
-                f32x4 ov;
-                ov[0] = o.x, ov[1] = o.y, ov[2] = o.z, ov[3] = o.w;
-                __builtin_nontemporal_store(ov, reinterpret_cast<f32x4*>(y + r * ldy) + c);
+                float4 o = norm4(v[i][k], mean, rstd);
+                if (AFFINE) o = affine4(g[k], o, b[k]);
+                store4(y + r * a.ldy + 4 * c, o);
             }
         }
     }
 }
 
-// ------------------------------------------------------ LDS-staged path ----
+// --------------------------------------------------------- workgroup rows --
 
-// One workgroup per row; the row is read from HBM once into LDS (when it fits)
-// and both reductions run from the staged copy.
-__global__ __launch_bounds__(kBlock) void ln_stats_lds(const float* __restrict__ x, int64_t rows, int64_t cols, int64_t ld,
-                                                       float* __restrict__ stats, int staged) {
-    __shared__ float row[kLdsFloats];
+// One workgroup per row, NV pieces of four per thread (cols <= 1024 NV, cols
+// % 4 == 0); the grid walks the rows.
+template <typename T, int NV, int MODE, bool AFFINE>
+__global__ __launch_bounds__(kBlock) void ln_block_rows(const LnArgs a, const PartCounts pc) {
     __shared__ float scratch[kWavesPerBlock];
-    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
-        const float* xr = x + r * ld;
-        float s = 0.f;
-        for (int64_t c = threadIdx.x; c < cols; c += kBlock) {
-            const float t = xr[c];
-            if (staged) row[c] = t;
-            s += t;
+    const T* __restrict__ x = static_cast<const T*>(a.x);
+    T* __restrict__ y = static_cast<T*>(a.y);
+    const int t = threadIdx.x, lane = t & (kWave - 1);
+    const int nv = a.cols >> 2;
+    const float inv = 1.0f / static_cast<float>(a.cols);
+    for (int64_t r = blockIdx.x; r < a.rows; r += gridDim.x) {
+        float2 first = make_float2(0.f, 0.f);
+        if (MODE == kNorm && lane < a.nparts) first = load_part(a.part_stats, a.rows, r, lane);
+        float4 v[NV];
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const int c = t + k * kBlock;
+            v[k] = c < nv ? load4(x + r * a.ld + 4 * c) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
-        const float mean = block_sum(s, scratch) / static_cast<float>(cols);
-        float q = 0.f;
-        for (int64_t c = threadIdx.x; c < cols; c += kBlock) {
-            const float d = (staged ? row[c] : xr[c]) - mean;
-            q += d * d;
-        }
-        q = block_sum(q, scratch);
-        if (threadIdx.x == 0) reinterpret_cast<float2*>(stats)[r] = make_float2(mean, q);
-        __syncthreads();
-    }
-}
-
-__global__ __launch_bounds__(kBlock) void ln_norm_stream(const float* __restrict__ x, int64_t rows, int64_t cols, int64_t ld,
-                                                         const float* __restrict__ part_stats, int nparts,
-                                                         const PartCounts pc, const float* __restrict__ gamma,
-                                                         const float* __restrict__ beta, float eps, float* __restrict__ y,
-                                                         int64_t ldy, float* __restrict__ mean_out,
-                                                         float* __restrict__ rstd_out) {
-    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
         float mean, rstd;
-        const int lane = threadIdx.x & (kWave - 1);
-        combine_parts(part_stats, rows, r, nparts, pc, eps, lane,
-                      lane < nparts ? load_part(part_stats, rows, r, lane) : make_float2(0.f, 0.f),
-                      lane < nparts ? pc.inv_n[lane] : 0.f, &mean, &rstd);
-        if (threadIdx.x == 0) {
-            if (mean_out) mean_out[r] = mean;
-            if (rstd_out) rstd_out[r] = rstd;
+        if (MODE == kNorm) {
+            // every wavefront combines the pairs for itself: no exchange needed
+            combine_parts(a.part_stats, a.rows, r, a.nparts, pc, a.eps, lane, first, lane < a.nparts ? pc.inv_n[lane] : 0.f,
+                          &mean, &rstd);
+        } else {
+            float s = 0.f;
+#pragma unroll
+            for (int k = 0; k < NV; ++k) s += sum4(v[k]);
+            mean = block_sum(s, scratch) * inv;
+            float q = 0.f;
+#pragma unroll
+            for (int k = 0; k < NV; ++k)
+                if (t + k * kBlock < nv) q += sq4(v[k], mean);
+            q = block_sum(q, scratch);
+            if (MODE == kStats) {
+                if (t == 0) reinterpret_cast<float2*>(a.stats)[r] = make_float2(mean, q);
+                continue;
+            }
+            rstd = 1.0f / sqrtf(q * inv + a.eps);
         }
-        const float* xr = x + r * ld;
-        float* yr = y + r * ldy;
-        for (int64_t c = threadIdx.x; c < cols; c += kBlock) {
-            float o = (xr[c] - mean) * rstd;
-            if (gamma) o = gamma[c] * o + beta[c];
-            yr[c] = o;
+        if (t == 0) {
+            if (a.mean_out) a.mean_out[r] = mean;
+            if (a.rstd_out) a.rstd_out[r] = rstd;
+        }
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const int c = t + k * kBlock;
+            if (c < nv) {
+                float4 o = norm4(v[k], mean, rstd);
+                if (AFFINE) o = affine4(load4(static_cast<const T*>(a.gamma) + 4 * c), o, load4(static_cast<const T*>(a.beta) + 4 * c));
+                store4(y + r * a.ldy + 4 * c, o);
+            }
         }
     }
 }
 
-bool rows_vectorizable(const void* p, int64_t cols, int64_t ld) {
-    return cols % 4 == 0 && ld % 4 == 0 && cols <= 2048 && aligned_to(p, 16);
+// ---------------------------------------------------------- streamed rows --
+
+// One workgroup per row, the row read once per reduction.  VEC: pieces of four
+// (cols % 4 == 0, pitches and addresses allow it), else element by element.
+template <typename T, int MODE, bool VEC>
+__global__ __launch_bounds__(kBlock) void ln_stream_rows(const LnArgs a, const PartCounts pc) {
+    __shared__ float scratch[kWavesPerBlock];
+    const T* __restrict__ x = static_cast<const T*>(a.x);
+    T* __restrict__ y = static_cast<T*>(a.y);
+    const T* __restrict__ gamma = static_cast<const T*>(a.gamma);
+    const T* __restrict__ beta = static_cast<const T*>(a.beta);
+    const int t = threadIdx.x, lane = t & (kWave - 1);
+    const int64_t cols = a.cols;
+    const float inv = 1.0f / static_cast<float>(a.cols);
+    for (int64_t r = blockIdx.x; r < a.rows; r += gridDim.x) {
+        const T* xr = x + r * a.ld;
+        float mean, rstd;
+        if (MODE == kNorm) {
+            combine_parts(a.part_stats, a.rows, r, a.nparts, pc, a.eps, lane,
+                          lane < a.nparts ? load_part(a.part_stats, a.rows, r, lane) : make_float2(0.f, 0.f),
+                          lane < a.nparts ? pc.inv_n[lane] : 0.f, &mean, &rstd);
+        } else {
+            float s = 0.f;
+            if (VEC) {
+                for (int64_t c = 4 * t; c < cols; c += 4 * kBlock) s += sum4(load4(xr + c));
+            } else {
+                for (int64_t c = t; c < cols; c += kBlock) s += load1(xr + c);
+            }
+            mean = block_sum(s, scratch) * inv;
+            float q = 0.f;
+            if (VEC) {
+                for (int64_t c = 4 * t; c < cols; c += 4 * kBlock) q += sq4(load4(xr + c), mean);
+            } else {
+                for (int64_t c = t; c < cols; c += kBlock) {
+                    const float d = load1(xr + c) - mean;
+                    q += d * d;
+                }
+            }
+            q = block_sum(q, scratch);
+            if (MODE == kStats) {
+                if (t == 0) reinterpret_cast<float2*>(a.stats)[r] = make_float2(mean, q);
+                continue;
+            }
+            rstd = 1.0f / sqrtf(q * inv + a.eps);
+        }
+        if (t == 0) {
+            if (a.mean_out) a.mean_out[r] = mean;
+            if (a.rstd_out) a.rstd_out[r] = rstd;
+        }
+        T* yr = y + r * a.ldy;
+        if (VEC) {
+            for (int64_t c = 4 * t; c < cols; c += 4 * kBlock) {
+                float4 o = norm4(load4(xr + c), mean, rstd);
+                if (gamma) o = affine4(load4(gamma + c), o, load4(beta + c));
+                store4(yr + c, o);
+            }
+        } else {
+            for (int64_t c = t; c < cols; c += kBlock) {
+                float o = (load1(xr + c) - mean) * rstd;
+                if (gamma) o = load1(gamma + c) * o + load1(beta + c);
+                store1(yr + c, o);
+            }
+        }
+    }
 }
+
+// ------------------------------------------------------------------ host ---
 
 // Rows a wavefront keeps in flight.  Few rows per wavefront mean more
 // wavefronts, which is what a small input needs to occupy the whole chip; two
 // rows per wavefront stream a long input a little faster.
 constexpr int64_t kSmallRows = 65536;
 
-template <int NV, int RPW>
-int launch_stats_rpw(const float* x, int64_t rows, int cols, int64_t ld, float* stats, hipStream_t s) {
-    const int64_t waves = (rows + RPW - 1) / RPW;
+template <typename T, int MODE, bool AFFINE, int NV, int RPW>
+void launch_wave_rpw(const LnArgs& a, const PartCounts& pc, hipStream_t s) {
+    const int64_t waves = (a.rows + RPW - 1) / RPW;
     const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
-    hipLaunchKernelGGL((ln_stats_rows<NV, RPW>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, s, x, rows, cols, ld, stats);
-    return check_launch("ln_stats_rows");
+    hipLaunchKernelGGL((ln_wave_rows<T, NV, RPW, MODE, AFFINE>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, s, a, pc);
 }
 
-template <int NV>
-int launch_stats(const float* x, int64_t rows, int cols, int64_t ld, float* stats, hipStream_t s) {
-    if (NV <= 2 && rows > kSmallRows) return launch_stats_rpw<NV, 2>(x, rows, cols, ld, stats, s);
-    return launch_stats_rpw<NV, 1>(x, rows, cols, ld, stats, s);
-}
-
-template <int NV, int RPW>
-int launch_norm_rpw(const float* x, int64_t rows, int cols, int64_t ld, const float* ps, int nparts, const PartCounts& pc,
-                    const float* gamma, const float* beta, float eps, float* y, int64_t ldy, float* mo, float* ro,
-                    hipStream_t s) {
-    const int64_t waves = (rows + RPW - 1) / RPW;
-    const int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
-    if (gamma)
-        hipLaunchKernelGGL((ln_norm_rows<NV, RPW, true>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, s, x, rows, cols,
-                           ld, ps, nparts, pc, gamma, beta, eps, y, ldy, mo, ro);
+template <typename T, int MODE, bool AFFINE, int NV>
+void launch_wave(const LnArgs& a, const PartCounts& pc, hipStream_t s) {
+    if (NV <= 2 && a.rows > kSmallRows)
+        launch_wave_rpw<T, MODE, AFFINE, NV, 2>(a, pc, s);
     else
-        hipLaunchKernelGGL((ln_norm_rows<NV, RPW, false>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, s, x, rows,
-                           cols, ld, ps, nparts, pc, gamma, beta, eps, y, ldy, mo, ro);
-    return check_launch("ln_norm_rows");
+        launch_wave_rpw<T, MODE, AFFINE, NV, 1>(a, pc, s);
 }
 
-template <int NV>
-int launch_norm(const float* x, int64_t rows, int cols, int64_t ld, const float* ps, int nparts, const PartCounts& pc,
-                const float* gamma, const float* beta, float eps, float* y, int64_t ldy, float* mo, float* ro,
-                hipStream_t s) {
-    if (NV <= 2 && rows > kSmallRows) return launch_norm_rpw<NV, 2>(x, rows, cols, ld, ps, nparts, pc, gamma, beta, eps, y, ldy, mo, ro, s);
-    return launch_norm_rpw<NV, 1>(x, rows, cols, ld, ps, nparts, pc, gamma, beta, eps, y, ldy, mo, ro, s);
+template <typename T, int MODE, bool AFFINE, int NV>
+void launch_block(const LnArgs& a, const PartCounts& pc, hipStream_t s) {
+    const uint32_t blocks = static_cast<uint32_t>(a.rows < (1 << 20) ? a.rows : (1 << 20));
+    hipLaunchKernelGGL((ln_block_rows<T, NV, MODE, AFFINE>), dim3(blocks), dim3(kBlock), 0, s, a, pc);
+}
+
+template <typename T, int MODE, bool AFFINE>
+int launch_typed(const LnArgs& a, const PartCounts& pc, bool vec, hipStream_t s) {
+    const int cols = a.cols;
+    if (vec && cols <= kWaveRowCols) {
+        if (cols <= 256) launch_wave<T, MODE, AFFINE, 1>(a, pc, s);
+        else if (cols <= 512) launch_wave<T, MODE, AFFINE, 2>(a, pc, s);
+        else if (cols <= 1024) launch_wave<T, MODE, AFFINE, 4>(a, pc, s);
+        else launch_wave<T, MODE, AFFINE, 8>(a, pc, s);
+        return check_launch("ln_wave_rows");
+    }
+    if (vec && cols <= kBlockRowCols) {
+        if (cols <= 4096) launch_block<T, MODE, AFFINE, 4>(a, pc, s);
+        else if (cols <= 8192) launch_block<T, MODE, AFFINE, 8>(a, pc, s);
+        else launch_block<T, MODE, AFFINE, 16>(a, pc, s);
+        return check_launch("ln_block_rows");
+    }
+    const uint32_t blocks = static_cast<uint32_t>(a.rows < 65536 ? a.rows : 65536);
+    if (vec)
+        hipLaunchKernelGGL((ln_stream_rows<T, MODE, true>), dim3(blocks), dim3(kBlock), 0, s, a, pc);
+    else
+        hipLaunchKernelGGL((ln_stream_rows<T, MODE, false>), dim3(blocks), dim3(kBlock), 0, s, a, pc);
+    return check_launch("ln_stream_rows");
+}
+
+template <int MODE>
+int launch_mode(int dtype, const LnArgs& a, const PartCounts& pc, bool vec, hipStream_t s) {
+    const bool affine = MODE != kStats && a.gamma != nullptr;
+    switch (dtype) {
+        case DDL_DT_F32:
+            return affine ? launch_typed<float, MODE, true>(a, pc, vec, s) : launch_typed<float, MODE, false>(a, pc, vec, s);
+        case DDL_DT_BF16:
+            return affine ? launch_typed<bf16_t, MODE, true>(a, pc, vec, s) : launch_typed<bf16_t, MODE, false>(a, pc, vec, s);
+        default:
+            return affine ? launch_typed<__half, MODE, true>(a, pc, vec, s) : launch_typed<__half, MODE, false>(a, pc, vec, s);
+    }
+}
+
+int elem_size_of(int dtype) { return dtype == DDL_DT_F32 ? 4 : (dtype == DDL_DT_BF16 || dtype == DDL_DT_F16) ? 2 : 0; }
+
+// Four-element accesses need rows of a multiple of four columns whose first
+// elements are all aligned to four elements.
+bool quad_access(const void* p, int es, int64_t cols, int64_t ld) { return cols % 4 == 0 && ld % 4 == 0 && aligned_to(p, 4 * es); }
+
+int check_common(const char* what, int dtype, int64_t rows, int64_t cols, int64_t ld) {
+    if (elem_size_of(dtype) == 0) return fail(DDL_E_UNSUPP, "%s: dtype %d (f32, bf16 and f16 only)", what, dtype);
+    if (rows < 0 || cols < 1 || ld < cols) return fail(DDL_E_ARG, "%s: rows=%lld cols=%lld ld=%lld", what, (long long)rows, (long long)cols, (long long)ld);
+    if (rows > 0x7FFFFFFFll || cols > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "%s: more than 2^31 rows or columns", what);
+    return 0;
 }
 
 }  // namespace
@@ -297,57 +470,78 @@ int launch_norm(const float* x, int64_t rows, int cols, int64_t ld, const float*
 
 extern "C" {
 
-int ddl_ln_partial_stats_f32(const float* x, int64_t rows, int64_t cols, int64_t ld, float* stats, void* stream) {
+int ddl_ln_partial_stats(const void* x, int dtype, int64_t rows, int64_t cols, int64_t ld, float* stats, void* stream) {
     using namespace ddl;
-    if (rows < 0 || cols < 1 || ld < cols) return fail(DDL_E_ARG, "ln stats: rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld);
+    if (const int rc = check_common("ln stats", dtype, rows, cols, ld)) return rc;
     if (rows == 0) return 0;
     if (!x || !stats) return fail(DDL_E_ARG, "ln stats: null pointer");
-    if (!aligned_to(x, 4) || !aligned_to(stats, 8)) return fail(DDL_E_ALIGN, "ln stats: x must be 4-byte and stats 8-byte aligned");
-    if (rows > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "ln stats: more than 2^31 rows");
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (rows_vectorizable(x, cols, ld)) {
-        const int c = static_cast<int>(cols);
-        if (cols <= 256) return launch_stats<1>(x, rows, c, ld, stats, s);
-        if (cols <= 512) return launch_stats<2>(x, rows, c, ld, stats, s);
-        if (cols <= 1024) return launch_stats<4>(x, rows, c, ld, stats, s);
-        return launch_stats<8>(x, rows, c, ld, stats, s);
-    }
-    const uint32_t blocks = static_cast<uint32_t>(rows < 65536 ? rows : 65536);
-    hipLaunchKernelGGL(ln_stats_lds, dim3(blocks), dim3(kBlock), 0, s, x, rows, cols, ld, stats, cols <= kLdsFloats ? 1 : 0);
-    return check_launch("ln_stats_lds");
+    const int es = elem_size_of(dtype);
+    if (!aligned_to(x, es) || !aligned_to(stats, 8)) return fail(DDL_E_ALIGN, "ln stats: x must be element-aligned and stats 8-byte aligned");
+    LnArgs a{};
+    a.x = x;
+    a.stats = stats;
+    a.rows = rows, a.ld = ld, a.cols = static_cast<int>(cols);
+    const PartCounts pc{};
+    return launch_mode<kStats>(dtype, a, pc, quad_access(x, es, cols, ld), static_cast<hipStream_t>(stream));
 }
 
-int ddl_ln_normalize_affine_f32(const float* x, int64_t rows, int64_t cols, int64_t ld, const float* part_stats,
-                                int nparts, const int64_t* part_cols, const float* gamma, const float* beta, float eps,
-                                float* y, int64_t ldy, float* mean_out, float* rstd_out, void* stream) {
+int ddl_ln_normalize_affine(const void* x, int dtype, int64_t rows, int64_t cols, int64_t ld, const float* part_stats,
+                            int nparts, const int64_t* part_cols, const void* gamma, const void* beta, float eps, void* y,
+                            int64_t ldy, float* mean_out, float* rstd_out, void* stream) {
     using namespace ddl;
-    if (rows < 0 || cols < 1 || ld < cols || ldy < cols) return fail(DDL_E_ARG, "ln normalize: rows=%lld cols=%lld ld=%lld ldy=%lld", (long long)rows, (long long)cols, (long long)ld, (long long)ldy);
+    if (const int rc = check_common("ln normalize", dtype, rows, cols, ld)) return rc;
+    if (ldy < cols) return fail(DDL_E_ARG, "ln normalize: ldy=%lld below cols=%lld", (long long)ldy, (long long)cols);
     if (nparts < 1 || nparts > kMaxParts) return fail(DDL_E_UNSUPP, "ln normalize: nparts=%d outside [1,%d]", nparts, kMaxParts);
     if ((gamma == nullptr) != (beta == nullptr)) return fail(DDL_E_ARG, "ln normalize: gamma and beta must both be given or both be NULL");
     if (rows == 0) return 0;
     if (!x || !y || !part_stats || !part_cols) return fail(DDL_E_ARG, "ln normalize: null pointer");
-    if (rows > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "ln normalize: more than 2^31 rows");
-    if (!aligned_to(x, 4) || !aligned_to(y, 4) || !aligned_to(part_stats, 8))
-        return fail(DDL_E_ALIGN, "ln normalize: x, y must be 4-byte and the statistics 8-byte aligned");
+    const int es = elem_size_of(dtype);
+    if (!aligned_to(x, es) || !aligned_to(y, es) || !aligned_to(gamma, es) || !aligned_to(beta, es) || !aligned_to(part_stats, 8))
+        return fail(DDL_E_ALIGN, "ln normalize: x, y, gamma, beta must be element-aligned and the statistics 8-byte aligned");
     PartCounts pc{};
     for (int p = 0; p < nparts; ++p) {
         if (part_cols[p] < 1) return fail(DDL_E_ARG, "ln normalize: worker %d holds %lld columns", p, (long long)part_cols[p]);
         pc.inv_n[p] = 1.0f / static_cast<float>(part_cols[p]);
     }
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool vec = rows_vectorizable(x, cols, ld) && ldy % 4 == 0 && aligned_to(y, 16) &&
-                     (!gamma || (aligned_to(gamma, 16) && aligned_to(beta, 16)));
-    if (vec) {
-        const int c = static_cast<int>(cols);
-        if (cols <= 256) return launch_norm<1>(x, rows, c, ld, part_stats, nparts, pc, gamma, beta, eps, y, ldy, mean_out, rstd_out, s);
-        if (cols <= 512) return launch_norm<2>(x, rows, c, ld, part_stats, nparts, pc, gamma, beta, eps, y, ldy, mean_out, rstd_out, s);
-        if (cols <= 1024) return launch_norm<4>(x, rows, c, ld, part_stats, nparts, pc, gamma, beta, eps, y, ldy, mean_out, rstd_out, s);
-        return launch_norm<8>(x, rows, c, ld, part_stats, nparts, pc, gamma, beta, eps, y, ldy, mean_out, rstd_out, s);
-    }
-    const uint32_t blocks = static_cast<uint32_t>(rows < 65536 ? rows : 65536);
-    hipLaunchKernelGGL(ln_norm_stream, dim3(blocks), dim3(kBlock), 0, s, x, rows, cols, ld, part_stats, nparts, pc, gamma,
-                       beta, eps, y, ldy, mean_out, rstd_out);
-    return check_launch("ln_norm_stream");
+    LnArgs a{};
+    a.x = x, a.y = y, a.gamma = gamma, a.beta = beta, a.part_stats = part_stats;
+    a.mean_out = mean_out, a.rstd_out = rstd_out;
+    a.rows = rows, a.ld = ld, a.ldy = ldy, a.cols = static_cast<int>(cols), a.nparts = nparts, a.eps = eps;
+    const bool vec = quad_access(x, es, cols, ld) && quad_access(y, es, cols, ldy) &&
+                     (!gamma || (aligned_to(gamma, 4 * es) && aligned_to(beta, 4 * es)));
+    return launch_mode<kNorm>(dtype, a, pc, vec, static_cast<hipStream_t>(stream));
+}
+
+int ddl_layer_norm(const void* x, int dtype, int64_t rows, int64_t cols, int64_t ld, const void* gamma, const void* beta,
+                   float eps, void* y, int64_t ldy, float* mean_out, float* rstd_out, void* stream) {
+    using namespace ddl;
+    if (const int rc = check_common("layer norm", dtype, rows, cols, ld)) return rc;
+    if (ldy < cols) return fail(DDL_E_ARG, "layer norm: ldy=%lld below cols=%lld", (long long)ldy, (long long)cols);
+    if ((gamma == nullptr) != (beta == nullptr)) return fail(DDL_E_ARG, "layer norm: gamma and beta must both be given or both be NULL");
+    if (rows == 0) return 0;
+    if (!x || !y) return fail(DDL_E_ARG, "layer norm: null pointer");
+    const int es = elem_size_of(dtype);
+    if (!aligned_to(x, es) || !aligned_to(y, es) || !aligned_to(gamma, es) || !aligned_to(beta, es))
+        return fail(DDL_E_ALIGN, "layer norm: x, y, gamma, beta must be element-aligned");
+    LnArgs a{};
+    a.x = x, a.y = y, a.gamma = gamma, a.beta = beta;
+    a.mean_out = mean_out, a.rstd_out = rstd_out;
+    a.rows = rows, a.ld = ld, a.ldy = ldy, a.cols = static_cast<int>(cols), a.nparts = 1, a.eps = eps;
+    const PartCounts pc{};
+    const bool vec = quad_access(x, es, cols, ld) && quad_access(y, es, cols, ldy) &&
+                     (!gamma || (aligned_to(gamma, 4 * es) && aligned_to(beta, 4 * es)));
+    return launch_mode<kFused>(dtype, a, pc, vec, static_cast<hipStream_t>(stream));
+}
+
+int ddl_ln_partial_stats_f32(const float* x, int64_t rows, int64_t cols, int64_t ld, float* stats, void* stream) {
+    return ddl_ln_partial_stats(x, DDL_DT_F32, rows, cols, ld, stats, stream);
+}
+
+int ddl_ln_normalize_affine_f32(const float* x, int64_t rows, int64_t cols, int64_t ld, const float* part_stats,
+                                int nparts, const int64_t* part_cols, const float* gamma, const float* beta, float eps,
+                                float* y, int64_t ldy, float* mean_out, float* rstd_out, void* stream) {
+    return ddl_ln_normalize_affine(x, DDL_DT_F32, rows, cols, ld, part_stats, nparts, part_cols, gamma, beta, eps, y, ldy,
+                                   mean_out, rstd_out, stream);
 }
 
 }  // extern "C"

@@ -239,43 +239,79 @@ class HaloPadPlan:
         return out
 
 
+_LN_DTYPES = {
+    torch.float32: _lib.DDL_DT_F32,
+    torch.bfloat16: _lib.DDL_DT_BF16,
+    torch.float16: _lib.DDL_DT_F16,
+}
+
+
+def _ln_rows(x2d, name):
+    """dtype code and row pitch of a 2-D LayerNorm operand (last stride 1)."""
+    dt = _LN_DTYPES.get(x2d.dtype)
+    if dt is None or x2d.dim() != 2 or (x2d.shape[1] > 1 and x2d.stride(1) != 1):
+        raise ValueError(f"{name}: need a 2-D float32, bfloat16 or float16 tensor with unit column stride")
+    return dt, (x2d.stride(0) if x2d.shape[0] > 1 else x2d.shape[1])
+
+
+def _ln_params(x2d, gamma, beta, name):
+    for p in (gamma, beta):
+        if p is not None and (p.dtype != x2d.dtype or p.numel() != x2d.shape[1] or not p.is_contiguous()):
+            raise ValueError(f"{name}: gamma / beta must be contiguous, of the input's dtype, with `cols` elements")
+
+
 def ln_partial_stats(x2d, out=None):
-    """{mean, M2} per row of a [rows, cols] fp32 view (last stride 1)."""
+    """{mean, M2} per row of a [rows, cols] view (last stride 1), fp32."""
     _require_gpu(x2d)
-    if x2d.dtype != torch.float32 or x2d.dim() != 2 or (x2d.shape[1] > 1 and x2d.stride(1) != 1):
-        raise ValueError("ln_partial_stats: need a 2-D fp32 tensor with unit column stride")
+    dt, ld = _ln_rows(x2d, "ln_partial_stats")
     rows, cols = x2d.shape
     if out is None:
         out = torch.empty((rows, 2), dtype=torch.float32, device=x2d.device)
-    rc = _lib.load().ddl_ln_partial_stats_f32(x2d.data_ptr(), rows, cols, x2d.stride(0) if rows > 1 else cols,
-                                              out.data_ptr(), _stream())
-    _lib.check(rc, "ddl_ln_partial_stats_f32")
+    rc = _lib.load().ddl_ln_partial_stats(x2d.data_ptr(), dt, rows, cols, ld, out.data_ptr(), _stream())
+    _lib.check(rc, "ddl_ln_partial_stats")
     return out
 
 
-def ln_normalize_affine(x2d, part_stats, part_cols, gamma, beta, eps, want_stats=False):
-    """Combines [P, rows, 2] partial statistics and normalises x2d; returns y (and mean, rstd)."""
+def ln_normalize_affine(x2d, part_stats, part_cols, gamma, beta, eps, want_stats=False, part_cols_arr=None):
+    """Combines [P, rows, 2] partial statistics and normalises x2d; returns y
+    (and mean, rstd).  ``part_cols_arr``: ``part_cols`` already converted with
+    ``_lib.i64_array`` (callers that run every step keep it)."""
     _require_gpu(x2d, part_stats, gamma, beta)
-    if x2d.dtype != torch.float32 or x2d.dim() != 2 or (x2d.shape[1] > 1 and x2d.stride(1) != 1):
-        raise ValueError("ln_normalize_affine: need a 2-D fp32 tensor with unit column stride")
+    dt, ld = _ln_rows(x2d, "ln_normalize_affine")
     rows, cols = x2d.shape
     nparts = len(part_cols)
     if part_stats.dtype != torch.float32 or tuple(part_stats.shape) != (nparts, rows, 2) or \
        not part_stats.is_contiguous():
         raise ValueError(f"ln_normalize_affine: part_stats must be contiguous fp32 [{nparts}, {rows}, 2]")
-    for p in (gamma, beta):
-        if p is not None and (p.dtype != torch.float32 or p.numel() != cols or not p.is_contiguous()):
-            raise ValueError("ln_normalize_affine: gamma / beta must be contiguous fp32 with `cols` elements")
-    y = torch.empty((rows, cols), dtype=torch.float32, device=x2d.device)
+    _ln_params(x2d, gamma, beta, "ln_normalize_affine")
+    y = torch.empty((rows, cols), dtype=x2d.dtype, device=x2d.device)
     mean = rstd = None
     if want_stats:
         mean = torch.empty((rows,), dtype=torch.float32, device=x2d.device)
         rstd = torch.empty((rows,), dtype=torch.float32, device=x2d.device)
-    rc = _lib.load().ddl_ln_normalize_affine_f32(x2d.data_ptr(), rows, cols, x2d.stride(0) if rows > 1 else cols,
-                                                 part_stats.data_ptr(), nparts, _lib.i64_array(part_cols),
-                                                 _ptr(gamma), _ptr(beta), float(eps), y.data_ptr(), cols,
-                                                 _ptr(mean), _ptr(rstd), _stream())
-    _lib.check(rc, "ddl_ln_normalize_affine_f32")
+    if part_cols_arr is None:
+        part_cols_arr = _lib.i64_array(part_cols)
+    rc = _lib.load().ddl_ln_normalize_affine(x2d.data_ptr(), dt, rows, cols, ld, part_stats.data_ptr(), nparts,
+                                             part_cols_arr, _ptr(gamma), _ptr(beta), float(eps), y.data_ptr(), cols,
+                                             _ptr(mean), _ptr(rstd), _stream())
+    _lib.check(rc, "ddl_ln_normalize_affine")
+    return (y, mean, rstd) if want_stats else y
+
+
+def layer_norm(x2d, gamma, beta, eps, want_stats=False):
+    """Layer norm of rows held whole by this worker, one launch; returns y (and mean, rstd)."""
+    _require_gpu(x2d, gamma, beta)
+    dt, ld = _ln_rows(x2d, "layer_norm")
+    rows, cols = x2d.shape
+    _ln_params(x2d, gamma, beta, "layer_norm")
+    y = torch.empty((rows, cols), dtype=x2d.dtype, device=x2d.device)
+    mean = rstd = None
+    if want_stats:
+        mean = torch.empty((rows,), dtype=torch.float32, device=x2d.device)
+        rstd = torch.empty((rows,), dtype=torch.float32, device=x2d.device)
+    rc = _lib.load().ddl_layer_norm(x2d.data_ptr(), dt, rows, cols, ld, _ptr(gamma), _ptr(beta), float(eps),
+                                    y.data_ptr(), cols, _ptr(mean), _ptr(rstd), _stream())
+    _lib.check(rc, "ddl_layer_norm")
     return (y, mean, rstd) if want_stats else y
 
 

@@ -15,6 +15,7 @@ import torch
 import torch.nn.functional as F
 
 from .. import hip_ops
+from ..backends.stub_hip import buffer as _buffer
 from ..utilities.slicing import assemble_slices
 from ..utilities.slicing import compute_nd_slice_shape
 from ..utilities.torch import TensorStructure
@@ -208,9 +209,6 @@ class DistributedFeatureConvBase(Module, HaloMixin, ConvMixin):
         if total_padding.sum() == 0 and self.P_x.size == 1:
             return input
         if getattr(transport, "ghosts_preloaded", False):
-            # The four pooled halo buffers are shared by all dimensions
-            # (reference buffer_allocator.py:69-74), so a fused pass over all
-            # dimensions needs its own slab per (dimension, side).
             ghost, bulk = self._fused_slabs(input)
             exchanged = _HaloStaging.apply(input, self._staging_plan, ghost, bulk)
         else:
@@ -219,19 +217,28 @@ class DistributedFeatureConvBase(Module, HaloMixin, ConvMixin):
         return exchanged[self.needed_slices]
 
     def _fused_slabs(self, input):
+        """Ghost and bulk slabs of the fused pass as ``[dim][side]`` tables of
+        views into pooled buffers.  The halo layer's four buffers are shared by
+        all dimensions (reference buffer_allocator.py:69-74), which only works
+        when dimensions are exchanged one after the other; one pass over all
+        dimensions needs a slab per (dimension, side, kind), so it asks the
+        same buffer manager for that many buffers (the first four are the halo
+        layer's own: the two ways of staging never run together)."""
         plan = self._staging_plan
         slabs = getattr(self, "_fused_slab_cache", None)
-        key = (tuple(input.shape), input.dtype)
+        key = (tuple(input.shape), input.dtype, _buffer.reallocations())
         if slabs is None or slabs[0] != key:
-            ghost, bulk = [], []
-            for d in range(plan.ndim):
-                grow, brow = [], []
-                for s in range(2):
-                    gs, bs = plan.slab_shape(d, s, "ghost"), plan.slab_shape(d, s, "bulk")
-                    grow.append(None if gs is None else torch.zeros(gs, dtype=input.dtype, device=input.device))
-                    brow.append(None if bs is None else torch.empty(bs, dtype=input.dtype, device=input.device))
-                ghost.append(grow)
-                bulk.append(brow)
+            wanted = [(d, s, kind, plan.slab_shape(d, s, kind))
+                      for d in range(plan.ndim) for s in range(2) for kind in ("ghost", "bulk")]
+            wanted = [w for w in wanted if w[3] is not None]
+            pool = self.buffer_manager.request_buffers(len(wanted), dtype=input.dtype)
+            for buf, w in zip(pool, wanted):
+                buf.allocate_view(w[3])        # may reallocate: take the views only afterwards
+            ghost = [[None, None] for _ in range(plan.ndim)]
+            bulk = [[None, None] for _ in range(plan.ndim)]
+            for buf, (d, s, kind, shape) in zip(pool, wanted):
+                (ghost if kind == "ghost" else bulk)[d][s] = buf.get_view(shape)
+            key = (tuple(input.shape), input.dtype, _buffer.reallocations())
             slabs = self._fused_slab_cache = (key, ghost, bulk)
         return slabs[1], slabs[2]
 

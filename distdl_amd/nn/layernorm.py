@@ -5,7 +5,11 @@ the distributed branch (reference :295-309: local mean, all-reduce, local mean
 of squared deviations, all-reduce, normalise, affine -- six or more elementwise
 kernels and two collectives) runs here as two HIP kernels around ONE gather of
 per-row ``{mean, M2}`` pairs; the combination rule reproduces the reference's
-mean of local means and mean of local variances exactly.
+mean of local means and mean of local variances exactly.  When the normalised
+dimensions are not partitioned the reference calls
+``torch.nn.functional.layer_norm`` (:310-319); here that is one HIP kernel.
+Inputs may be float32, bfloat16 or float16 (sums are float32); the backward
+kernels are float32 only.
 """
 
 import numbers
@@ -13,6 +17,7 @@ import numbers
 import numpy as np
 import torch
 
+from .. import _lib
 from .. import hip_ops
 from ..utilities.slicing import compute_subshape
 from ..utilities.slicing import range_index
@@ -34,21 +39,31 @@ class _LayerNormShard(torch.autograd.Function):
     (nn/layernorm.py:230-247, 295-309), whose all-reduces are self-adjoint."""
 
     @staticmethod
-    def forward(ctx, input, weight, bias, P_reduce, part_cols, eps):
+    def forward(ctx, input, weight, bias, P_reduce, part_cols, eps, part_cols_arr=None, grad_mode=True):
         x = input.detach()
         cols = int(part_cols[P_reduce.rank if P_reduce.active else 0])
         x2d = x.reshape(-1, cols)
         if x2d.shape[1] > 1 and x2d.stride(1) != 1:
             x2d = x2d.contiguous()
-        stats = hip_ops.ln_partial_stats(x2d)
-        if len(part_cols) > 1:
-            gathered = P_reduce._world.transport.allgather(P_reduce, stats, tag=STATS_TAG)
-            gathered = gathered.contiguous()
-        else:
-            gathered = stats.unsqueeze(0)
         gamma = None if weight is None else weight.detach().reshape(-1)
         beta = None if bias is None else bias.detach().reshape(-1)
-        y, mean, rstd = hip_ops.ln_normalize_affine(x2d, gathered, part_cols, gamma, beta, eps, want_stats=True)
+        # mean and rstd are only kept when a gradient can be asked for (``grad_mode``: whether autograd was
+        # recording when the layer was called; inside ``forward`` it never is)
+        keep = grad_mode and any(ctx.needs_input_grad[:3])
+        if len(part_cols) > 1:
+            stats = hip_ops.ln_partial_stats(x2d)
+            gathered = P_reduce._world.transport.allgather(P_reduce, stats, tag=STATS_TAG)
+            gathered = gathered.contiguous()
+            res = hip_ops.ln_normalize_affine(x2d, gathered, part_cols, gamma, beta, eps, want_stats=keep,
+                                              part_cols_arr=part_cols_arr)
+        else:
+            res = hip_ops.layer_norm(x2d, gamma, beta, eps, want_stats=keep)
+        if not keep:
+            return res.view(input.shape)
+        y, mean, rstd = res
+        if x2d.dtype != torch.float32:
+            raise NotImplementedError(f"DistributedLayerNorm backward kernels are fp32 only, got {x2d.dtype}; "
+                                      "run the forward under torch.no_grad() or in float32")
         ctx.save_for_backward(x2d, mean, rstd, gamma)
         ctx.P_reduce, ctx.nparts, ctx.cols = P_reduce, len(part_cols), cols
         ctx.param_shapes = (None if weight is None else weight.shape, None if bias is None else bias.shape)
@@ -85,7 +100,7 @@ class _LayerNormShard(torch.autograd.Function):
             dw, db = hip_ops.ln_backward_params(dy2d, x2d, mean, rstd, want_w, want_b)
         dw = None if dw is None else dw.view(w_shape)
         db = None if db is None else db.view(b_shape)
-        return dx, dw, db, None, None, None
+        return dx, dw, db, None, None, None, None, None
 
 
 class DistributedLayerNorm(Module):
@@ -137,6 +152,8 @@ class DistributedLayerNorm(Module):
         self.part_cols = [int(np.prod(compute_subshape(reduce_shape, idx, self.normalized_shape)))
                           for idx in range_index(reduce_shape)]
         local_norm_shape = compute_subshape(reduce_shape, P_x.index[self.dim_reduce_slice], self.normalized_shape)
+        self._part_cols_arr = _lib.i64_array(self.part_cols)     # what the normalize kernel's entry point takes
+        self._checked_shape = None                               # last input shape found consistent with part_cols
 
         if self.elementwise_affine:
             # Parameters live on the workers with index 0 in every dimension that
@@ -188,17 +205,24 @@ class DistributedLayerNorm(Module):
             return input
         weight = bias = None
         if self.elementwise_affine:
-            if self.weight_buffer is None:
-                weight = self.broadcast(self.weight)
-                bias = self.broadcast(self.bias)
-            else:
+            if self.weight_buffer is not None:
                 weight, bias = self.weight_buffer, self.bias_buffer
                 self.weight_buffer = self.bias_buffer = None
-        if input.dtype != torch.float32:
-            raise NotImplementedError(f"DistributedLayerNorm kernels are fp32 only, got {input.dtype}")
-        local_cols = int(np.prod(input.shape[self.dim_reduce_slice.start - self.P_x.dim:]))
-        mine = self.allreduce.P_allreduce.rank if self.num_reduce > 1 else 0
-        if local_cols != self.part_cols[mine]:
-            raise ValueError(f"input shard has {local_cols} normalised elements, the partition of "
-                             f"normalized_shape={self.normalized_shape} gives this worker {self.part_cols[mine]}")
-        return _LayerNormShard.apply(input, weight, bias, self.allreduce.P_allreduce, self.part_cols, self.eps)
+            elif self.broadcast.identity:      # every worker stores its own parameters: nothing to fetch
+                weight, bias = self.weight, self.bias
+            else:
+                weight = self.broadcast(self.weight)
+                bias = self.broadcast(self.bias)
+        if input.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+            raise NotImplementedError(f"DistributedLayerNorm kernels take float32, bfloat16 and float16, got {input.dtype}")
+        if weight is not None and weight.dtype != input.dtype:
+            raise ValueError(f"DistributedLayerNorm parameters are {weight.dtype}, the input is {input.dtype}")
+        if input.shape != self._checked_shape:
+            local_cols = int(np.prod(input.shape[self.dim_reduce_slice.start - self.P_x.dim:]))
+            mine = self.allreduce.P_allreduce.rank if self.num_reduce > 1 else 0
+            if local_cols != self.part_cols[mine]:
+                raise ValueError(f"input shard has {local_cols} normalised elements, the partition of "
+                                 f"normalized_shape={self.normalized_shape} gives this worker {self.part_cols[mine]}")
+            self._checked_shape = input.shape
+        return _LayerNormShard.apply(input, weight, bias, self.allreduce.P_allreduce, self.part_cols, self.eps,
+                                     self._part_cols_arr, torch.is_grad_enabled())

@@ -42,6 +42,12 @@ const char* ddl_version(void);
 /* Message for the last non-zero return on the calling thread ("" if none). */
 const char* ddl_last_error(void);
 
+/* Enqueues a kernel that does nothing, `workgroups` workgroups of `threads`
+ * threads (1..1024).  No counterpart in the reference: a measurement aid that
+ * gives the time a launch of that size costs on its own, the floor under every
+ * small kernel of this library. */
+int ddl_probe_launch(int64_t workgroups, int threads, void* stream);
+
 /* ------------------------------------------------------------------------ *
  * Box copies (Repartition / HaloExchange pack, unpack, self-copy)
  * ------------------------------------------------------------------------ */
@@ -162,18 +168,17 @@ int ddl_halo_pad_exchange(const void* x, void* xpad, const int64_t* x_shape,
                           int kernel, void* stream);
 
 /* ------------------------------------------------------------------------ *
- * DistributedLayerNorm local shard (fp32)
+ * DistributedLayerNorm local shard (fp32, bf16 or fp16 elements; fp32 sums)
  * ------------------------------------------------------------------------ */
 
 /* Per-row partial statistics of the local shard x[rows, cols] (row stride
- * `ld` elements): stats[r] = { mean_r, M2_r } with M2 = sum (x - mean_r)^2,
- * fp32 accumulation.  One read of x.
+ * `ld` elements, dtype DDL_DT_F32 / _BF16 / _F16): stats[r] = { mean_r, M2_r }
+ * with M2 = sum (x - mean_r)^2, fp32 accumulation.  One read of x.
  *
  * Replaces the local halves of DistributedLayerNorm._compute_mean / _compute_var,
  *   nn/layernorm.py:230 (input.mean(dim, keepdim)) and :246-247. */
-int ddl_ln_partial_stats_f32(const float* x, int64_t rows, int64_t cols,
-                             int64_t ld, float* stats /*[rows][2]*/,
-                             void* stream);
+int ddl_ln_partial_stats(const void* x, int dtype, int64_t rows, int64_t cols,
+                         int64_t ld, float* stats /*[rows][2]*/, void* stream);
 
 /* Combines the partial statistics of the `nparts` workers that share a row and
  * normalises the local shard:
@@ -183,10 +188,33 @@ int ddl_ln_partial_stats_f32(const float* x, int64_t rows, int64_t cols,
  * which is the reference's mean-of-local-means / mean-of-local-variances,
  *   nn/layernorm.py:230-233, :246-247, :298-302, :309,
  * with the two all-reduces replaced by one gather of {mean, M2}.
- *   part_stats [nparts][rows][2]  (this worker's own partials included)
+ *   x, y, gamma, beta   elements of `dtype`
+ *   part_stats [nparts][rows][2]  fp32 (this worker's own partials included)
  *   part_cols  [nparts]           host array: columns n_p held by each worker
  *   gamma/beta [cols] or NULL (both or neither)
- *   mean_out/rstd_out [rows] or NULL: the combined statistics, for backward. */
+ *   mean_out/rstd_out [rows] fp32 or NULL: the combined statistics, for backward. */
+int ddl_ln_normalize_affine(const void* x, int dtype, int64_t rows, int64_t cols,
+                            int64_t ld, const float* part_stats,
+                            int nparts, const int64_t* part_cols,
+                            const void* gamma, const void* beta,
+                            float eps, void* y, int64_t ldy,
+                            float* mean_out, float* rstd_out, void* stream);
+
+/* Layer norm of rows that this worker holds whole, in ONE launch and one read
+ * of x:  y = (x - mean) / sqrt(var + eps) [* gamma + beta]  with the row's own
+ * mean and biased variance.  Replaces
+ *   torch.nn.functional.layer_norm(input, normalized_shape, weight, bias, eps)
+ * in the branch of DistributedLayerNorm.forward that runs when the normalised
+ * dimensions are not partitioned, nn/layernorm.py:310-319.  Arguments as above. */
+int ddl_layer_norm(const void* x, int dtype, int64_t rows, int64_t cols, int64_t ld,
+                   const void* gamma, const void* beta, float eps,
+                   void* y, int64_t ldy, float* mean_out, float* rstd_out,
+                   void* stream);
+
+/* The fp32 forms of the first two (dtype = DDL_DT_F32). */
+int ddl_ln_partial_stats_f32(const float* x, int64_t rows, int64_t cols,
+                             int64_t ld, float* stats /*[rows][2]*/,
+                             void* stream);
 int ddl_ln_normalize_affine_f32(const float* x, int64_t rows, int64_t cols,
                                 int64_t ld, const float* part_stats,
                                 int nparts, const int64_t* part_cols,

@@ -42,6 +42,29 @@ def forward_shards(shards, gammas, betas, eps, num_norm_dims=1, dtype=np.float32
     return outs
 
 
+def forward_rank(x, peer_mean_sum, peer_var_sum, num_reduce, gamma, beta, eps, num_norm_dims=1, dtype=np.float32):
+    """One worker's share of ``forward_shards``, in the reference's order of
+    operations, with the two all-reduces replaced by what they deliver: the sum
+    of the OTHER workers' local means (``peer_mean_sum``) and of their local
+    mean squared deviations from the global mean (``peer_var_sum``), both of
+    shape ``x.shape[:-num_norm_dims] + (1,) * num_norm_dims``.
+
+        m_loc = x.mean(dims)                 mean = (m_loc + peers) / P     :230-233
+        v_loc = ((x - mean)**2).mean(dims)   var  = (v_loc + peers) / P     :246-247
+        y = (x - mean) / sqrt(var + eps);  y = weight * y + bias             :302, :309
+
+    Pinned in tests/test_oracle_golden.py against ``forward_shards``."""
+    axes = tuple(range(-num_norm_dims, 0))
+    x = np.asarray(x, dtype=dtype)
+    P = dtype(num_reduce)
+    mean = (x.mean(axis=axes, keepdims=True, dtype=dtype) + peer_mean_sum) / P
+    var = (((x - mean) ** 2).mean(axis=axes, keepdims=True, dtype=dtype) + peer_var_sum) / P
+    y = (x - mean) / np.sqrt(var + dtype(eps))
+    if gamma is not None:
+        y = np.asarray(gamma, dtype=dtype) * y + np.asarray(beta, dtype=dtype)
+    return y.astype(dtype)
+
+
 def partial_stats(shard, num_norm_dims=1, dtype=np.float64):
     """Per-row {local mean, local sum of squared deviations from it}."""
     axes = tuple(range(-num_norm_dims, 0))

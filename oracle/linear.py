@@ -28,9 +28,17 @@ def f32_to_bf16_bits(x):
 def linear(x_bits, w_bits, bias_bits=None, dtype=np.float32):
     x = bf16_bits_to_f32(x_bits).astype(dtype)
     w = bf16_bits_to_f32(w_bits).astype(dtype)
+    return linear_values(x, w, None if bias_bits is None else bf16_bits_to_f32(bias_bits).astype(dtype))
+
+
+def linear_values(x, w, bias=None):
+    """``linear`` on operands that are already values (any float dtype): the
+    product and bias add alone, without the conversion from bit patterns.
+    ``linear(xb, wb, bb, dtype)`` equals ``linear_values`` of the converted
+    operands by construction; used where only the arithmetic is to be timed."""
     y = x.reshape(-1, x.shape[-1]) @ w.T
-    if bias_bits is not None:
-        y = y + bf16_bits_to_f32(bias_bits).astype(dtype)
+    if bias is not None:
+        y = y + bias
     return y.reshape(x.shape[:-1] + (w.shape[0],))
 
 

@@ -84,12 +84,13 @@ def test_layernorm_config1_rank0(ops):
 
 
 @pytest.mark.parametrize("cols", [[4, 4], [64, 64, 64], [300, 212], [1000, 24], [2048], [7, 9], [4100, 4100],
-                                  [20000, 100], [8] * 70, [4] * 200])
+                                  [20000, 100], [8] * 70, [4] * 200, [2052, 4096], [8192, 16384], [16388, 12000],
+                                  [4101, 33]])
 @pytest.mark.parametrize("affine", [True, False])
 def test_layernorm_shapes_and_paths(ops, cols, affine):
-    """Register path (aligned, <= 2048 columns), LDS-staged path (unaligned or
-    long rows), streaming path (rows longer than the LDS stage), unequal widths,
-    more workers per row than a wavefront has lanes."""
+    """Wavefront rows (aligned, <= 2048 columns), workgroup rows (aligned, <=
+    16384 columns), streamed rows (longer, with and without four-element
+    accesses), unequal widths, more workers per row than a wavefront has lanes."""
     rng = np.random.default_rng(sum(cols))
     rows = 37
     shards = [(rng.standard_normal((rows, c)) * 3 + 1.5).astype(np.float32) for c in cols]
@@ -98,6 +99,112 @@ def test_layernorm_shapes_and_paths(ops, cols, affine):
     beta = (0.1 * rng.standard_normal(total)).astype(np.float32) if affine else None
     for live in {0, len(cols) - 1}:
         _ln_case(ops, shards, gamma, beta, 1e-5, live=live)
+
+
+@pytest.mark.parametrize("cols", [1, 7, 64, 256, 300, 1024, 2048, 2052, 4096, 8192, 12000, 16384, 16388, 40001])
+@pytest.mark.parametrize("affine", [True, False])
+def test_layer_norm_single_launch_fp32(ops, cols, affine):
+    """Rows held whole by one worker: one kernel, against torch's layer_norm in
+    float64 (the call the reference makes in that branch, nn/layernorm.py:319)
+    and against the oracle with a single shard."""
+    rng = np.random.default_rng(cols)
+    rows = 29
+    x = (rng.standard_normal((rows, cols)) * 2 - 0.7).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(cols)).astype(np.float32) if affine else None
+    beta = (0.1 * rng.standard_normal(cols)).astype(np.float32) if affine else None
+    g = None if gamma is None else torch.from_numpy(gamma).cuda()
+    b = None if beta is None else torch.from_numpy(beta).cuda()
+    y, mean, rstd = ops.layer_norm(torch.from_numpy(x).cuda(), g, b, 1e-5, want_stats=True)
+    torch.cuda.synchronize()
+    exact = F.layer_norm(torch.from_numpy(x).double(), (cols,), None if gamma is None else torch.from_numpy(gamma).double(),
+                         None if beta is None else torch.from_numpy(beta).double(), 1e-5).numpy()
+    oracle = o_ln.forward_shards([x], [gamma], [beta], 1e-5, dtype=np.float64)[0]
+    assert np.allclose(oracle, exact, rtol=1e-12, atol=1e-12)
+    got = y.cpu().numpy().astype(np.float64)
+    assert (np.abs(got - exact) <= LN_RTOL * np.maximum(np.abs(exact), 1.0)).all(), float(np.abs(got - exact).max())
+    m = x.astype(np.float64).mean(axis=1)
+    v = x.astype(np.float64).var(axis=1)
+    assert np.allclose(mean.cpu().numpy(), m, rtol=1e-5, atol=1e-5)
+    assert np.allclose(rstd.cpu().numpy(), 1 / np.sqrt(v + 1e-5), rtol=1e-5)
+    # a strided view (row pitch larger than the row) gives the same bits
+    wide = torch.zeros(rows, cols + 8, device="cuda")
+    wide[:, :cols] = torch.from_numpy(x).cuda()
+    y2 = ops.layer_norm(wide[:, :cols], g, b, 1e-5)
+    assert torch.equal(y2, y)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("cols", [[8], [256], [300], [2048], [6000], [20000], [256, 256, 256, 256], [300, 212], [4100, 4100]])
+def test_layernorm_16_bit_elements(ops, dtype, cols):
+    """bf16 / fp16 inputs, parameters and outputs with fp32 sums: one rounding
+    of the exact result of the reference's op sequence on the same 16-bit
+    inputs (2e-2 relative is the bar for bf16; these stay within 2^-7)."""
+    rng = np.random.default_rng(sum(cols) + len(cols))
+    rows = 21
+    shards_t = [torch.from_numpy((rng.standard_normal((rows, c)) * 2 + 0.5).astype(np.float32)).to(dtype) for c in cols]
+    total = sum(cols)
+    gamma_t = torch.from_numpy((1 + 0.1 * rng.standard_normal(total)).astype(np.float32)).to(dtype)
+    beta_t = torch.from_numpy((0.1 * rng.standard_normal(total)).astype(np.float32)).to(dtype)
+    shards64 = [t.double().numpy() for t in shards_t]
+    offs = np.cumsum([0] + cols)
+    gs = [gamma_t.double().numpy()[offs[p]:offs[p + 1]] for p in range(len(cols))]
+    bs = [beta_t.double().numpy()[offs[p]:offs[p + 1]] for p in range(len(cols))]
+    exact = o_ln.forward_shards(shards64, gs, bs, 1e-5, dtype=np.float64)
+    tol = 2.0 ** -7
+    for live in {0, len(cols) - 1}:
+        x2d = shards_t[live].cuda()
+        g = gamma_t[offs[live]:offs[live + 1]].contiguous().cuda()
+        b = beta_t[offs[live]:offs[live + 1]].contiguous().cuda()
+        if len(cols) == 1:
+            y = ops.layer_norm(x2d, g, b, 1e-5)
+        else:
+            stats = ops.ln_partial_stats(x2d)
+            want_stats = o_ln.partial_stats(shards64[live])
+            assert np.allclose(stats.cpu().numpy()[:, 0], want_stats[:, 0], rtol=1e-5, atol=1e-5)
+            parts = [stats if p == live else torch.from_numpy(o_ln.partial_stats(shards64[p]).astype(np.float32)).cuda()
+                     for p in range(len(cols))]
+            y = ops.ln_normalize_affine(x2d, torch.stack(parts).contiguous(), cols, g, b, 1e-5)
+        assert y.dtype == dtype
+        got = y.cpu().double().numpy()
+        assert (np.abs(got - exact[live]) <= tol * np.maximum(np.abs(exact[live]), 1.0)).all()
+
+
+def test_layernorm_layer_single_worker_and_bf16(ops):
+    """The layer on one worker takes the single-launch kernel (the reference's
+    F.layer_norm branch) and is differentiable in fp32; in bf16 it runs forward."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedLayerNorm
+    torch.manual_seed(3)
+    x = torch.randn(6, 10, 96)
+    ref = torch.nn.LayerNorm(96)
+    with torch.no_grad():
+        ref.weight.copy_(1 + 0.1 * torch.randn(96))
+        ref.bias.copy_(0.1 * torch.randn(96))
+
+    def body(P_world):
+        P_x = P_world.create_partition_inclusive([0]).create_cartesian_topology_partition([1, 1, 1])
+        layer = DistributedLayerNorm(P_x, 96)
+        with torch.no_grad():
+            layer.weight.copy_(ref.weight.reshape(1, 1, 96))
+            layer.bias.copy_(ref.bias.reshape(1, 1, 96))
+        xg = x.cuda().requires_grad_(True)
+        y = layer(xg)
+        y.backward(torch.ones_like(y) * 0.5 + y.detach())
+        half = DistributedLayerNorm(P_x, 96, dtype=torch.bfloat16)
+        with torch.no_grad():
+            half.weight.copy_(ref.weight.reshape(1, 1, 96))
+            half.bias.copy_(ref.bias.reshape(1, 1, 96))
+            yh = half(x.cuda().to(torch.bfloat16))
+        return y.detach().cpu(), xg.grad.cpu(), layer.weight.grad.cpu().reshape(-1), yh.float().cpu()
+
+    y, dx, dw, yh = SimWorld(1).run(body)[0]
+    xr = x.clone().requires_grad_(True)
+    yr = ref(xr)
+    yr.backward(torch.ones_like(yr) * 0.5 + yr.detach())
+    assert torch.allclose(y, yr.detach(), rtol=1e-5, atol=1e-5)
+    assert torch.allclose(dx, xr.grad, rtol=1e-4, atol=1e-5)
+    assert torch.allclose(dw, ref.weight.grad, rtol=1e-4, atol=1e-4)
+    assert torch.allclose(yh, yr.detach(), rtol=2e-2, atol=2e-2)
 
 
 def test_layernorm_large_offset_keeps_accuracy(ops):

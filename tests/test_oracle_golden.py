@@ -400,6 +400,23 @@ def test_layernorm_backward_oracle_matches_autograd_of_the_reference_sequence(wi
         assert np.allclose(np.concatenate(dgs), g.grad.numpy(), rtol=1e-9, atol=1e-11)
 
 
+def test_layernorm_forward_rank_equals_forward_shards():
+    """The one-worker form used for the CPU baseline is the all-worker form seen from worker 0."""
+    rng = np.random.default_rng(8)
+    widths = [5, 7, 4]
+    shards = [rng.standard_normal((3, 6, w)) for w in widths]
+    gammas = [rng.standard_normal(w) for w in widths]
+    betas = [rng.standard_normal(w) for w in widths]
+    want = o_ln.forward_shards(shards, gammas, betas, 1e-5, dtype=np.float64)
+    P = len(widths)
+    mean = sum(s.mean(axis=-1, keepdims=True) for s in shards) / P
+    for live in range(P):
+        peer_mean = sum(s.mean(axis=-1, keepdims=True) for p, s in enumerate(shards) if p != live)
+        peer_var = sum(((s - mean) ** 2).mean(axis=-1, keepdims=True) for p, s in enumerate(shards) if p != live)
+        got = o_ln.forward_rank(shards[live], peer_mean, peer_var, P, gammas[live], betas[live], 1e-5, dtype=np.float64)
+        assert np.allclose(got, want[live], rtol=1e-12, atol=1e-12)
+
+
 def test_embedding_backward_oracle_matches_torch_autograd():
     torch.manual_seed(6)
     table = torch.randn(20, 5, dtype=torch.float64, requires_grad=True)
