@@ -11,41 +11,55 @@
 //   workgroup  512 threads = 8 wavefronts (2 along m x 4 along n), tile
 //              256(m) x 256(n); two wavefronts share a SIMD so that one can
 //              issue MFMAs while the other waits
-//   wavefront  128(m) x 64(n) = 4 x 2 tiles of v_mfma_f32_32x32x16_bf16, 128 fp32
-//              accumulators per lane
+//   wavefront  128(m) x 64(n) = 8 x 4 tiles of v_mfma_f32_16x16x32_bf16, 128 fp32
+//              accumulators per lane.  On random operands the chip is limited
+//              by power, and this instruction delivers about 14 % more flop/s
+//              under that limit than the 32x32x16 one (it moves half as many
+//              accumulator bytes per flop)
 //   LDS        ring of five operand tiles (W0 X0 W1 X1 W2 | X2 W3 ...), each
 //              256 rows x 64 k = 32 KiB, 160 KiB in all.  Rows are 128 B; the
 //              16-byte chunk index is XOR-ed with ((row >> 1) & 7): the 16
 //              lanes served per LDS cycle read 16 consecutive rows, and
 //              (row & 1, (row >> 1) & 7) is distinct for each, so they cover all
-//              64 banks
+//              64 banks (an MFMA operand piece is 16 rows x 32 k: lane l reads
+//              row l % 16, chunk l / 16 of the k-step)
 //   global     tiles go from global memory straight into LDS
 //              (buffer_load_dwordx4 ... lds: each wavefront instruction fills
 //              1 KiB = 8 rows, the eight lanes of a row fetching one whole
 //              128-byte line; half-line requests run at little more than half
 //              the rate).  No staging registers, no LDS stores, one 32-bit
 //              offset per lane and the k offset in a scalar
-//   schedule   per k-tile of 64: four k-steps of 8 MFMAs, one LDS fragment
-//              read issued behind each MFMA (the fragments of the next k-step,
-//              crossing into tile t+1 at the end).  W(t+2) is requested during
-//              k-step 0 into the slot X(t-1) left, X(t+2) during k-step 3 into
-//              the slot of W(t); before k-step 3 each wavefront waits for its
-//              own requests of tile t+1 and all its LDS reads, then one
-//              barrier: tile t+1 is readable, tile t's slots are free
+//   schedule   per k-tile of 64: two k-steps of 32 MFMAs, one LDS fragment
+//              read issued behind every second MFMA (the fragments of the next
+//              k-step, crossing into tile t+1 in the second k-step).  W(t+2) is
+//              requested during k-step 0 into the slot X(t-1) left, X(t+2)
+//              during k-step 1 into the slot of W(t); between the two k-steps
+//              each wavefront waits for its own requests of tile t+1 and all
+//              its LDS reads, then one barrier: tile t+1 is readable, tile t's
+//              slots are free
 //   epilogue   bias add and bf16 rounding in registers, then each wavefront
 //              transposes its block through LDS so that rows of y are written
 //              in 16-byte pieces, whole 128-byte lines per instruction
-//   launch     workgroup ids are regrouped so that the 32 workgroups resident
-//              on one XCD cover a compact patch of the tile grid and share
-//              their operand panels in that XCD's L2
+//   launch     one workgroup per CU is resident, so the tiles run in rounds of
+//              one per CU and a last round that is only partly filled costs as
+//              much as a full one; when it pays, the columns are split between
+//              256-wide tiles (whole rounds) and 192-wide tiles (4 x 2
+//              wavefronts of 64 x 96), whose rounds are shorter, in a launch of
+//              their own.  (Both kinds in one grid, so that a CU starts on a
+//              narrow tile the moment its wide one is stored, measured 2 %
+//              slower: the workgroups of an XCD then drift apart in k and share
+//              fewer operand lines in its L2.)  Workgroup ids are regrouped so
+//              that the 32 workgroups resident on one XCD cover a compact patch
+//              of the tile grid and share their operand panels in that XCD's L2
 #include "ddl_common.h"
+#include <atomic>
 #include <type_traits>
 
 namespace ddl {
 namespace {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
-typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 constexpr int BK = 64;
 constexpr int kMaxTileRows = 256;                    // rows of an operand tile: 256 of x; 256 or 192 of w
@@ -72,15 +86,15 @@ __device__ inline void dma16(__amdgpu_buffer_rsrc_t buffer, int voffset, int sof
     __builtin_amdgcn_raw_ptr_buffer_load_lds(buffer, (lds_ptr)dst, 16, voffset, soffset, 0, 0);
 }
 
-// acc += a . b (32 x 32 x 16, bf16 in, fp32 accumulate).  Written as assembly
+// acc += a . b (16 x 16 x 32, bf16 in, fp32 accumulate).  Written as assembly
 // so that the accumulators live in the accumulation registers ("a" operands):
 // left to itself the compiler keeps them in the vector registers next to the
 // fragments, which measures 2 % slower.  The compiler still tracks the
 // operands (it waits for the LDS reads that produce a and b); what it does not
 // do for assembly is pad the distance between an MFMA and a later non-MFMA
 // read of acc -- the kernel does that once, in front of the epilogue.
-__device__ inline void mfma_32x32x16(floatx16& acc, const bf16x8& a, const bf16x8& b) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+__device__ inline void mfma_16x16x32(floatx4& acc, const bf16x8& a, const bf16x8& b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
 
 // s_waitcnt immediate (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4,
@@ -88,20 +102,34 @@ __device__ inline void mfma_32x32x16(floatx16& acc, const bf16x8& a, const bf16x
 // and all LDS reads have returned.
 constexpr int wait_vm_lgkm0(int n) { return 0x0070 | (n & 15) | ((n >> 4) << 14); }
 
-// NWM x NWN wavefronts, each owning TM x TN sub-tiles of 32 x 32: the workgroup
-// tile is (32 NWM TM) x (32 NWN TN).
+// NWM x NWN wavefronts, each owning TM x TN sub-tiles of 16 x 16: the workgroup
+// tile is (16 NWM TM) x (16 NWN TN).
+// The columns of the output that one kind of tile covers: operands and result
+// already offset to the first of those columns.
+struct Part {
+    const uint16_t* x;
+    const uint16_t* w;
+    const uint16_t* bias;
+    uint16_t* y;
+    int64_t M, N, K, ldx, ldw, ldy;
+    int tiles_m, tiles_n, vec_store;
+};
+
 template <int NWM, int NWN, int TM, int TN>
-__global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
-                                                               const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
-                                                               int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw,
-                                                               int64_t ldy, int tiles_m, int tiles_n, int vec_store) {
-    extern __shared__ __attribute__((aligned(16))) char lds[];
+__device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* lds) {
+    static_assert(NWM * NWN == 8, "eight wavefronts per workgroup");
+    const uint16_t* __restrict__ x = part.x;
+    const uint16_t* __restrict__ w = part.w;
+    const uint16_t* __restrict__ bias = part.bias;
+    uint16_t* __restrict__ y = part.y;
+    const int64_t M = part.M, N = part.N, K = part.K, ldx = part.ldx, ldw = part.ldw, ldy = part.ldy;
+    const int tiles_m = part.tiles_m, tiles_n = part.tiles_n, vec_store = part.vec_store;
 
     // XCD-aware tile assignment: hardware deals workgroup ids round-robin over
     // the XCDs, so id % 8 names the XCD.  Give each XCD a contiguous range of
     // the tile sequence, and walk that sequence in bands of 8 m-tiles.
     const int ntiles = tiles_m * tiles_n;
-    int id = blockIdx.x;
+    int id = tile_id;
     {
         const int per = ntiles / kXcds, main = per * kXcds;
         if (id < main) id = (id % kXcds) * per + id / kXcds;
@@ -114,24 +142,24 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
     const int tm = band_m0 + in_band % band_h;
     const int tn = in_band / band_h;
 
-    constexpr int BM = 32 * NWM * TM, BN = 32 * NWN * TN;
+    constexpr int BM = 16 * NWM * TM, BN = 16 * NWN * TN;
     static_assert(BM <= kMaxTileRows && BN <= kMaxTileRows, "operand tile larger than a ring slot");
     const int64_t m0 = static_cast<int64_t>(tm) * BM, n0 = static_cast<int64_t>(tn) * BN;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // the same in all lanes: keep it scalar
     constexpr int NW = NWM * NWN;
     // request instructions (8 rows each) per wavefront for a w tile and an x tile
     constexpr int JW_W = BN / 8 / NW, JW_X = BM / 8 / NW;
     static_assert(JW_W * 8 * NW == BN && JW_X * 8 * NW == BM, "tile rows do not divide among the wavefronts");
-    const int wm = (wave % NWM) * (TM * 32), wn = (wave / NWM) * (TN * 32);   // wavefront origin inside the tile
-    const int l32 = lane & 31, kg = lane >> 5;
+    const int wm = (wave % NWM) * (TM * 16), wn = (wave / NWM) * (TN * 16);   // wavefront origin inside the tile
+    const int l16 = lane & 15, kg = lane >> 4;
 
-    floatx16 acc[TN][TM];           // [n sub-tile][m sub-tile]
+    floatx4 acc[TN][TM];           // [n sub-tile][m sub-tile]
 #pragma unroll
     for (int a = 0; a < TN; ++a)
 #pragma unroll
         for (int b = 0; b < TM; ++b)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
+            for (int e = 0; e < 4; ++e) acc[a][b][e] = 0.f;
 
     // Global -> LDS requests of this lane.  Instruction j of this wavefront
     // fills rows (J wave + j) 8 .. +7 of an operand tile (J instructions per
@@ -193,29 +221,64 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
         }
     };
 
-    // Fragment addresses: row (sub-tile origin + l32), logical chunk 2 ks + kg.
-    // Sub-tile origins are multiples of 32, so the swizzle term is (l32 >> 1) & 7.
-    const int frag_row = l32 * (BK * 2);
-    int sw_off[4];   // byte offset of this lane's chunk in its row, per k-step
+    // Fragment addresses: row (sub-tile origin + l16), logical chunk 4 ks + kg.
+    // Sub-tile origins are multiples of 16, so the swizzle term is (l16 >> 1) & 7.
+    const int frag_row = l16 * (BK * 2);
+    int sw_off[2];   // byte offset of this lane's chunk in its row, per k-step
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) sw_off[ks] = ((2 * ks + kg) ^ ((l32 >> 1) & 7)) << 4;
+    for (int ks = 0; ks < 2; ++ks) sw_off[ks] = ((4 * ks + kg) ^ ((l16 >> 1) & 7)) << 4;
     const int off_w = wn * (BK * 2) + frag_row;
     const int off_x = wm * (BK * 2) + frag_row;
 
-    auto read_frag = [&](const char* wt, const char* xt, int ks, bf16x8 (&fa)[TN], bf16x8 (&fb)[TM], int i) {
+    // The operand with more pieces per wavefront runs in the outer loop of a
+    // k-step: a piece of it is used by a few consecutive MFMAs and is dead
+    // afterwards, so that its successor can take its registers; the pieces of the
+    // other operand stay live for the whole k-step.
+    constexpr bool kOuterX = TM >= TN;
+    constexpr int NI = kOuterX ? TN : TM;    // pieces of the inner operand
+    constexpr int NMFMA = TN * TM, NREAD = TN + TM;
+    static_assert(2 * NREAD - 1 < NMFMA, "a k-step has too few MFMAs to hide its fragment reads");
+
+    // Read number r of a k-step (issued behind MFMA 2 r + 1), in the order the
+    // next k-step needs the pieces: outer 0, all inner ones, outer 1, 2, ...
+    auto read_frag = [&](const char* wt, const char* xt, int ks, bf16x8 (&fa)[TN], bf16x8 (&fb)[TM], int r) {
         const int sw = sw_off[ks];
-        if (i < TN)
-            fa[i] = *reinterpret_cast<const bf16x8*>(wt + off_w + i * (32 * BK * 2) + sw);
+        const bool outer = r == 0 || r > NI;
+        const int idx = r == 0 ? 0 : (r <= NI ? r - 1 : r - NI);
+        const bool is_x = outer == kOuterX;
+        if (is_x)
+            fb[idx] = *reinterpret_cast<const bf16x8*>(xt + off_x + idx * (16 * BK * 2) + sw);
         else
-            fb[i - TN] = *reinterpret_cast<const bf16x8*>(xt + off_x + (i - TN) * (32 * BK * 2) + sw);
+            fa[idx] = *reinterpret_cast<const bf16x8*>(wt + off_w + idx * (16 * BK * 2) + sw);
     };
 
-    constexpr int kGapW = (TN * TM) / JW_W, kGapX = (TN * TM) / JW_X;   // MFMAs from one request instruction to the next
+    // Request instructions go behind even MFMAs (the fragment reads take the odd
+    // ones).  Those of W(t+2) have a tile and a half to land and are spread over
+    // their k-step; those of X(t+2) have one tile, so they go out in the first
+    // slots after the barrier that frees their ring slot.
+    constexpr int kGapW = NMFMA / JW_W;   // MFMAs from one request instruction of W to the next
+    static_assert(kGapW % 2 == 0 && kGapW >= 2 && 2 * JW_X <= NMFMA, "request slots must fall on even MFMAs");
     auto unit_off = [](int slot) { return (slot >= kUnits ? slot - kUnits : slot) * kUnitBytes; };
     int s0 = 0;   // ring slot of W(t); X(t), W(t+1), X(t+1), W(t+2) follow
     bf16x8 fa[2][TN], fb[2][TM];
 
-    // One k-tile = four k-steps of 16.  On entry the fragments of (t, k-step 0)
+    // One k-step: NMFMA MFMAs on the pieces in fa[cur] / fb[cur]; the pieces
+    // of the next k-step are read from (wt, xt) at k-step `ks_next` into
+    // fa[cur ^ 1] / fb[cur ^ 1]; `request(j)` issues request instruction j of
+    // `nreq`, behind MFMA `first + j * gap`.
+    auto k_step = [&](int cur, const char* wt, const char* xt, int ks_next, int first, int gap, int nreq, auto request) {
+#pragma unroll
+        for (int q = 0; q < NMFMA; ++q) {
+            const int o = q / NI, i = q % NI;
+            const int a = kOuterX ? i : o, b = kOuterX ? o : i;
+            mfma_16x16x32(acc[a][b], fa[cur][a], fb[cur][b]);
+            if ((q & 1) && (q >> 1) < NREAD) read_frag(wt, xt, ks_next, fa[cur ^ 1], fb[cur ^ 1], q >> 1);
+            if (q >= first && (q - first) % gap == 0 && (q - first) / gap < nreq) request((q - first) / gap);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // One k-tile = two k-steps of 32.  On entry the fragments of (t, k-step 0)
     // are in fa[0] / fb[0] or on their way, W(t+1) and X(t+1) have been
     // requested.  STEADY: tile t+2 exists and is a full tile; its request
     // instructions are spread between the MFMAs.
@@ -228,17 +291,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
         const int w2_off = unit_off(s0 + 4);   // slot of X(t-1), free since the barrier of tile t-1
         const int x2_off = unit_off(s0);       // slot of W(t), free after this tile's barrier
         if (!STEADY && t + 2 < ktiles) request_unit(buf_w, base_w, off_gw, t + 2, w2_off);
-#pragma unroll
-        for (int ks = 0; ks < 3; ++ks) {
-#pragma unroll
-            for (int i = 0; i < TN * TM; ++i) {
-                const int a = i / TM, b = i % TM;
-                mfma_32x32x16(acc[a][b], fa[ks & 1][a], fb[ks & 1][b]);
-                if (i < TN + TM) read_frag(wt, xt, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1], i);
-                if (STEADY && ks == 0 && i % kGapW == kGapW - 1 && i / kGapW < JW_W) request_part(buf_w, off_gw, t + 2, w2_off, i / kGapW);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
+        k_step(0, wt, xt, 1, kGapW - 2, kGapW, STEADY ? JW_W : 0, [&](int j) { request_part(buf_w, off_gw, t + 2, w2_off, j); });
         // Own requests of W(t+1), X(t+1) have landed (W(t+2)'s may still be in
         // flight) and every LDS read issued so far -- all of tile t's -- has
         // returned; the barrier extends both to the workgroup, so tile t+1 may
@@ -247,19 +300,11 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         if (!STEADY && t + 2 < ktiles) request_unit(buf_x, base_x, off_gx, t + 2, x2_off);
-#pragma unroll
-        for (int i = 0; i < TN * TM; ++i) {
-            const int a = i / TM, b = i % TM;
-            mfma_32x32x16(acc[a][b], fa[1][a], fb[1][b]);
-            // Past the last tile these reads fetch stale LDS contents that are never used.
-            if (i < TN + TM) read_frag(wn1, xn1, 0, fa[0], fb[0], i);
-            if (STEADY && i % kGapX == kGapX - 1 && i / kGapX < JW_X) request_part(buf_x, off_gx, t + 2, x2_off, i / kGapX);
-            __builtin_amdgcn_sched_barrier(0);
-        }
+        // Past the last tile the reads of this k-step fetch stale LDS contents that are never used.
+        k_step(1, wn1, xn1, 0, 0, 2, STEADY ? JW_X : 0, [&](int j) { request_part(buf_x, off_gx, t + 2, x2_off, j); });
         s0 = s0 + 2 >= kUnits ? s0 + 2 - kUnits : s0 + 2;
     };
 
-    static_assert(TN * TM >= JW_W && TN * TM >= JW_X, "not enough MFMAs in a k-step to spread the requests");
     request_unit(buf_w, base_w, off_gw, 0, 0);
     request_unit(buf_x, base_x, off_gx, 0, kUnitBytes);
     if (ktiles > 1) {
@@ -271,7 +316,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 #pragma unroll
-    for (int i = 0; i < TN + TM; ++i) read_frag(lds, lds + kUnitBytes, 0, fa[0], fb[0], i);
+    for (int r = 0; r < NREAD; ++r) read_frag(lds, lds + kUnitBytes, 0, fa[0], fb[0], r);
 
     const int steady_end = full_tiles - 2 > 0 ? full_tiles - 2 : 0;
     int t = 0;
@@ -283,53 +328,51 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
     // The last MFMAs must have left the pipeline before acc is read by anything
     // else (18 wait states cover every case; these are 32).
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-    // Epilogue.  Lane holds, per 32x32 tile, output row m = l32 and the columns
-    // n = 8*g + 4*kg + {0,1,2,3} for g = 0..3 in acc[...][4*g + {0..3}].
+    // Epilogue.  Lane holds, per 16x16 tile, output row m = l16 and the columns
+    // n = 4 kg + {0,1,2,3} in acc[...][0..3].
     if (vec_store == 2) {
         // Through LDS, so that global stores are 16 bytes per lane and whole
         // 128-byte (or longer) row segments per instruction.  Each wavefront
-        // transposes its own (32 TM) x (32 TN) block in a private LDS region:
-        // row pitch 64 TN bytes, the 16-byte chunk index XOR-ed with a function
-        // of the row so that neither the 8-byte writes (32 rows, one column
-        // group) nor the 16-byte reads (whole rows) pile up on banks.
-        constexpr int kChunks = TN * 4;              // 16-byte chunks per row of the block
+        // transposes its own (16 TM) x (16 TN) block in a private LDS region:
+        // row pitch 32 TN bytes, the 16-byte chunk index XOR-ed with a function
+        // of the row so that neither the 8-byte writes (16 rows, four column
+        // groups) nor the 16-byte reads (whole rows) pile up on banks.
+        constexpr int kChunks = TN * 2;              // 16-byte chunks per row of the block
         constexpr bool kPow2 = (kChunks & (kChunks - 1)) == 0;
         // A power-of-two row is swizzled; any other row length is padded by one
         // chunk instead, which staggers consecutive rows over the banks.
-        constexpr int kPitch = kPow2 ? TN * 64 : TN * 64 + 16;
+        constexpr int kPitch = kPow2 ? TN * 32 : TN * 32 + 16;
         auto swz = [](int row) { return !kPow2 ? 0 : kChunks == 8 ? ((row >> 1) & 7) : (row & (kChunks - 1)); };
         __syncthreads();   // every wavefront is done with the operand stages (and every request has landed)
-        char* region = lds + wave * (TM * 32 * kPitch);
+        char* region = lds + wave * (TM * 16 * kPitch);
 #pragma unroll
         for (int a = 0; a < TN; ++a) {
+            const int64_t n = n0 + wn + a * 16 + 4 * kg;
+            float bv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (bias) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int64_t n = n0 + wn + a * 32 + 8 * g + 4 * kg;
-                float bv[4] = {0.f, 0.f, 0.f, 0.f};
-                if (bias) {
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < N) bv[e] = bf16_bits_to_f32(bias[n + e]);
+            }
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (n + e < N) bv[e] = bf16_bits_to_f32(bias[n + e]);
-                }
+            for (int b = 0; b < TM; ++b) {
+                const int row = b * 16 + l16;
+                uint16_t o[4];
 #pragma unroll
-                for (int b = 0; b < TM; ++b) {
-                    const int row = b * 32 + l32;
-                    uint16_t o[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16_bits(acc[a][b][4 * g + e] + bv[e]);
-                    uint2 pk;
-                    pk.x = static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16);
-                    pk.y = static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16);
-                    *reinterpret_cast<uint2*>(region + row * kPitch + (((a * 4 + g) ^ swz(row)) << 4) + kg * 8) = pk;
-                }
+                for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16_bits(acc[a][b][e] + bv[e]);
+                uint2 pk;
+                pk.x = static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16);
+                pk.y = static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16);
+                // columns a 16 + 4 kg .. + 3 of the block: chunk 2 a + kg / 2, half kg % 2
+                *reinterpret_cast<uint2*>(region + row * kPitch + (((a * 2 + (kg >> 1)) ^ swz(row)) << 4) + (kg & 1) * 8) = pk;
             }
         }
         // LDS operations of one wavefront complete in order, so its reads below
         // see its writes above; no other wavefront touches this region.
         asm volatile("" ::: "memory");
-        static_assert((TM * 32 * kChunks) % 64 == 0, "block does not split into whole wavefront passes");
+        static_assert((TM * 16 * kChunks) % 64 == 0, "block does not split into whole wavefront passes");
 #pragma unroll 4
-        for (int p = 0; p < TM * 32 * kChunks / 64; ++p) {
+        for (int p = 0; p < TM * 16 * kChunks / 64; ++p) {
             const int idx = p * 64 + lane;
             const int row = idx / kChunks, chunk = idx % kChunks;
             const int64_t m = m0 + wm + row;
@@ -350,40 +393,57 @@ __global__ __launch_bounds__(64 * NWM * NWN) void linear_bf16_kernel(const uint1
             }
         }
     } else {
-    #pragma unroll
+#pragma unroll
         for (int a = 0; a < TN; ++a) {
-    #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int64_t n = n0 + wn + a * 32 + 8 * g + 4 * kg;
-                float bv[4] = {0.f, 0.f, 0.f, 0.f};
-                if (bias) {
-    #pragma unroll
+            const int64_t n = n0 + wn + a * 16 + 4 * kg;
+            float bv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (bias) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < N) bv[e] = bf16_bits_to_f32(bias[n + e]);
+            }
+#pragma unroll
+            for (int b = 0; b < TM; ++b) {
+                const int64_t m = m0 + wm + b * 16 + l16;
+                if (m >= M) continue;
+                uint16_t o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16_bits(acc[a][b][e] + bv[e]);
+                uint16_t* dst = y + m * ldy + n;
+                if (vec_store && n + 3 < N) {
+                    uint2 pk;
+                    pk.x = static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16);
+                    pk.y = static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16);
+                    *reinterpret_cast<uint2*>(dst) = pk;
+                } else {
+#pragma unroll
                     for (int e = 0; e < 4; ++e)
-                        if (n + e < N) bv[e] = bf16_bits_to_f32(bias[n + e]);
-                }
-    #pragma unroll
-                for (int b = 0; b < TM; ++b) {
-                    const int64_t m = m0 + wm + b * 32 + l32;
-                    if (m >= M) continue;
-                    uint16_t o[4];
-    #pragma unroll
-                    for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16_bits(acc[a][b][4 * g + e] + bv[e]);
-                    uint16_t* dst = y + m * ldy + n;
-                    if (vec_store && n + 3 < N) {
-                        uint2 pk;
-                        pk.x = static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16);
-                        pk.y = static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16);
-                        *reinterpret_cast<uint2*>(dst) = pk;
-                    } else {
-    #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (n + e < N) dst[e] = o[e];
-                    }
+                        if (n + e < N) dst[e] = o[e];
                 }
             }
         }
     }
 }
+
+constexpr int kThreads = 512;
+
+// 256 x 256 tiles: 2 x 4 wavefronts of 128 x 64.
+__global__ __launch_bounds__(kThreads) void linear_bf16_wide(const Part part) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    gemm_tile<2, 4, 8, 4>(part, blockIdx.x, lds);
+}
+
+// 256 x 192 tiles: 4 x 2 wavefronts of 64 x 96.
+__global__ __launch_bounds__(kThreads) void linear_bf16_narrow(const Part part) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    gemm_tile<4, 2, 4, 6>(part, blockIdx.x, lds);
+}
+
+// Per-device state, set on first use by whichever thread gets there (the
+// values are the same for all of them).
+constexpr int kMaxDevices = 64;
+std::atomic<bool> lds_reserved[kMaxDevices][2];   // the dynamic LDS size of the wide / narrow kernel has been raised
+std::atomic<int> cu_count[kMaxDevices];           // 0: not asked yet
 
 }  // namespace
 }  // namespace ddl
@@ -409,40 +469,35 @@ extern "C" int ddl_linear_bf16(const void* x, const void* w, const void* bias, v
     const uint16_t* const bp = static_cast<const uint16_t*>(bias);
     uint16_t* const yp = static_cast<uint16_t*>(y);
 
-    // Columns [n_begin, n_begin + n_count) of the output with tiles of 256 x bn.
-    auto launch = [&](auto kernel, bool& attr_done, int threads, int bn, int64_t n_begin, int64_t n_count) -> int {
-        const int64_t tiles_m = (M + 255) / 256, tiles_n = (n_count + bn - 1) / bn;
-        if (tiles_m * tiles_n > 0x7FFFFFFFll || tiles_m > 0x7FFFFFll || tiles_n > 0x7FFFFFll)
-            return fail(DDL_E_UNSUPP, "linear: too many output tiles");
-        if (!attr_done) {   // the attribute sticks to the function; set it on first use
-            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-            if (e != hipSuccess) return fail(static_cast<int>(e), "linear: cannot reserve %d bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
-            attr_done = true;
-        }
-        hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(tiles_m * tiles_n)), dim3(threads), kLdsBytes,
-                           static_cast<hipStream_t>(stream), xp, wp + n_begin * ldw, bp ? bp + n_begin : nullptr, yp + n_begin, M,
-                           n_count, K, ldx, ldw, ldy, static_cast<int>(tiles_m), static_cast<int>(tiles_n), vec_store);
-        return check_launch("linear_bf16_kernel");
-    };
-    static bool wide_ready = false, narrow_ready = false;
-    auto wide = [&](int64_t n_begin, int64_t n_count) { return launch(linear_bf16_kernel<2, 4, 4, 2>, wide_ready, 512, 256, n_begin, n_count); };
-    auto narrow = [&](int64_t n_begin, int64_t n_count) { return launch(linear_bf16_kernel<4, 2, 2, 3>, narrow_ready, 512, 192, n_begin, n_count); };
-
-    // One workgroup per CU is resident, so the tiles run in rounds of one per
-    // CU and a last round that is only partly filled costs as much as a full
-    // one.  When it pays, the columns are split: whole rounds of 256-wide
-    // tiles first, the rest with 192-wide tiles, whose rounds are shorter.
-    static int cus = 0;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
+    int cus = cu_count[dev].load(std::memory_order_relaxed);
     if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1)
-            n = 256;
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
         cus = n;
+        cu_count[dev].store(n, std::memory_order_relaxed);
     }
+    auto launch = [&](int which, const Part& p) -> int {
+        const void* fn = which == 0 ? reinterpret_cast<const void*>(linear_bf16_wide) : reinterpret_cast<const void*>(linear_bf16_narrow);
+        if (!lds_reserved[dev][which].load(std::memory_order_acquire)) {   // the attribute sticks to the function on this device
+            const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+            if (e != hipSuccess) return fail(static_cast<int>(e), "linear: cannot reserve %d bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
+            lds_reserved[dev][which].store(true, std::memory_order_release);
+        }
+        const dim3 grid(static_cast<uint32_t>(static_cast<int64_t>(p.tiles_m) * p.tiles_n));
+        if (which == 0)
+            hipLaunchKernelGGL(linear_bf16_wide, grid, dim3(kThreads), kLdsBytes, static_cast<hipStream_t>(stream), p);
+        else
+            hipLaunchKernelGGL(linear_bf16_narrow, grid, dim3(kThreads), kLdsBytes, static_cast<hipStream_t>(stream), p);
+        return check_launch(which == 0 ? "linear_bf16_wide" : "linear_bf16_narrow");
+    };
+
+    // How many 256-column strips go to the wide tiles: whole rounds of them,
+    // the rest of the columns to 192-wide tiles, if that shortens the last round.
     const int64_t tiles_m = (M + 255) / 256, cols = (N + 255) / 256;
     auto rounds = [&](int64_t tiles) { return (tiles + cus - 1) / cus; };
-    const int64_t cost_wide = rounds(tiles_m * cols) * 256;
-    int64_t best_cost = cost_wide, best_split = cols;   // columns of 256 given to the wide kernel
+    int64_t best_cost = rounds(tiles_m * cols) * 256, best_split = cols;   // strips of 256 columns given to the wide tiles
     for (int64_t c = cols - 1; c >= 0 && c >= cols - 16; --c) {
         const int64_t rest = N - c * 256;
         const int64_t cost = rounds(tiles_m * c) * 256 + rounds(tiles_m * ((rest + 191) / 192)) * 192;
@@ -451,10 +506,21 @@ extern "C" int ddl_linear_bf16(const void* x, const void* w, const void* bias, v
             best_split = c;
         }
     }
-    if (best_split == cols) return wide(0, N);
-    if (best_split > 0) {
-        const int rc = wide(0, best_split * 256);
+    // Columns [n_begin, n_begin + n_count) of the output with tiles of 256 x bn.
+    auto part = [&](int bn, int64_t n_begin, int64_t n_count) {
+        Part p{};
+        p.x = xp, p.w = wp + n_begin * ldw, p.bias = bp ? bp + n_begin : nullptr, p.y = yp + n_begin;
+        p.M = M, p.N = n_count, p.K = K, p.ldx = ldx, p.ldw = ldw, p.ldy = ldy;
+        p.tiles_m = static_cast<int>(tiles_m), p.tiles_n = static_cast<int>((n_count + bn - 1) / bn), p.vec_store = vec_store;
+        return p;
+    };
+    if (tiles_m > 0x7FFFFFll || cols > 0x7FFFFFll || tiles_m * (cols + 1) > 0x7FFFFFFFll)
+        return fail(DDL_E_UNSUPP, "linear: too many output tiles");
+    const int64_t wide_cols = best_split == cols ? N : best_split * 256;
+    if (wide_cols > 0) {
+        const int rc = launch(0, part(256, 0, wide_cols));
         if (rc) return rc;
     }
-    return narrow(best_split * 256, N - best_split * 256);
+    if (wide_cols < N) return launch(1, part(192, wide_cols, N - wide_cols));
+    return 0;
 }
