@@ -39,6 +39,7 @@ class SoloTransport:
     def __init__(self, world):
         self.world = world
         self._gather_providers = {}
+        self._seeded = {}            # tag -> identity of the buffer whose peer slots a provider has filled
         self._shape_provider = None
 
     # -- configuration by tests / benchmarks --------------------------------
@@ -48,6 +49,7 @@ class SoloTransport:
         would contribute to a gather carrying ``tag`` (entry ``P.rank`` is
         replaced by the live tensor)."""
         self._gather_providers[tag] = fn
+        self._seeded.pop(tag, None)
 
     def set_peer_shape_provider(self, fn):
         """``fn(P, index, my_shape) -> shape`` of the shard held by the peer at
@@ -99,6 +101,23 @@ class SoloTransport:
                 raise TransportError(f"gather provider for {tag!r} returned {len(parts)} parts for {P.size} workers")
             parts[P.rank] = tensor
         return torch.stack(parts)
+
+    def allgather_into(self, P, buffer, tag=None):
+        """In-place all-gather: ``buffer`` is ``[P.size, ...]`` and slot
+        ``P.rank`` already holds this worker's part.  The other slots hold what
+        the caller seeded them with; a gather provider registered for ``tag``
+        fills them once per buffer (it stands for peers whose contribution does
+        not change between calls)."""
+        fn = self._gather_providers.get(tag)
+        if fn is not None and self._seeded.get(tag) != (buffer.data_ptr(), tuple(buffer.shape)):
+            parts = list(fn(P, buffer[P.rank]))
+            if len(parts) != P.size:
+                raise TransportError(f"gather provider for {tag!r} returned {len(parts)} parts for {P.size} workers")
+            for p, part in enumerate(parts):
+                if p != P.rank:
+                    buffer[p].copy_(part)
+            self._seeded[tag] = (buffer.data_ptr(), tuple(buffer.shape))
+        return buffer
 
     def broadcast(self, P_src, P_dst, tensor, tag=None):
         if P_src.active:
@@ -290,6 +309,18 @@ class LoopbackTransport:
         # Nobody may overwrite its contribution before everyone has stacked it.
         self._allgather_obj(P, None, ("tgather-done", tag))
         return out
+
+    def allgather_into(self, P, buffer, tag=None):
+        """In-place all-gather: ``buffer`` is ``[P.size, ...]`` and slot
+        ``P.rank`` already holds this worker's part; the other slots are filled
+        from the peers' buffers (copies enqueued on the shared stream)."""
+        buffers = self._allgather_obj(P, buffer, ("tgather-into", tag))
+        for p, theirs in enumerate(buffers):
+            if p != P.rank:
+                buffer[p].copy_(theirs[p])
+        # Nobody may overwrite its own slot before everyone has copied it.
+        self._allgather_obj(P, None, ("tgather-into-done", tag))
+        return buffer
 
     def broadcast(self, P_src, P_dst, tensor, tag=None):
         """Every worker of ``P_dst`` receives the tensor held by the worker of

@@ -33,41 +33,52 @@ STATS_TAG = "layernorm_stats"
 BWD_SUMS_TAG = "layernorm_backward_sums"
 
 
+def _shard_forward(input, weight, bias, P_reduce, part_cols, eps, part_cols_arr, stats_buffers, keep):
+    """Forward of one shard: ``(y, x2d, mean, rstd, gamma)``; mean and rstd are
+    None unless ``keep``.  ``stats_buffers``: the layer's cache of gathered
+    statistics buffers ``[P, rows, 2]`` by row count (the stats kernel writes
+    this worker's slot in place, the transport fills the others)."""
+    x = input.detach()
+    cols = int(part_cols[P_reduce.rank if P_reduce.active else 0])
+    x2d = x.reshape(-1, cols)
+    if x2d.shape[1] > 1 and x2d.stride(1) != 1:
+        x2d = x2d.contiguous()
+    gamma = None if weight is None else weight.detach().reshape(-1)
+    beta = None if bias is None else bias.detach().reshape(-1)
+    nparts = len(part_cols)
+    if nparts > 1:
+        rows = x2d.shape[0]
+        gathered = stats_buffers.get(rows)
+        if gathered is None or gathered.device != x2d.device:
+            gathered = stats_buffers[rows] = torch.zeros((nparts, rows, 2), dtype=torch.float32, device=x2d.device)
+        hip_ops.ln_partial_stats(x2d, out=gathered[P_reduce.rank])
+        P_reduce._world.transport.allgather_into(P_reduce, gathered, tag=STATS_TAG)
+        res = hip_ops.ln_normalize_affine(x2d, gathered, part_cols, gamma, beta, eps, want_stats=keep,
+                                          part_cols_arr=part_cols_arr)
+    else:
+        res = hip_ops.layer_norm(x2d, gamma, beta, eps, want_stats=keep)
+    if not keep:
+        return res.view(input.shape), x2d, None, None, gamma
+    y, mean, rstd = res
+    return y.view(input.shape), x2d, mean, rstd, gamma
+
+
 class _LayerNormShard(torch.autograd.Function):
     """Local shard of a layer norm whose statistics span ``P_reduce``, and its
     adjoint: the gradient autograd derives from the reference's forward
     (nn/layernorm.py:230-247, 295-309), whose all-reduces are self-adjoint."""
 
     @staticmethod
-    def forward(ctx, input, weight, bias, P_reduce, part_cols, eps, part_cols_arr=None, grad_mode=True):
-        x = input.detach()
-        cols = int(part_cols[P_reduce.rank if P_reduce.active else 0])
-        x2d = x.reshape(-1, cols)
-        if x2d.shape[1] > 1 and x2d.stride(1) != 1:
-            x2d = x2d.contiguous()
-        gamma = None if weight is None else weight.detach().reshape(-1)
-        beta = None if bias is None else bias.detach().reshape(-1)
-        # mean and rstd are only kept when a gradient can be asked for (``grad_mode``: whether autograd was
-        # recording when the layer was called; inside ``forward`` it never is)
-        keep = grad_mode and any(ctx.needs_input_grad[:3])
-        if len(part_cols) > 1:
-            stats = hip_ops.ln_partial_stats(x2d)
-            gathered = P_reduce._world.transport.allgather(P_reduce, stats, tag=STATS_TAG)
-            gathered = gathered.contiguous()
-            res = hip_ops.ln_normalize_affine(x2d, gathered, part_cols, gamma, beta, eps, want_stats=keep,
-                                              part_cols_arr=part_cols_arr)
-        else:
-            res = hip_ops.layer_norm(x2d, gamma, beta, eps, want_stats=keep)
-        if not keep:
-            return res.view(input.shape)
-        y, mean, rstd = res
-        if x2d.dtype != torch.float32:
-            raise NotImplementedError(f"DistributedLayerNorm backward kernels are fp32 only, got {x2d.dtype}; "
+    def forward(ctx, input, weight, bias, P_reduce, part_cols, eps, part_cols_arr=None, stats_buffers=None):
+        if input.dtype != torch.float32:
+            raise NotImplementedError(f"DistributedLayerNorm backward kernels are fp32 only, got {input.dtype}; "
                                       "run the forward under torch.no_grad() or in float32")
+        y, x2d, mean, rstd, gamma = _shard_forward(input, weight, bias, P_reduce, part_cols, eps, part_cols_arr,
+                                                   {} if stats_buffers is None else stats_buffers, True)
         ctx.save_for_backward(x2d, mean, rstd, gamma)
-        ctx.P_reduce, ctx.nparts, ctx.cols = P_reduce, len(part_cols), cols
+        ctx.P_reduce, ctx.nparts, ctx.cols = P_reduce, len(part_cols), x2d.shape[1]
         ctx.param_shapes = (None if weight is None else weight.shape, None if bias is None else bias.shape)
-        return y.view(input.shape)
+        return y
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -154,6 +165,8 @@ class DistributedLayerNorm(Module):
         local_norm_shape = compute_subshape(reduce_shape, P_x.index[self.dim_reduce_slice], self.normalized_shape)
         self._part_cols_arr = _lib.i64_array(self.part_cols)     # what the normalize kernel's entry point takes
         self._checked_shape = None                               # last input shape found consistent with part_cols
+        self._stats_buffers = {}                                 # rows -> gathered statistics buffer [P, rows, 2]
+        self._call_plan = None                                   # what _forward_contiguous worked out for the last shape
 
         if self.elementwise_affine:
             # Parameters live on the workers with index 0 in every dimension that
@@ -200,6 +213,52 @@ class DistributedLayerNorm(Module):
         self.weight_buffer = self.broadcast(self.weight)
         self.bias_buffer = self.broadcast(self.bias)
 
+    def _forward_contiguous(self, input, weight, bias):
+        """The forward of ``_shard_forward`` for a contiguous input when no
+        gradient is recorded: everything that only depends on the input's
+        shape (row and column counts, the gathered-statistics buffer and the
+        address of this worker's slot in it) is worked out once per shape, and a
+        call is the two entry points with the transport's gather between."""
+        plan = self._call_plan
+        if plan is None or plan[0] != input.shape or plan[1] != input.dtype or plan[2] != input.device:
+            P_reduce = self.allreduce.P_allreduce
+            nparts = len(self.part_cols)
+            cols = int(self.part_cols[P_reduce.rank if (nparts > 1 and P_reduce.active) else 0])
+            rows = input.numel() // cols
+            gathered = own = None
+            if nparts > 1:
+                gathered = self._stats_buffers.get(rows)
+                if gathered is None or gathered.device != input.device:
+                    gathered = self._stats_buffers[rows] = torch.zeros((nparts, rows, 2), dtype=torch.float32,
+                                                                       device=input.device)
+                own = gathered.data_ptr() + P_reduce.rank * rows * 8
+            plan = self._call_plan = (input.shape, input.dtype, input.device, rows, cols, hip_ops._LN_DTYPES[input.dtype],
+                                      nparts, gathered, own, P_reduce, _lib.load())
+        _, _, _, rows, cols, dt, nparts, gathered, own, P_reduce, lib = plan
+        if weight is not None and (weight.numel() != cols or bias.numel() != cols):
+            raise ValueError(f"DistributedLayerNorm parameters hold {weight.numel()} / {bias.numel()} elements, "
+                             f"the local rows hold {cols}")
+        y = torch.empty_like(input)
+        stream = hip_ops._stream()
+        gamma = None if weight is None else weight.data_ptr()
+        beta = None if bias is None else bias.data_ptr()
+        if nparts > 1:
+            rc = lib.ddl_ln_partial_stats(input.data_ptr(), dt, rows, cols, cols, own, stream)
+            if rc:
+                _lib.check(rc, "ddl_ln_partial_stats")
+            P_reduce._world.transport.allgather_into(P_reduce, gathered, tag=STATS_TAG)
+            rc = lib.ddl_ln_normalize_affine(input.data_ptr(), dt, rows, cols, cols, gathered.data_ptr(), nparts,
+                                             self._part_cols_arr, gamma, beta, self.eps, y.data_ptr(), cols, None, None,
+                                             stream)
+            if rc:
+                _lib.check(rc, "ddl_ln_normalize_affine")
+        else:
+            rc = lib.ddl_layer_norm(input.data_ptr(), dt, rows, cols, cols, gamma, beta, self.eps, y.data_ptr(), cols,
+                                    None, None, stream)
+            if rc:
+                _lib.check(rc, "ddl_layer_norm")
+        return y
+
     def forward(self, input):
         if not self.P_x.active:
             return input
@@ -224,5 +283,12 @@ class DistributedLayerNorm(Module):
                 raise ValueError(f"input shard has {local_cols} normalised elements, the partition of "
                                  f"normalized_shape={self.normalized_shape} gives this worker {self.part_cols[mine]}")
             self._checked_shape = input.shape
+        wants_grad = torch.is_grad_enabled() and (input.requires_grad or (weight is not None and weight.requires_grad) or
+                                                  (bias is not None and bias.requires_grad))
+        if not wants_grad:      # nothing to record: skip the autograd machinery and the statistics kept for backward
+            if input.is_cuda and input.is_contiguous() and (weight is None or (weight.is_contiguous() and bias.is_contiguous())):
+                return self._forward_contiguous(input, weight, bias)
+            return _shard_forward(input, weight, bias, self.allreduce.P_allreduce, self.part_cols, self.eps,
+                                  self._part_cols_arr, self._stats_buffers, False)[0]
         return _LayerNormShard.apply(input, weight, bias, self.allreduce.P_allreduce, self.part_cols, self.eps,
-                                     self._part_cols_arr, torch.is_grad_enabled())
+                                     self._part_cols_arr, self._stats_buffers)

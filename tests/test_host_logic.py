@@ -207,6 +207,43 @@ def test_loopback_transport_moves_data_between_rank_threads():
         assert summed == 6 and root == "hello"
 
 
+def test_allgather_into_fills_the_other_slots_in_place():
+    """In-place all-gather: every worker writes its own slot, the transport fills
+    the rest (loopback), or leaves seeded slots alone and consults a provider
+    once per buffer (solo)."""
+    world = SimWorld(3, device=torch.device("cpu"))
+
+    def body(P):
+        results = []
+        buf = torch.full((3, 2), -1.0)
+        for step in range(2):                       # the same buffer on consecutive calls
+            buf[P.rank] = torch.tensor([10.0 * step + P.rank, 0.5])
+            world.transport.allgather_into(P, buf, tag="s")
+            results.append(buf.clone())
+        return results
+
+    for rank, results in enumerate(world.run(body)):
+        for step, got in enumerate(results):
+            assert got[:, 0].tolist() == [10.0 * step, 10.0 * step + 1, 10.0 * step + 2] and got[:, 1].tolist() == [0.5] * 3
+
+    solo = SimWorld(3, device=torch.device("cpu"))
+    P = solo.partition(1)
+    buf = torch.zeros(3, 2)
+    buf[0], buf[2] = torch.tensor([7.0, 7.0]), torch.tensor([9.0, 9.0])      # seeded by the caller
+    buf[1] = 1.0
+    assert solo.transport.allgather_into(P, buf, tag="s") is buf and buf.tolist() == [[7, 7], [1, 1], [9, 9]]
+    calls = []
+
+    def provider(P_, mine):
+        calls.append(1)
+        return [torch.full((2,), 3.0), None, torch.full((2,), 4.0)]
+    solo.transport.set_gather_provider("s", provider)
+    solo.transport.allgather_into(P, buf, tag="s")
+    buf[1] = 2.0
+    solo.transport.allgather_into(P, buf, tag="s")
+    assert buf.tolist() == [[3, 3], [2, 2], [4, 4]] and len(calls) == 1
+
+
 def test_loopback_transport_propagates_failures():
     world = SimWorld(2, device=torch.device("cpu"))
 
