@@ -90,6 +90,11 @@ SIGNATURES = {
                                        c_int, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "ddl_embedding_backward_static": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64,
                                               c_int64, c_int, c_void_p, c_int64, c_void_p]),
+    "ddl_linear": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int64,
+                           c_int64, c_void_p]),
+    "ddl_gemm_f32": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int64,
+                             c_int64, c_int64, c_void_p]),
+    "ddl_colsum": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_void_p]),
     "ddl_linear_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                 c_int64, c_void_p]),
     "ddl_transpose_2d": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),

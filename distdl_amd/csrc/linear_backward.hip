@@ -12,6 +12,8 @@
 // db is a column sum with fp32 accumulation.
 #include "ddl_common.h"
 
+#include <hip/hip_fp16.h>
+
 namespace ddl {
 namespace {
 
@@ -86,11 +88,57 @@ __device__ inline uint16_t f32_to_bf16(float f) {
     return static_cast<uint16_t>(u >> 16);
 }
 
+// Element types of the column sum: 0 = bf16, 1 = fp16, 2 = fp32.
+template <int DT>
+struct Elem;
+template <>
+struct Elem<0> {
+    typedef uint16_t type;
+    static __device__ float load(const uint16_t* p) { return bf16_to_f32(*p); }
+    static __device__ void store(uint16_t* p, float f) { *p = f32_to_bf16(f); }
+    static __device__ void load8(const uint16_t* p, float (&v)[8]) {
+        const uint4 q = *reinterpret_cast<const uint4*>(p);
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            v[2 * e] = __uint_as_float(w[e] << 16);
+            v[2 * e + 1] = __uint_as_float(w[e] & 0xFFFF0000u);
+        }
+    }
+};
+template <>
+struct Elem<1> {
+    typedef __half type;
+    static __device__ float load(const __half* p) { return __half2float(*p); }
+    static __device__ void store(__half* p, float f) { *p = __float2half_rn(f); }
+    static __device__ void load8(const __half* p, float (&v)[8]) {
+        const uint4 q = *reinterpret_cast<const uint4*>(p);
+        const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float2 f = __half22float2(*reinterpret_cast<const __half2*>(&w[e]));
+            v[2 * e] = f.x;
+            v[2 * e + 1] = f.y;
+        }
+    }
+};
+template <>
+struct Elem<2> {
+    typedef float type;
+    static __device__ float load(const float* p) { return *p; }
+    static __device__ void store(float* p, float f) { *p = f; }
+    static __device__ void load8(const float* p, float (&v)[8]) {
+        const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+        v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+    }
+};
+
 // Stage 1 of the column sum: workgroup (strip, split) adds rows
 // [split * rows_per_split, ...) of a 64-column strip in fp32 and writes 64
 // partial sums to partial[split, col].  8 lanes cover the 64 columns of a row,
 // 32 rows are in flight per pass; LDS folds the 32 row groups.
-__global__ __launch_bounds__(kBlock) void colsum_partial_kernel(const uint16_t* __restrict__ a, int64_t rows, int64_t cols,
+template <int DT>
+__global__ __launch_bounds__(kBlock) void colsum_partial_kernel(const typename Elem<DT>::type* __restrict__ a, int64_t rows, int64_t cols,
                                                                 int64_t ld, int64_t rows_per_split, float* __restrict__ partial,
                                                                 int strips, int vec_ok) {
     __shared__ float fold[32][kTile + 1];
@@ -103,20 +151,17 @@ __global__ __launch_bounds__(kBlock) void colsum_partial_kernel(const uint16_t* 
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if (vec_ok && gc + 8 <= cols) {
         for (int64_t r = r_begin + g; r < r_end; r += 32) {
-            const uint4 q = *reinterpret_cast<const uint4*>(a + r * ld + gc);
-            const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+            float v[8];
+            Elem<DT>::load8(a + r * ld + gc, v);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                acc[2 * e] += __uint_as_float(w[e] << 16);
-                acc[2 * e + 1] += __uint_as_float(w[e] & 0xFFFF0000u);
-            }
+            for (int e = 0; e < 8; ++e) acc[e] += v[e];
         }
     } else {
         for (int64_t r = r_begin + g; r < r_end; r += 32) {
-            const uint16_t* s = a + r * ld + gc;
+            const typename Elem<DT>::type* s = a + r * ld + gc;
 #pragma unroll
             for (int e = 0; e < 8; ++e)
-                if (gc + e < cols) acc[e] += bf16_to_f32(s[e]);
+                if (gc + e < cols) acc[e] += Elem<DT>::load(s + e);
         }
     }
 #pragma unroll
@@ -131,11 +176,12 @@ __global__ __launch_bounds__(kBlock) void colsum_partial_kernel(const uint16_t* 
     }
 }
 
-// Stage 2: out[col] = bf16(sum over splits of partial[split, col]).  A workgroup
+// Stage 2: out[col] = sum over splits of partial[split, col], rounded to the element type.  A workgroup
 // per 64-column strip; lane group t / 64 adds every fourth split (eight
 // independent loads in flight), LDS folds the four groups.
+template <int DT>
 __global__ __launch_bounds__(kBlock) void colsum_final_kernel(const float* __restrict__ partial, int64_t cols, int splits,
-                                                              uint16_t* __restrict__ out) {
+                                                              typename Elem<DT>::type* __restrict__ out) {
     constexpr int kGroups = kBlock / kTile;
     __shared__ float fold[kGroups][kTile];
     const int g = threadIdx.x / kTile, t = threadIdx.x % kTile;
@@ -158,7 +204,7 @@ __global__ __launch_bounds__(kBlock) void colsum_final_kernel(const float* __res
         float r = 0.f;
 #pragma unroll
         for (int k = 0; k < kGroups; ++k) r += fold[k][t];
-        out[col] = f32_to_bf16(r);
+        Elem<DT>::store(out + col, r);
     }
 }
 
@@ -184,13 +230,35 @@ extern "C" int ddl_transpose_2d(const void* src, void* dst, int64_t rows, int64_
     return check_launch("transpose16_kernel");
 }
 
-extern "C" int ddl_colsum_bf16(const void* a, int64_t rows, int64_t cols, int64_t ld, void* out, float* workspace,
-                               int64_t workspace_elems, void* stream) {
+namespace ddl {
+namespace {
+
+template <int DT>
+int run_colsum(const void* a, int64_t rows, int64_t cols, int64_t ld, void* out, float* workspace, int64_t splits,
+               int64_t rows_per_split, int64_t strips, hipStream_t s) {
+    typedef typename Elem<DT>::type T;
+    const int vec_ok = (aligned_to(a, 8 * sizeof(T)) && (ld * sizeof(T)) % 16 == 0) ? 1 : 0;
+    hipLaunchKernelGGL((colsum_partial_kernel<DT>), dim3(static_cast<uint32_t>(strips * splits)), dim3(kBlock), 0, s,
+                       static_cast<const T*>(a), rows, cols, ld, rows_per_split, workspace, static_cast<int>(strips), vec_ok);
+    const int rc = check_launch("colsum_partial_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL((colsum_final_kernel<DT>), dim3(static_cast<uint32_t>(strips)), dim3(kBlock), 0, s, workspace, cols,
+                       static_cast<int>(splits), static_cast<T*>(out));
+    return check_launch("colsum_final_kernel");
+}
+
+}  // namespace
+}  // namespace ddl
+
+extern "C" int ddl_colsum(const void* a, int dtype, int64_t rows, int64_t cols, int64_t ld, void* out, float* workspace,
+                          int64_t workspace_elems, void* stream) {
     using namespace ddl;
+    if (dtype != DDL_DT_BF16 && dtype != DDL_DT_F16 && dtype != DDL_DT_F32) return fail(DDL_E_UNSUPP, "colsum: dtype %d (bf16, f16 and f32 only)", dtype);
     if (rows < 0 || cols < 0 || ld < cols) return fail(DDL_E_ARG, "colsum: rows=%lld cols=%lld ld=%lld", (long long)rows, (long long)cols, (long long)ld);
     if (cols == 0) return 0;
     if (!out || !workspace || (rows > 0 && !a)) return fail(DDL_E_ARG, "colsum: null pointer");
-    if (!aligned_to(a, 2) || !aligned_to(out, 2) || !aligned_to(workspace, 4)) return fail(DDL_E_ALIGN, "colsum: pointer misaligned");
+    const int es = dtype == DDL_DT_F32 ? 4 : 2;
+    if (!aligned_to(a, es) || !aligned_to(out, es) || !aligned_to(workspace, 4)) return fail(DDL_E_ALIGN, "colsum: pointer misaligned");
     // as many row splits as the workspace holds, up to 64 and to 128 rows per split
     int64_t splits = workspace_elems / cols;
     if (splits < 1) return fail(DDL_E_ARG, "colsum: workspace of %lld floats is smaller than one row of %lld", (long long)workspace_elems, (long long)cols);
@@ -201,12 +269,12 @@ extern "C" int ddl_colsum_bf16(const void* a, int64_t rows, int64_t cols, int64_
     const int64_t strips = (cols + kTile - 1) / kTile;
     if (strips * splits > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "colsum: too many workgroups");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(colsum_partial_kernel, dim3(static_cast<uint32_t>(strips * splits)), dim3(kBlock), 0, s,
-                       static_cast<const uint16_t*>(a), rows, cols, ld, rows_per_split, workspace, static_cast<int>(strips),
-                       (aligned_to(a, 16) && ld % 8 == 0) ? 1 : 0);
-    int rc = check_launch("colsum_partial_kernel");
-    if (rc) return rc;
-    hipLaunchKernelGGL(colsum_final_kernel, dim3(static_cast<uint32_t>(strips)), dim3(kBlock), 0, s,
-                       workspace, cols, static_cast<int>(splits), static_cast<uint16_t*>(out));
-    return check_launch("colsum_final_kernel");
+    if (dtype == DDL_DT_BF16) return run_colsum<0>(a, rows, cols, ld, out, workspace, splits, rows_per_split, strips, s);
+    if (dtype == DDL_DT_F16) return run_colsum<1>(a, rows, cols, ld, out, workspace, splits, rows_per_split, strips, s);
+    return run_colsum<2>(a, rows, cols, ld, out, workspace, splits, rows_per_split, strips, s);
+}
+
+extern "C" int ddl_colsum_bf16(const void* a, int64_t rows, int64_t cols, int64_t ld, void* out, float* workspace,
+                               int64_t workspace_elems, void* stream) {
+    return ddl_colsum(a, DDL_DT_BF16, rows, cols, ld, out, workspace, workspace_elems, stream);
 }

@@ -1,6 +1,7 @@
-// DistributedLinear shard GEMM: y[M,N] = x[M,K] . w[N,K]^T + bias[N], bf16
-// operands, fp32 accumulation on the matrix cores, bf16 result (reference:
-// nn/linear.py:103, nn/linear_ag.py:486 -- torch.nn.functional.linear).
+// DistributedLinear shard GEMM: y[M,N] = x[M,K] . w[N,K]^T + bias[N], bf16 (or
+// fp16) operands, fp32 accumulation on the matrix cores, result in the operands'
+// type (reference: nn/linear.py:103, nn/linear_ag.py:486 --
+// torch.nn.functional.linear).
 //
 // Both operands are K-contiguous, so a 16-byte load anywhere gives eight
 // consecutive k of one row: exactly one lane's share of an MFMA operand.  The
@@ -52,6 +53,7 @@
 //              that the 32 workgroups resident on one XCD cover a compact patch
 //              of the tile grid and share their operand panels in that XCD's L2
 #include "ddl_common.h"
+#include <hip/hip_fp16.h>
 #include <atomic>
 #include <type_traits>
 
@@ -93,8 +95,33 @@ __device__ inline void dma16(__amdgpu_buffer_rsrc_t buffer, int voffset, int sof
 // operands (it waits for the LDS reads that produce a and b); what it does not
 // do for assembly is pad the distance between an MFMA and a later non-MFMA
 // read of acc -- the kernel does that once, in front of the epilogue.
+template <bool F16>
 __device__ inline void mfma_16x16x32(floatx4& acc, const bf16x8& a, const bf16x8& b) {
-    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+    if (F16)   // the same eight 16-bit elements per lane, read as fp16
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+    else
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+
+// 16-bit element <-> fp32, round to nearest even on the way back.
+template <bool F16>
+__device__ inline float elem_to_f32(uint16_t b) {
+    if (F16) {
+        __half h;
+        __builtin_memcpy(&h, &b, 2);
+        return __half2float(h);
+    }
+    return bf16_bits_to_f32(b);
+}
+template <bool F16>
+__device__ inline uint16_t f32_to_elem(float f) {
+    if (F16) {
+        const __half h = __float2half_rn(f);
+        uint16_t b;
+        __builtin_memcpy(&b, &h, 2);
+        return b;
+    }
+    return f32_to_bf16_bits(f);
 }
 
 // s_waitcnt immediate (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4,
@@ -115,7 +142,7 @@ struct Part {
     int tiles_m, tiles_n, vec_store;
 };
 
-template <int NWM, int NWN, int TM, int TN>
+template <bool F16, int NWM, int NWN, int TM, int TN>
 __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* lds) {
     static_assert(NWM * NWN == 8, "eight wavefronts per workgroup");
     const uint16_t* __restrict__ x = part.x;
@@ -271,7 +298,7 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
         for (int q = 0; q < NMFMA; ++q) {
             const int o = q / NI, i = q % NI;
             const int a = kOuterX ? i : o, b = kOuterX ? o : i;
-            mfma_16x16x32(acc[a][b], fa[cur][a], fb[cur][b]);
+            mfma_16x16x32<F16>(acc[a][b], fa[cur][a], fb[cur][b]);
             if ((q & 1) && (q >> 1) < NREAD) read_frag(wt, xt, ks_next, fa[cur ^ 1], fb[cur ^ 1], q >> 1);
             if (q >= first && (q - first) % gap == 0 && (q - first) / gap < nreq) request((q - first) / gap);
             __builtin_amdgcn_sched_barrier(0);
@@ -352,14 +379,14 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
             if (bias) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    if (n + e < N) bv[e] = bf16_bits_to_f32(bias[n + e]);
+                    if (n + e < N) bv[e] = elem_to_f32<F16>(bias[n + e]);
             }
 #pragma unroll
             for (int b = 0; b < TM; ++b) {
                 const int row = b * 16 + l16;
                 uint16_t o[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16_bits(acc[a][b][e] + bv[e]);
+                for (int e = 0; e < 4; ++e) o[e] = f32_to_elem<F16>(acc[a][b][e] + bv[e]);
                 uint2 pk;
                 pk.x = static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16);
                 pk.y = static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16);
@@ -400,7 +427,7 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
             if (bias) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    if (n + e < N) bv[e] = bf16_bits_to_f32(bias[n + e]);
+                    if (n + e < N) bv[e] = elem_to_f32<F16>(bias[n + e]);
             }
 #pragma unroll
             for (int b = 0; b < TM; ++b) {
@@ -408,7 +435,7 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
                 if (m >= M) continue;
                 uint16_t o[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16_bits(acc[a][b][e] + bv[e]);
+                for (int e = 0; e < 4; ++e) o[e] = f32_to_elem<F16>(acc[a][b][e] + bv[e]);
                 uint16_t* dst = y + m * ldy + n;
                 if (vec_store && n + 3 < N) {
                     uint2 pk;
@@ -428,29 +455,48 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
 constexpr int kThreads = 512;
 
 // 256 x 256 tiles: 2 x 4 wavefronts of 128 x 64.
-__global__ __launch_bounds__(kThreads) void linear_bf16_wide(const Part part) {
+template <bool F16>
+__global__ __launch_bounds__(kThreads) void linear16_wide(const Part part) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
-    gemm_tile<2, 4, 8, 4>(part, blockIdx.x, lds);
+    gemm_tile<F16, 2, 4, 8, 4>(part, blockIdx.x, lds);
 }
 
 // 256 x 192 tiles: 4 x 2 wavefronts of 64 x 96.
-__global__ __launch_bounds__(kThreads) void linear_bf16_narrow(const Part part) {
+template <bool F16>
+__global__ __launch_bounds__(kThreads) void linear16_narrow(const Part part) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
-    gemm_tile<4, 2, 4, 6>(part, blockIdx.x, lds);
+    gemm_tile<F16, 4, 2, 4, 6>(part, blockIdx.x, lds);
 }
 
 // Per-device state, set on first use by whichever thread gets there (the
 // values are the same for all of them).
 constexpr int kMaxDevices = 64;
-std::atomic<bool> lds_reserved[kMaxDevices][2];   // the dynamic LDS size of the wide / narrow kernel has been raised
+std::atomic<bool> lds_reserved[kMaxDevices][4];   // the dynamic LDS size of kernel (fp16 ? 2 : 0) + (narrow ? 1 : 0) has been raised
 std::atomic<int> cu_count[kMaxDevices];           // 0: not asked yet
 
 }  // namespace
 }  // namespace ddl
 
+extern "C" int ddl_gemm_f32(const float* a, int64_t a_row_stride, int64_t a_k_stride, const float* b, int64_t b_row_stride,
+                            int64_t b_k_stride, const float* bias, float* y, int64_t ldy, int64_t M, int64_t N, int64_t K,
+                            void* stream);
+
 extern "C" int ddl_linear_bf16(const void* x, const void* w, const void* bias, void* y, int64_t M, int64_t N, int64_t K,
                                int64_t ldx, int64_t ldw, int64_t ldy, void* stream) {
+    return ddl_linear(x, w, bias, y, DDL_DT_BF16, M, N, K, ldx, ldw, ldy, stream);
+}
+
+extern "C" int ddl_linear(const void* x, const void* w, const void* bias, void* y, int dtype, int64_t M, int64_t N, int64_t K,
+                          int64_t ldx, int64_t ldw, int64_t ldy, void* stream) {
     using namespace ddl;
+    if (dtype != DDL_DT_BF16 && dtype != DDL_DT_F16 && dtype != DDL_DT_F32)
+        return fail(DDL_E_UNSUPP, "linear: dtype %d (bf16, f16 and f32 only)", dtype);
+    if (dtype == DDL_DT_F32) {
+        if (ldx < K || ldw < K) return fail(DDL_E_ARG, "linear: ldx=%lld ldw=%lld below K=%lld", (long long)ldx, (long long)ldw, (long long)K);
+        return ddl_gemm_f32(static_cast<const float*>(x), ldx, 1, static_cast<const float*>(w), ldw, 1, static_cast<const float*>(bias),
+                            static_cast<float*>(y), ldy, M, N, K, stream);
+    }
+    const bool f16 = dtype == DDL_DT_F16;
     if (M < 0 || N < 0 || K < 0 || ldx < K || ldw < K || ldy < N)
         return fail(DDL_E_ARG, "linear: M=%lld N=%lld K=%lld ldx=%lld ldw=%lld ldy=%lld", (long long)M, (long long)N,
                     (long long)K, (long long)ldx, (long long)ldw, (long long)ldy);
@@ -479,18 +525,17 @@ extern "C" int ddl_linear_bf16(const void* x, const void* w, const void* bias, v
         cu_count[dev].store(n, std::memory_order_relaxed);
     }
     auto launch = [&](int which, const Part& p) -> int {
-        const void* fn = which == 0 ? reinterpret_cast<const void*>(linear_bf16_wide) : reinterpret_cast<const void*>(linear_bf16_narrow);
-        if (!lds_reserved[dev][which].load(std::memory_order_acquire)) {   // the attribute sticks to the function on this device
-            const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+        typedef void (*Kernel)(const Part);
+        const Kernel kernels[4] = {linear16_wide<false>, linear16_narrow<false>, linear16_wide<true>, linear16_narrow<true>};
+        const int k = (f16 ? 2 : 0) + which;
+        if (!lds_reserved[dev][k].load(std::memory_order_acquire)) {   // the attribute sticks to the function on this device
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernels[k]), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
             if (e != hipSuccess) return fail(static_cast<int>(e), "linear: cannot reserve %d bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
-            lds_reserved[dev][which].store(true, std::memory_order_release);
+            lds_reserved[dev][k].store(true, std::memory_order_release);
         }
         const dim3 grid(static_cast<uint32_t>(static_cast<int64_t>(p.tiles_m) * p.tiles_n));
-        if (which == 0)
-            hipLaunchKernelGGL(linear_bf16_wide, grid, dim3(kThreads), kLdsBytes, static_cast<hipStream_t>(stream), p);
-        else
-            hipLaunchKernelGGL(linear_bf16_narrow, grid, dim3(kThreads), kLdsBytes, static_cast<hipStream_t>(stream), p);
-        return check_launch(which == 0 ? "linear_bf16_wide" : "linear_bf16_narrow");
+        hipLaunchKernelGGL(kernels[k], grid, dim3(kThreads), kLdsBytes, static_cast<hipStream_t>(stream), p);
+        return check_launch(which == 0 ? "linear16_wide" : "linear16_narrow");
     };
 
     // How many 256-column strips go to the wide tiles: whole rounds of them,

@@ -457,13 +457,35 @@ def embedding_backward(grad_output, ids, lo, hi, padding_idx=None, scale_grad_by
     return dw
 
 
-def linear_bf16(x, weight, bias=None, out=None):
-    """y = x @ weight.T + bias; bf16 operands, fp32 accumulation, bf16 result."""
+_LINEAR_DTYPES = {
+    torch.bfloat16: _lib.DDL_DT_BF16,
+    torch.float16: _lib.DDL_DT_F16,
+    torch.float32: _lib.DDL_DT_F32,
+}
+
+
+def _padded_k(t, k8):
+    """``t[rows, k]`` copied into a fresh ``[rows, k8]`` tensor whose extra columns are zero."""
+    rows, k = t.shape
+    out = torch.zeros((rows, k8), dtype=t.dtype, device=t.device)
+    if rows > 0 and k > 0:
+        full = [slice(0, rows), slice(0, k)]
+        copy_box(t, full, out, full)
+    return out
+
+
+def linear(x, weight, bias=None, out=None):
+    """y = x @ weight.T + bias with fp32 accumulation; operands and result
+    bfloat16, float16 or float32 (all the same).  The 16-bit kernel wants the
+    reduction length and the row pitches to be multiples of 8 and 16-byte
+    aligned operands; operands that are not are copied into zero-padded
+    temporaries first (zeros add nothing to the sums)."""
     _require_gpu(x, weight, bias)
-    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or (bias is not None and bias.dtype != torch.bfloat16):
-        raise ValueError("linear_bf16: operands must be bfloat16")
+    dt = _LINEAR_DTYPES.get(x.dtype)
+    if dt is None or weight.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
+        raise ValueError("linear: operands must all be bfloat16, all float16 or all float32")
     if weight.dim() != 2 or x.shape[-1] != weight.shape[1]:
-        raise ValueError(f"linear_bf16: x[..., {x.shape[-1]}] does not match weight {tuple(weight.shape)}")
+        raise ValueError(f"linear: x[..., {x.shape[-1]}] does not match weight {tuple(weight.shape)}")
     n, k = weight.shape
     x2 = x.reshape(-1, k)
     if x2.stride(1) != 1 and k > 1:
@@ -471,16 +493,35 @@ def linear_bf16(x, weight, bias=None, out=None):
     if weight.stride(1) != 1 and k > 1:
         weight = weight.contiguous()
     if bias is not None and (bias.numel() != n or not bias.is_contiguous()):
-        raise ValueError("linear_bf16: bias must be contiguous with out_features elements")
+        raise ValueError("linear: bias must be contiguous with out_features elements")
     m = x2.shape[0]
     if out is None:
-        out = torch.empty(tuple(x.shape[:-1]) + (n,), dtype=torch.bfloat16, device=x.device)
-    elif not out.is_contiguous() or out.numel() != m * n or out.dtype != torch.bfloat16:
-        raise ValueError("linear_bf16: bad output tensor")
-    rc = _lib.load().ddl_linear_bf16(x2.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(), m, n, k,
-                                     x2.stride(0) if m > 1 else k, weight.stride(0) if n > 1 else k, n, _stream())
-    _lib.check(rc, "ddl_linear_bf16")
+        out = torch.empty(tuple(x.shape[:-1]) + (n,), dtype=x.dtype, device=x.device)
+    elif not out.is_contiguous() or out.numel() != m * n or out.dtype != x.dtype:
+        raise ValueError("linear: bad output tensor")
+    if k == 0:
+        # an empty sum: the bias alone (the kernels refuse K = 0)
+        out.zero_()
+        if bias is not None and m > 0:
+            copy_box(bias.reshape(1, n).expand(m, n), [slice(0, m), slice(0, n)], out.view(m, n), [slice(0, m), slice(0, n)])
+        return out
+    if dt != _lib.DDL_DT_F32:
+        def fits(t, rows):
+            return k % 8 == 0 and t.data_ptr() % 16 == 0 and (rows <= 1 or t.stride(0) % 8 == 0)
+        if not (fits(x2, m) and fits(weight, n)):
+            k8 = _round_up(k, 8)
+            x2, weight, k = _padded_k(x2, k8), _padded_k(weight, k8), k8
+    rc = _lib.load().ddl_linear(x2.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(), dt, m, n, k,
+                                x2.stride(0) if m > 1 else k, weight.stride(0) if n > 1 else k, n, _stream())
+    _lib.check(rc, "ddl_linear")
     return out
+
+
+def linear_bf16(x, weight, bias=None, out=None):
+    """:func:`linear` restricted to bfloat16 operands."""
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or (bias is not None and bias.dtype != torch.bfloat16):
+        raise ValueError("linear_bf16: operands must be bfloat16")
+    return linear(x, weight, bias, out)
 
 
 def _round_up(n, m):
@@ -506,29 +547,42 @@ def transpose_2d(src, ld_dst=None):
     return dst
 
 
-def colsum_bf16(a):
-    """Column sums of a 2-D bf16 tensor, fp32 accumulation, bf16 result."""
+def colsum(a):
+    """Column sums of a 2-D bfloat16 / float16 / float32 tensor, fp32 accumulation, result in the tensor's type."""
     _require_gpu(a)
-    if a.dim() != 2 or a.dtype != torch.bfloat16:
-        raise ValueError("colsum_bf16: a 2-D bfloat16 tensor is required")
+    dt = _LINEAR_DTYPES.get(a.dtype)
+    if a.dim() != 2 or dt is None:
+        raise ValueError("colsum: a 2-D bfloat16, float16 or float32 tensor is required")
     if a.stride(1) != 1 and a.shape[1] > 1:
         a = a.contiguous()
     rows, cols = a.shape
-    out = torch.empty(cols, dtype=torch.bfloat16, device=a.device)
+    out = torch.empty(cols, dtype=a.dtype, device=a.device)
     splits = max(1, min(64, (rows + 127) // 128))
     work = torch.empty(splits * max(cols, 1), dtype=torch.float32, device=a.device)
-    rc = _lib.load().ddl_colsum_bf16(a.data_ptr(), rows, cols, a.stride(0) if rows > 1 else cols, out.data_ptr(),
-                                     work.data_ptr(), work.numel(), _stream())
-    _lib.check(rc, "ddl_colsum_bf16")
+    rc = _lib.load().ddl_colsum(a.data_ptr(), dt, rows, cols, a.stride(0) if rows > 1 else cols, out.data_ptr(),
+                                work.data_ptr(), work.numel(), _stream())
+    _lib.check(rc, "ddl_colsum")
     return out
 
 
-def linear_bf16_backward(x, weight, grad_output, need_input=True, need_weight=True, need_bias=True):
-    """Adjoint of :func:`linear_bf16`: ``(dx, dw, db)`` for ``y = x @ weight.T + bias``
-    (entries not asked for are None).  The operands that are not contiguous
-    along the reduction dimension are transposed into temporaries whose row
-    pitch is padded to a multiple of 8 with zeros, then the same GEMM runs."""
+def colsum_bf16(a):
+    """:func:`colsum` restricted to bfloat16."""
+    if a.dim() != 2 or a.dtype != torch.bfloat16:
+        raise ValueError("colsum_bf16: a 2-D bfloat16 tensor is required")
+    return colsum(a)
+
+
+def linear_backward(x, weight, grad_output, need_input=True, need_weight=True, need_bias=True):
+    """Adjoint of :func:`linear`: ``(dx, dw, db)`` for ``y = x @ weight.T + bias``
+    (entries not asked for are None).  float32 operands go through the strided
+    product, which reads them where they lie.  For the 16-bit types the operands
+    that are not contiguous along the reduction dimension are transposed into
+    temporaries whose row pitch is padded to a multiple of 8 with zeros, then the
+    forward kernel runs."""
     _require_gpu(x, weight, grad_output)
+    dt = _LINEAR_DTYPES.get(x.dtype)
+    if dt is None or weight.dtype != x.dtype or grad_output.dtype != x.dtype:
+        raise ValueError("linear_backward: operands must all be bfloat16, all float16 or all float32")
     n, k = weight.shape
     x2 = x.reshape(-1, k)
     dy = grad_output.reshape(-1, n)
@@ -536,31 +590,63 @@ def linear_bf16_backward(x, weight, grad_output, need_input=True, need_weight=Tr
         dy = dy.contiguous()
     m = x2.shape[0]
     dx = dw = db = None
+    if dt == _lib.DDL_DT_F32:
+        if x2.stride(1) != 1 and k > 1:
+            x2 = x2.contiguous()
+        if weight.stride(1) != 1 and k > 1:
+            weight = weight.contiguous()
+        lib = _lib.load()
+        ld_dy, ld_x, ld_w = (dy.stride(0) if m > 1 else n), (x2.stride(0) if m > 1 else k), (weight.stride(0) if n > 1 else k)
+        if need_input:
+            dx = torch.empty((m, k), dtype=x.dtype, device=x.device)
+            if n == 0:
+                dx.zero_()
+            else:   # dx[m, j] = sum_n dy[m, n] w[n, j]: rows of the second operand are the columns of w
+                rc = lib.ddl_gemm_f32(dy.data_ptr(), ld_dy, 1, weight.data_ptr(), 1, ld_w, None, dx.data_ptr(), k, m, k, n,
+                                      _stream())
+                _lib.check(rc, "ddl_gemm_f32")
+            dx = dx.reshape(x.shape)
+        if need_weight:
+            dw = torch.empty((n, k), dtype=x.dtype, device=x.device)
+            if m == 0:
+                dw.zero_()
+            else:   # dw[i, j] = sum_m dy[m, i] x[m, j]: both operands are read down their columns
+                rc = lib.ddl_gemm_f32(dy.data_ptr(), 1, ld_dy, x2.data_ptr(), 1, ld_x, None, dw.data_ptr(), k, n, k, m,
+                                      _stream())
+                _lib.check(rc, "ddl_gemm_f32")
+        if need_bias:
+            db = colsum(dy)
+        return dx, dw, db
     if need_input:
         # dx[m, k] = sum_n dy[m, n] w[n, k]: operands dy[M, N] and wT[K, N]
         np8 = _round_up(n, 8)
         w_t = transpose_2d(weight, np8)                       # [K, np8], padding columns zero
         dy_p = dy
         if np8 != n or (m > 1 and dy.stride(0) % 8 != 0) or dy.data_ptr() % 16 != 0:
-            dy_p = torch.zeros((m, np8), dtype=dy.dtype, device=dy.device)
-            full = [slice(0, m), slice(0, n)]
-            copy_box(dy, full, dy_p, full)
-        dx = _linear_padded(dy_p, w_t, m, k, np8).reshape(x.shape)
+            dy_p = _padded_k(dy, np8)
+        dx = _linear_padded(dy_p, w_t, m, k, np8, dt).reshape(x.shape)
     if need_weight:
         # dw[n, k] = sum_m dy[m, n] x[m, k]: operands dyT[N, M] and xT[K, M]
         mp8 = _round_up(m, 8)
         dy_t = transpose_2d(dy, mp8)                          # [N, mp8]
         x_t = transpose_2d(x2, mp8)                           # [K, mp8]
-        dw = _linear_padded(dy_t, x_t, n, k, mp8)
+        dw = _linear_padded(dy_t, x_t, n, k, mp8, dt)
     if need_bias:
-        db = colsum_bf16(dy)
+        db = colsum(dy)
     return dx, dw, db
 
 
-def _linear_padded(a, b, m, n, k_padded):
+def linear_bf16_backward(x, weight, grad_output, need_input=True, need_weight=True, need_bias=True):
+    """:func:`linear_backward`; kept under the name of the first, bfloat16-only version."""
+    return linear_backward(x, weight, grad_output, need_input, need_weight, need_bias)
+
+
+def _linear_padded(a, b, m, n, k_padded, dt):
     """``a[m, k_padded] @ b[n, k_padded].T`` where the padding columns are zero."""
-    out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
-    rc = _lib.load().ddl_linear_bf16(a.data_ptr(), b.data_ptr(), None, out.data_ptr(), m, n, k_padded,
-                                     a.stride(0) if m > 1 else k_padded, b.stride(0) if n > 1 else k_padded, n, _stream())
-    _lib.check(rc, "ddl_linear_bf16")
+    out = torch.empty((m, n), dtype=a.dtype, device=a.device)
+    if k_padded == 0 or m == 0 or n == 0:
+        return out.zero_()
+    rc = _lib.load().ddl_linear(a.data_ptr(), b.data_ptr(), None, out.data_ptr(), dt, m, n, k_padded,
+                                a.stride(0) if m > 1 else k_padded, b.stride(0) if n > 1 else k_padded, n, _stream())
+    _lib.check(rc, "ddl_linear")
     return out

@@ -1,7 +1,7 @@
 """DistributedLinear (reference: nn/linear.py:11-108): broadcast x over the rows
 of the weight partition, apply the local ``[out/P_fo, in/P_fi]`` shard, sum-reduce
 the partial outputs.  The local apply (reference :103, ``self.sublinear(x)``) is
-the bf16 MFMA kernel."""
+the MFMA kernel of the operands' type."""
 
 __all__ = ["DistributedLinear"]
 
@@ -22,22 +22,23 @@ class _LinearShard(torch.autograd.Function):
     def forward(ctx, x, weight, bias):
         ctx.save_for_backward(x, weight)
         ctx.has_bias = bias is not None
-        return hip_ops.linear_bf16(x.detach(), weight.detach(), None if bias is None else bias.detach())
+        return hip_ops.linear(x.detach(), weight.detach(), None if bias is None else bias.detach())
 
     @staticmethod
     def backward(ctx, grad_output):
         x, weight = ctx.saved_tensors
         need_x, need_w, need_b = ctx.needs_input_grad
-        dx, dw, db = hip_ops.linear_bf16_backward(x.detach(), weight.detach(), grad_output.detach().to(torch.bfloat16),
-                                                  need_x, need_w, need_b and ctx.has_bias)
+        dx, dw, db = hip_ops.linear_backward(x.detach(), weight.detach(), grad_output.detach().to(x.dtype),
+                                             need_x, need_w, need_b and ctx.has_bias)
         return dx, dw, db
 
 
 def linear_shard(x, weight, bias):
-    """``x @ weight.T + bias`` on the HIP kernel (bf16 operands only)."""
-    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
-        raise NotImplementedError(f"the linear shard kernel is bf16 only (got x {x.dtype}, weight {weight.dtype}); "
-                                  "convert the layer with .to(torch.bfloat16)")
+    """``x @ weight.T + bias`` on the HIP kernels: bfloat16 and float16 on the
+    tuned MFMA kernel, float32 (the layers' default) on the fp32 one."""
+    if x.dtype not in (torch.bfloat16, torch.float16, torch.float32) or weight.dtype != x.dtype:
+        raise NotImplementedError(f"the linear shard kernels take bfloat16, float16 or float32 operands of one type "
+                                  f"(got x {x.dtype}, weight {weight.dtype})")
     return _LinearShard.apply(x, weight, bias)
 
 

@@ -341,22 +341,44 @@ int ddl_embedding_backward_static(const void* dy, int dtype, int64_t dim, int64_
                                   void* dweight, int64_t ld_dw, void* stream);
 
 /* ------------------------------------------------------------------------ *
- * DistributedLinear shard GEMM (bf16 in, fp32 accumulate, bf16 out)
+ * DistributedLinear shard GEMM (fp32 accumulate; operands and result bf16,
+ * fp16 or fp32)
  * ------------------------------------------------------------------------ */
 
 /* y[M, N] = x[M, K] . w[N, K]^T + bias[N]   (bias may be NULL).
- * x, w, y row-major with leading dimensions ldx, ldw, ldy (elements).
+ * x, w, y row-major with leading dimensions ldx, ldw, ldy (elements), all of
+ * `dtype` (DDL_DT_BF16, DDL_DT_F16 or DDL_DT_F32), accumulation in fp32.
  * Replaces  self.sublinear(x)  nn/linear.py:103  and
- *   torch.nn.functional.linear(input, weight, bias)  nn/linear_ag.py:486. */
+ *   torch.nn.functional.linear(input, weight, bias)  nn/linear_ag.py:486.
+ * The 16-bit types run on the tuned MFMA kernel and need K, ldx, ldw multiples
+ * of 8 and x, w aligned to 16 bytes (DDL_E_ALIGN otherwise); fp32, the default
+ * dtype of the reference's layers and of its tests
+ * (tests/layers/test_linear.py:48-305), takes any K and pitch. */
+int ddl_linear(const void* x, const void* w, const void* bias, void* y, int dtype,
+               int64_t M, int64_t N, int64_t K,
+               int64_t ldx, int64_t ldw, int64_t ldy, void* stream);
+
+/* ddl_linear with dtype = DDL_DT_BF16. */
 int ddl_linear_bf16(const void* x, const void* w, const void* bias, void* y,
                     int64_t M, int64_t N, int64_t K,
                     int64_t ldx, int64_t ldw, int64_t ldy, void* stream);
 
-/* Adjoint of the shard GEMM (what autograd runs for the two calls above):
+/* The fp32 product with both operands addressed by two strides each (elements):
+ *   y[m, n] = sum_k a[m a_row_stride + k a_k_stride] b[n b_row_stride + k b_k_stride] + bias[n]
+ * so that the adjoint of the fp32 shard (what autograd runs for the two calls
+ * above: dx = dy . w, dw = dy^T . x) needs no transposed copies:
+ *   dx[M,K] = gemm(a = dy (N, 1),  b = w (1, K))       reduction over N
+ *   dw[N,K] = gemm(a = dy (1, N),  b = x (1, K))       reduction over M */
+int ddl_gemm_f32(const float* a, int64_t a_row_stride, int64_t a_k_stride,
+                 const float* b, int64_t b_row_stride, int64_t b_k_stride,
+                 const float* bias, float* y, int64_t ldy,
+                 int64_t M, int64_t N, int64_t K, void* stream);
+
+/* Adjoint of the 16-bit shard GEMM:
  *   dx = dy . w,   dw = dy^T . x,   db = column sums of dy.
- * ddl_linear_bf16 multiplies operands that are contiguous along the reduction
+ * The 16-bit kernel multiplies operands that are contiguous along the reduction
  * dimension, so the host transposes w (for dx), dy and x (for dw) with
- * ddl_transpose_2d into caller-provided buffers and calls ddl_linear_bf16 again:
+ * ddl_transpose_2d into caller-provided buffers and calls ddl_linear again:
  *   dx[M,K] = linear(dy[M,N],   wT[K,N])      dw[N,K] = linear(dyT[N,M], xT[K,M]).
  *
  * ddl_transpose_2d:  dst[c, r] = src[r, c] for r < rows, c < cols; 2-byte
@@ -364,10 +386,13 @@ int ddl_linear_bf16(const void* x, const void* w, const void* bias, void* y,
 int ddl_transpose_2d(const void* src, void* dst, int64_t rows, int64_t cols,
                      int64_t ld_src, int64_t ld_dst, int elem_size, void* stream);
 
-/* out[c] = bf16( sum over r < rows of a[r, c] ), fp32 accumulation, for the
- * bias gradient.  `workspace` is device memory for at least `cols` floats
- * (up to 64 * cols are used: one row of partial sums per row split); its
- * contents on entry do not matter. */
+/* out[c] = sum over r < rows of a[r, c], fp32 accumulation, rounded once to
+ * `dtype` (bf16, fp16 or fp32: the type of a and out), for the bias gradient.
+ * `workspace` is device memory for at least `cols` floats (up to 64 * cols are
+ * used: one row of partial sums per row split); its contents on entry do not
+ * matter.  ddl_colsum_bf16 is the bf16 form. */
+int ddl_colsum(const void* a, int dtype, int64_t rows, int64_t cols, int64_t ld,
+               void* out, float* workspace, int64_t workspace_elems, void* stream);
 int ddl_colsum_bf16(const void* a, int64_t rows, int64_t cols, int64_t ld,
                     void* out, float* workspace, int64_t workspace_elems,
                     void* stream);

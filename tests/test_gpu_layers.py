@@ -789,6 +789,123 @@ def test_linear_shard_autograd_matches_torch(ops):
             assert (err <= LIN_RTOL * (ref.abs() + ref.abs().mean())).all()
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("M,N,K", [(1, 1, 8), (32, 32, 16), (300, 200, 72), (513, 259, 136), (130, 1000, 1024), (7, 5, 3),
+                                   (129, 131, 17)])
+@pytest.mark.parametrize("use_bias", [True, False])
+def test_linear_fp16_and_fp32_small_integer_cases_are_exact(ops, dtype, M, N, K, use_bias):
+    """Small integers: every product and partial sum is exact, so the result
+    must equal the fp64 product exactly -- any indexing mistake shows.  fp32
+    takes any K; fp16 shapes with K not a multiple of 8 go through the padded
+    copies."""
+    gen = torch.Generator().manual_seed(M * 7 + N * 3 + K)
+    x = torch.randint(-2, 3, (M, K), generator=gen).to(dtype)
+    w = torch.randint(-2, 3, (N, K), generator=gen).to(dtype)
+    b = torch.randint(-3, 4, (N,), generator=gen).to(dtype) if use_bias else None
+    y = ops.linear(x.cuda(), w.cuda(), None if b is None else b.cuda())
+    want = x.double() @ w.double().T + (0 if b is None else b.double())
+    assert y.dtype == dtype and y.shape == (M, N)
+    assert torch.equal(y.cpu().double(), want)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float16, 2.0 ** -9), (torch.float32, 1e-5)])
+def test_linear_fp16_and_fp32_random_within_tolerance(ops, dtype, tol):
+    """Random operands against the fp64 product of the same values: fp32
+    accumulation and one rounding to the result type."""
+    gen = torch.Generator().manual_seed(77)
+    M, N, K = 384, 520, 2048
+    x = torch.randn(3, M // 3, K, generator=gen).to(dtype)
+    w = (0.05 * torch.randn(N, K, generator=gen)).to(dtype)
+    b = torch.randn(N, generator=gen).to(dtype)
+    y = ops.linear(x.cuda(), w.cuda(), b.cuda())
+    exact = x.double().reshape(-1, K) @ w.double().T + b.double()
+    mag = np.sqrt(K) * float(x.float().abs().mean()) * float(w.float().abs().mean())
+    err = (y.cpu().double().reshape(-1, N) - exact).abs()
+    assert bool((err <= tol * (exact.abs() + mag) + 1e-30).all()), float((err / (exact.abs() + mag)).max())
+    # the reference's call on the same values, on the CPU in float32
+    ref = F.linear(x.float(), w.float(), b.float())
+    assert torch.allclose(y.cpu().float(), ref, rtol=4 * tol, atol=4 * tol * float(ref.abs().mean()))
+
+
+def test_linear_bf16_forward_pads_unaligned_operands(ops):
+    """K not a multiple of 8, an offset view as input: the layer-level entry
+    copies into padded temporaries instead of refusing (the C entry point refuses)."""
+    gen = torch.Generator().manual_seed(5)
+    for K in (1, 12, 33):
+        x = torch.randint(-2, 3, (40, K), generator=gen).to(torch.bfloat16)
+        w = torch.randint(-2, 3, (24, K), generator=gen).to(torch.bfloat16)
+        y = ops.linear(x.cuda(), w.cuda())
+        assert torch.equal(y.cpu().double(), x.double() @ w.double().T)
+    base = torch.randint(-2, 3, (50, 72), generator=gen).to(torch.bfloat16).cuda()
+    view = base[3:43, 4:68]                                    # pitch 72, first element 8 bytes off a 16-byte boundary
+    w = torch.randint(-2, 3, (16, 64), generator=gen).to(torch.bfloat16)
+    y = ops.linear(view, w.cuda())
+    assert torch.equal(y.cpu().double(), view.cpu().double() @ w.double().T)
+    from distdl_amd import _lib
+    rc = _lib.load().ddl_linear(view.data_ptr(), w.cuda().data_ptr(), None, y.data_ptr(), _lib.DDL_DT_BF16, 40, 16, 64, 72, 64, 16,
+                                None)
+    assert rc == -3
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("M,N,K", [(8, 8, 8), (64, 48, 40), (300, 130, 72), (5, 3, 2), (129, 257, 33)])
+def test_linear_backward_fp16_and_fp32_exact_and_autograd(ops, dtype, M, N, K):
+    """dx = dy w, dw = dy^T x, db = column sums on small integers (exact), and
+    the autograd hook-up of the shard against torch's on the CPU."""
+    from distdl_amd.nn.linear import linear_shard
+    gen = torch.Generator().manual_seed(M + N + K)
+    x = torch.randint(-2, 3, (M, K), generator=gen).to(dtype)
+    w = torch.randint(-2, 3, (N, K), generator=gen).to(dtype)
+    dy = torch.randint(-2, 3, (M, N), generator=gen).to(dtype)
+    dx, dw, db = ops.linear_backward(x.cuda(), w.cuda(), dy.cuda())
+    assert torch.equal(dx.cpu().double(), dy.double() @ w.double())
+    assert torch.equal(dw.cpu().double(), dy.double().T @ x.double())
+    assert torch.equal(db.cpu().double(), dy.double().sum(0))
+    xg, wg = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+    bg = torch.zeros(N, dtype=dtype, device="cuda", requires_grad=True)
+    linear_shard(xg, wg, bg).backward(dy.cuda())
+    xr, wr, br = x.double().requires_grad_(True), w.double().requires_grad_(True), torch.zeros(N, dtype=torch.double, requires_grad=True)
+    F.linear(xr, wr, br).backward(dy.double())
+    assert torch.equal(xg.grad.cpu().double(), xr.grad) and torch.equal(wg.grad.cpu().double(), wr.grad)
+    assert torch.equal(bg.grad.cpu().double(), br.grad)
+
+
+def test_linear_layers_run_in_float32_like_the_reference_tests(ops):
+    """DistributedLinear keeps torch's default dtype, as in the reference's
+    layer tests (tests/layers/test_linear.py:48-305 build float32 layers): the
+    shard runs on the fp32 kernel, forward and backward, against torch on the CPU."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedLinear, DistributedLinearAllGather
+    Pw = SimWorld(8).partition(0)
+    P_x = Pw.create_partition_inclusive([0]).create_cartesian_topology_partition([1, 1])
+    P_y = Pw.create_partition_inclusive(list(range(8))).create_cartesian_topology_partition([1, 8])
+    P_w = Pw.create_partition_inclusive(list(range(8))).create_cartesian_topology_partition([8, 1])
+    torch.manual_seed(9)
+    layer = DistributedLinear(P_x, P_y, P_w, 60, 400)
+    assert layer.sublinear.weight.dtype == torch.float32 and tuple(layer.sublinear.weight.shape) == (50, 60)
+    x = torch.randn(33, 60)
+    xg = x.cuda().requires_grad_(True)
+    y = layer(xg)
+    y.backward(torch.ones_like(y))
+    w, b = layer.sublinear.weight.detach().cpu(), layer.sublinear.bias.detach().cpu()
+    xr = x.clone().requires_grad_(True)
+    wr, br = w.clone().requires_grad_(True), b.clone().requires_grad_(True)
+    yr = F.linear(xr, wr, br)
+    yr.backward(torch.ones_like(yr))
+    assert torch.allclose(y.detach().cpu(), yr.detach(), rtol=1e-5, atol=1e-5)
+    assert torch.allclose(xg.grad.cpu(), xr.grad, rtol=1e-5, atol=1e-5)
+    assert torch.allclose(layer.sublinear.weight.grad.cpu(), wr.grad, rtol=1e-5, atol=1e-4)
+    assert torch.allclose(layer.sublinear.bias.grad.cpu(), br.grad, rtol=1e-5, atol=1e-5)
+    P_y3 = Pw.create_partition_inclusive(list(range(8))).create_cartesian_topology_partition([1, 1, 8])
+    ag = DistributedLinearAllGather(P_y3, 72, 160)
+    assert ag.weight.dtype == torch.float32
+    x3 = torch.randn(2, 9, 72)
+    with torch.no_grad():
+        y3 = ag(x3.cuda())
+    want = F.linear(x3, ag.weight.detach().cpu().view(20, 72), ag.bias.detach().cpu().view(20))
+    assert torch.allclose(y3.cpu(), want, rtol=1e-5, atol=1e-5)
+
+
 def test_linear_layers_forward(ops):
     """DistributedLinear and DistributedLinearAllGather (solo rank 0 of 8,
     weights split on out_features) call the same kernel."""
