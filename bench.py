@@ -812,6 +812,22 @@ def build_launch_floor(torch, lib, _lib, nsets):
     return steps, [], 0
 
 
+def _build_mfma_probe(instruction, random):
+    def build(torch, lib, _lib, nsets):
+        """Nothing but MFMAs on register operands (ddl_probe_mfma): what the matrix
+        cores of this machine sustain with this instruction on this kind of data,
+        the ceiling the shard GEMM's figure is read against."""
+        sink = torch.empty(512 * 256, device="cuda")
+        flop = ctypes.c_int64(0)
+        iters = 4000
+        args = (instruction, random, iters, sink.data_ptr(), sink.numel(), ctypes.byref(flop))
+        rc = lib.ddl_probe_mfma(*args, STREAM[0])
+        _lib.check(rc, "ddl_probe_mfma")
+        torch.cuda.synchronize()
+        return [[_call(lib, _lib, "ddl_probe_mfma", args)] for _ in range(nsets)], [sink, flop], int(flop.value)
+    return build
+
+
 # name -> (builder, buffer sets, launches per step, bound, rule for combining the traffic figures of a step's kernels,
 #          layer timer, cpu baseline, BASELINE.json configuration number)
 WORKLOADS = {
@@ -830,6 +846,10 @@ WORKLOADS = {
     "embedding_bwd": (build_embedding_bwd, 4, 1, "hbm", None, None, None, None),
     "linear_bwd": (build_linear_bwd, 2, 1, "mfma", None, None, None, None),
     "launch_floor": (build_launch_floor, 8, 2, "hbm", None, None, None, None),
+    "mfma_32x32x16_constant": (_build_mfma_probe(0, 0), 1, 1, "mfma", None, None, None, None),
+    "mfma_32x32x16_random": (_build_mfma_probe(0, 1), 1, 1, "mfma", None, None, None, None),
+    "mfma_16x16x32_constant": (_build_mfma_probe(1, 0), 1, 1, "mfma", None, None, None, None),
+    "mfma_16x16x32_random": (_build_mfma_probe(1, 1), 1, 1, "mfma", None, None, None, None),
     # only with --only:
     "linear_library": (build_linear_library, 4, 1, "mfma", None, None, None, None),
     "calib": (build_calib, 4, 1, "hbm", None, None, None, None),

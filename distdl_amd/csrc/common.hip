@@ -22,20 +22,9 @@ int check_launch(const char* what) {
     return fail(static_cast<int>(e), "%s: %s", what, hipGetErrorString(e));
 }
 
-namespace {
-__global__ void probe_kernel() {}
-}  // namespace
-
 }  // namespace ddl
 
 extern "C" {
-
-int ddl_probe_launch(int64_t workgroups, int threads, void* stream) {
-    if (workgroups < 1 || workgroups > 0x7FFFFFFFll || threads < 1 || threads > 1024)
-        return ddl::fail(DDL_E_ARG, "probe: %lld workgroups of %d threads", (long long)workgroups, threads);
-    hipLaunchKernelGGL(ddl::probe_kernel, dim3(static_cast<uint32_t>(workgroups)), dim3(threads), 0, static_cast<hipStream_t>(stream));
-    return ddl::check_launch("probe_kernel");
-}
 
 const char* ddl_version(void) { return "distdl_hip 0.1.0 gfx950"; }
 
