@@ -751,34 +751,49 @@ def build_embedding_bwd(torch, lib, _lib, nsets):
     return steps, keep, sum(nbytes) / len(nbytes)
 
 
-def build_linear_bwd(torch, lib, _lib, nsets):
-    """Backward of config 4 on rank 0: dx = dy w and dw = dy^T x through the
-    shard GEMM on transposed operands (the three transposes are part of the
-    step), db = column sums of dy.  Work: 2 x 2 M N K flop."""
-    M, N, K = 8192, 3584, 8192
-    gen = torch.Generator(device="cuda").manual_seed(6004)
-    w = (0.02 * torch.randn(N, K, generator=gen, device="cuda")).to(torch.bfloat16)
-    w_t = torch.empty(K, N, dtype=torch.bfloat16, device="cuda")
-    dy_t = torch.empty(N, M, dtype=torch.bfloat16, device="cuda")
-    x_t = torch.empty(K, M, dtype=torch.bfloat16, device="cuda")
-    work = torch.empty(64 * N, device="cuda")
-    keep, steps = [w, w_t, dy_t, x_t, work], []
-    for s in range(nsets):
-        x = torch.randn(M, K, generator=gen, device="cuda").to(torch.bfloat16)
-        dy = torch.randn(M, N, generator=gen, device="cuda").to(torch.bfloat16)
-        dx = torch.empty(M, K, dtype=torch.bfloat16, device="cuda")
-        dw = torch.empty(N, K, dtype=torch.bfloat16, device="cuda")
-        db = torch.empty(N, dtype=torch.bfloat16, device="cuda")
-        keep.append((x, dy, dx, dw, db))
-        steps.append([
-            _call(lib, _lib, "ddl_transpose_2d", (w.data_ptr(), w_t.data_ptr(), N, K, K, N, 2)),
-            _call(lib, _lib, "ddl_linear_bf16", (dy.data_ptr(), w_t.data_ptr(), None, dx.data_ptr(), M, K, N, N, N, K)),
-            _call(lib, _lib, "ddl_transpose_2d", (dy.data_ptr(), dy_t.data_ptr(), M, N, N, M, 2)),
-            _call(lib, _lib, "ddl_transpose_2d", (x.data_ptr(), x_t.data_ptr(), M, K, K, M, 2)),
-            _call(lib, _lib, "ddl_linear_bf16", (dy_t.data_ptr(), x_t.data_ptr(), None, dw.data_ptr(), N, K, M, M, M, K)),
-            _call(lib, _lib, "ddl_colsum_bf16", (dy.data_ptr(), M, N, N, db.data_ptr(), work.data_ptr(), work.numel())),
-        ])
-    return steps, keep, 2 * 2 * M * N * K
+def _build_linear_bwd(in_place):
+    def build(torch, lib, _lib, nsets):
+        M, N, K = 8192, 3584, 8192
+        gen = torch.Generator(device="cuda").manual_seed(6004)
+        w = (0.02 * torch.randn(N, K, generator=gen, device="cuda")).to(torch.bfloat16)
+        work = torch.empty(64 * N, device="cuda")
+        keep, steps = [w, work], []
+        if not in_place:
+            w_t = torch.empty(K, N, dtype=torch.bfloat16, device="cuda")
+            dy_t = torch.empty(N, M, dtype=torch.bfloat16, device="cuda")
+            x_t = torch.empty(K, M, dtype=torch.bfloat16, device="cuda")
+            keep += [w_t, dy_t, x_t]
+        bf16 = _lib.DDL_DT_BF16
+        for s in range(nsets):
+            x = torch.randn(M, K, generator=gen, device="cuda").to(torch.bfloat16)
+            dy = torch.randn(M, N, generator=gen, device="cuda").to(torch.bfloat16)
+            dx = torch.empty(M, K, dtype=torch.bfloat16, device="cuda")
+            dw = torch.empty(N, K, dtype=torch.bfloat16, device="cuda")
+            db = torch.empty(N, dtype=torch.bfloat16, device="cuda")
+            keep.append((x, dy, dx, dw, db))
+            if in_place:
+                products = [
+                    _call(lib, _lib, "ddl_gemm", (dy.data_ptr(), N, 1, w.data_ptr(), 1, K, None, dx.data_ptr(), bf16, K, M, K, N)),
+                    _call(lib, _lib, "ddl_gemm", (dy.data_ptr(), 1, N, x.data_ptr(), 1, K, None, dw.data_ptr(), bf16, K, N, K, M)),
+                ]
+            else:
+                products = [
+                    _call(lib, _lib, "ddl_transpose_2d", (w.data_ptr(), w_t.data_ptr(), N, K, K, N, 2)),
+                    _call(lib, _lib, "ddl_linear_bf16", (dy.data_ptr(), w_t.data_ptr(), None, dx.data_ptr(), M, K, N, N, N, K)),
+                    _call(lib, _lib, "ddl_transpose_2d", (dy.data_ptr(), dy_t.data_ptr(), M, N, N, M, 2)),
+                    _call(lib, _lib, "ddl_transpose_2d", (x.data_ptr(), x_t.data_ptr(), M, K, K, M, 2)),
+                    _call(lib, _lib, "ddl_linear_bf16", (dy_t.data_ptr(), x_t.data_ptr(), None, dw.data_ptr(), N, K, M, M, M, K)),
+                ]
+            steps.append(products + [
+                _call(lib, _lib, "ddl_colsum_bf16", (dy.data_ptr(), M, N, N, db.data_ptr(), work.data_ptr(), work.numel())),
+            ])
+        return steps, keep, 2 * 2 * M * N * K
+    build.__doc__ = ("Backward of config 4 on rank 0: dx = dy w and dw = dy^T x through the shard GEMM, "
+                     + ("which reads w, dy and x where they lie (ddl_gemm)" if in_place else
+                        "on transposed copies of w, dy and x (the three transposes are part of the step; what shapes "
+                        "that ddl_gemm cannot read in place fall back to)")
+                     + ", db = column sums of dy.  Work: 2 x 2 M N K flop.")
+    return build
 
 
 # ----------------------------------------------------------------------------
@@ -844,7 +859,7 @@ WORKLOADS = {
     "halo_slabs_interior": (build_halo_slabs_interior, 8, 6, "hbm", None, None, None, None),
     "layernorm_bwd": (build_layernorm_bwd, 32, 2, "hbm", None, None, None, None),
     "embedding_bwd": (build_embedding_bwd, 4, 1, "hbm", None, None, None, None),
-    "linear_bwd": (build_linear_bwd, 2, 1, "mfma", None, None, None, None),
+    "linear_bwd": (_build_linear_bwd(True), 2, 1, "mfma", None, None, None, None),
     "launch_floor": (build_launch_floor, 8, 2, "hbm", None, None, None, None),
     "mfma_32x32x16_constant": (_build_mfma_probe(0, 0), 1, 1, "mfma", None, None, None, None),
     "mfma_32x32x16_random": (_build_mfma_probe(0, 1), 1, 1, "mfma", None, None, None, None),
@@ -852,9 +867,10 @@ WORKLOADS = {
     "mfma_16x16x32_random": (_build_mfma_probe(1, 1), 1, 1, "mfma", None, None, None, None),
     # only with --only:
     "linear_library": (build_linear_library, 4, 1, "mfma", None, None, None, None),
+    "linear_bwd_transposed": (_build_linear_bwd(False), 2, 1, "mfma", None, None, None, None),
     "calib": (build_calib, 4, 1, "hbm", None, None, None, None),
 }
-ONLY_ON_REQUEST = ("linear_library", "calib")
+ONLY_ON_REQUEST = ("linear_library", "linear_bwd_transposed", "calib")
 
 
 def cpu_host():

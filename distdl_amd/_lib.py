@@ -93,6 +93,8 @@ SIGNATURES = {
                                               c_int64, c_int, c_void_p, c_int64, c_void_p]),
     "ddl_linear": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int64,
                            c_int64, c_void_p]),
+    "ddl_gemm": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_int64, c_int64,
+                         c_int64, c_int64, c_void_p]),
     "ddl_gemm_f32": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_int64,
                              c_int64, c_int64, c_void_p]),
     "ddl_colsum": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int64, c_void_p]),

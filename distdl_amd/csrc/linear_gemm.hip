@@ -79,13 +79,30 @@ __device__ inline uint16_t f32_to_bf16_bits(float f) {
 
 __device__ inline float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(static_cast<uint32_t>(b) << 16); }
 
-typedef __attribute__((address_space(3))) void* lds_ptr;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// Raw buffer descriptor over all of memory from `base` on (no stride, no bounds).
+__device__ inline u32x4 raw_buffer(const void* base) {
+    const uint64_t a = reinterpret_cast<uint64_t>(base);
+    u32x4 r;
+    r[0] = static_cast<uint32_t>(a), r[1] = static_cast<uint32_t>(a >> 32) & 0xFFFFu, r[2] = 0xFFFFFFFFu, r[3] = 0x00020000u;
+    return r;
+}
 
 // One wavefront instruction: lane l copies the 16 bytes at byte (voffset +
 // soffset) of the buffer to LDS byte (dst + 16 l); dst and soffset are the same
-// for all lanes.
-__device__ inline void dma16(__amdgpu_buffer_rsrc_t buffer, int voffset, int soffset, char* dst) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(buffer, (lds_ptr)dst, 16, voffset, soffset, 0, 0);
+// for all lanes.  Written as assembly: the compiler makes every later LDS read
+// through a transposing read wait for all such copies in flight (it cannot
+// tell that they go to another ring slot), which would serialise the pipeline.
+// The kernel waits for these copies itself (s_waitcnt vmcnt in front of the
+// barriers); the compiler does not count them, which only makes its own waits
+// for ordinary loads longer, never shorter (requests complete in order).
+__device__ inline void dma16(u32x4 buffer, int voffset, int soffset, const char* dst) {
+    const uint32_t lds_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst));   // low half of a generic LDS address: the LDS offset
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voffset), "s"(buffer), "s"(soffset)
+                 : "memory", "m0");
 }
 
 // acc += a . b (16 x 16 x 32, bf16 in, fp32 accumulate).  Written as assembly
@@ -142,7 +159,7 @@ struct Part {
     int tiles_m, tiles_n, vec_store;
 };
 
-template <bool F16, int NWM, int NWN, int TM, int TN>
+template <bool F16, bool XT, bool WT, int NWM, int NWN, int TM, int TN>
 __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* lds) {
     static_assert(NWM * NWN == 8, "eight wavefronts per workgroup");
     const uint16_t* __restrict__ x = part.x;
@@ -188,74 +205,123 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[a][b][e] = 0.f;
 
-    // Global -> LDS requests of this lane.  Instruction j of this wavefront
-    // fills rows (J wave + j) 8 .. +7 of an operand tile (J instructions per
-    // wavefront); lane l lands on row
-    // l / 8, physical chunk l % 8 of that row, i.e. logical chunk
-    // (l % 8) ^ ((row >> 1) & 7): the eight lanes of a row fetch one whole
-    // 128-byte line.  Rows past the end of the matrix repeat its last row
-    // (their products are never stored).
-    // The operands are addressed as raw buffers that start at the tile's first
-    // row: a 32-bit byte offset per lane, the k-tile offset in a scalar.
-    const char* const base_w = reinterpret_cast<const char*>(w + n0 * ldw);
-    const char* const base_x = reinterpret_cast<const char*>(x + m0 * ldx);
-    const __amdgpu_buffer_rsrc_t buf_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base_w), 0, -1, 0x00020000);
-    const __amdgpu_buffer_rsrc_t buf_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base_x), 0, -1, 0x00020000);
+    // Global -> LDS requests of this lane.  The operands are addressed as raw
+    // buffers that start at the tile's first row: a 32-bit byte offset per lane,
+    // the k-tile offset in a scalar.
+    //
+    // Operand contiguous along k: instruction j of this wavefront fills rows
+    // (J wave + j) 8 .. +7 of an operand tile (J instructions per wavefront);
+    // lane l lands on row l / 8, physical chunk l % 8 of that row, i.e. logical
+    // chunk (l % 8) ^ ((row >> 1) & 7): the eight lanes of a row fetch one whole
+    // 128-byte line.  Rows past the end of the matrix repeat its last row (their
+    // products are never stored).
+    //
+    // Operand contiguous along its rows ("transposed": element (row, k) lies at
+    // k ld + row): the tile is kept in LDS as panels of 64 rows, each panel 64
+    // k-lines of 128 bytes.  Instruction j of wavefront v fills k-lines 8 v .. +7
+    // of panel j; lane l lands on k-line l / 8, physical chunk l % 8, and fetches
+    // the logical chunk (l % 8) ^ 2 h(k), h(k) = bit 1 of k + 2 (bit 3 of k): again
+    // one whole 128-byte line per eight lanes.  Chunks past the last row of the
+    // matrix repeat the first chunk of the tile.
+    const char* const base_w = reinterpret_cast<const char*>(WT ? w + n0 : w + n0 * ldw);
+    const char* const base_x = reinterpret_cast<const char*>(XT ? x + m0 : x + m0 * ldx);
+    const u32x4 buf_w = raw_buffer(base_w), buf_x = raw_buffer(base_x);
+    // bytes from one k-tile of an operand to the next
+    const int step_w = WT ? static_cast<int>(ldw) * (BK * 2) : BK * 2;
+    const int step_x = XT ? static_cast<int>(ldx) * (BK * 2) : BK * 2;
     int off_gw[JW_W], off_gx[JW_X];
     {
-        const int r = lane >> 3;
+        auto lane_offset = [&](bool transposed, int J, int j, int64_t origin, int64_t rows, int64_t ld) -> int {
+            if (!transposed) {
+                const int row = (J * wave + j) * 8 + (lane >> 3);
+                const int ck = ((lane & 7) ^ ((row >> 1) & 7)) * 8;   // first k of this lane's chunk inside a k-tile
+                const int64_t rr = origin + row < rows ? row : rows - 1 - origin;
+                return static_cast<int>((rr * ld + ck) * 2);
+            }
+            const int k = 8 * wave + (lane >> 3);
+            const int h = ((k >> 1) & 1) | (((k >> 3) & 1) << 1);
+            int col = j * 64 + ((lane & 7) ^ (h << 1)) * 8;              // first tile row of this lane's chunk
+            if (origin + col >= rows) col = 0;
+            return static_cast<int>((k * ld + col) * 2);
+        };
 #pragma unroll
-        for (int j = 0; j < JW_W; ++j) {
-            const int row = (JW_W * wave + j) * 8 + r;
-            const int ck = ((lane & 7) ^ ((row >> 1) & 7)) * 8;   // first k of this lane's chunk inside a k-tile
-            const int64_t rn = n0 + row < N ? row : N - 1 - n0;
-            off_gw[j] = static_cast<int>((rn * ldw + ck) * 2);
-        }
+        for (int j = 0; j < JW_W; ++j) off_gw[j] = lane_offset(WT, JW_W, j, n0, N, ldw);
 #pragma unroll
-        for (int j = 0; j < JW_X; ++j) {
-            const int row = (JW_X * wave + j) * 8 + r;
-            const int ck = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
-            const int64_t rm = m0 + row < M ? row : M - 1 - m0;
-            off_gx[j] = static_cast<int>((rm * ldx + ck) * 2);
-        }
+        for (int j = 0; j < JW_X; ++j) off_gx[j] = lane_offset(XT, JW_X, j, m0, M, ldx);
     }
 
     const int ktiles = static_cast<int>((K + BK - 1) / BK);
     const int full_tiles = static_cast<int>(K / BK);   // tiles [full_tiles, ktiles) straddle K
 
+    // LDS byte, inside an operand tile, where request instruction j of this wavefront starts.
+    auto lds_dst = [&](bool transposed, int J, int j) { return transposed ? j * 8192 + wave * 1024 : (J * wave + j) * 1024; };
     // One request instruction (j = 0 .. J-1) of operand tile t, a full tile.
-    auto request_part = [&](__amdgpu_buffer_rsrc_t buf, const auto& off, int t, int unit_off, int j) {
+    auto request_part = [&](auto transposed, u32x4 buf, const auto& off, int step, int t, int unit_off, int j) {
         constexpr int J = sizeof(off) / sizeof(int);
-        dma16(buf, off[j], t * (BK * 2), lds + unit_off + (J * wave + j) * 1024);
+        dma16(buf, off[j], t * step, lds + unit_off + lds_dst(decltype(transposed)::value, J, j));
     };
     // A whole operand tile.  One that straddles K goes through registers so
-    // that the chunks past K can be written as zeros.
-    auto request_unit = [&](__amdgpu_buffer_rsrc_t buf, const char* base, const auto& off, int t, int unit_off) {
+    // that the elements past K can be written as zeros.
+    auto request_unit = [&](auto transposed, u32x4 buf, const char* base, const auto& off, int step, int t, int unit_off) {
         constexpr int J = sizeof(off) / sizeof(int);
+        constexpr bool T = decltype(transposed)::value;
         if (t < full_tiles) {
 #pragma unroll
-            for (int j = 0; j < J; ++j) request_part(buf, off, t, unit_off, j);
+            for (int j = 0; j < J; ++j) request_part(transposed, buf, off, step, t, unit_off, j);
         } else {
 #pragma unroll
             for (int j = 0; j < J; ++j) {
-                const int row = (J * wave + j) * 8 + (lane >> 3);
-                const int ck = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
+                bool inside;
+                if (T) {
+                    inside = static_cast<int64_t>(t) * BK + 8 * wave + (lane >> 3) < K;
+                } else {
+                    const int row = (J * wave + j) * 8 + (lane >> 3);
+                    const int ck = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
+                    inside = static_cast<int64_t>(t) * BK + ck < K;
+                }
                 uint4 v = make_uint4(0, 0, 0, 0);
-                if (static_cast<int64_t>(t) * BK + ck < K)
-                    v = *reinterpret_cast<const uint4*>(base + off[j] + static_cast<int64_t>(t) * (BK * 2));
-                *reinterpret_cast<uint4*>(lds + unit_off + (J * wave + j) * 1024 + lane * 16) = v;
+                if (inside) v = *reinterpret_cast<const uint4*>(base + off[j] + static_cast<int64_t>(t) * step);
+                *reinterpret_cast<uint4*>(lds + unit_off + lds_dst(T, J, j) + lane * 16) = v;
             }
         }
     };
+    const std::integral_constant<bool, WT> w_kind{};
+    const std::integral_constant<bool, XT> x_kind{};
 
-    // Fragment addresses: row (sub-tile origin + l16), logical chunk 4 ks + kg.
-    // Sub-tile origins are multiples of 16, so the swizzle term is (l16 >> 1) & 7.
+    // Fragment addresses.  Operand contiguous along k: row (sub-tile origin +
+    // l16), logical chunk 4 ks + kg; sub-tile origins are multiples of 16, so the
+    // swizzle term is (l16 >> 1) & 7.
     const int frag_row = l16 * (BK * 2);
     int sw_off[2];   // byte offset of this lane's chunk in its row, per k-step
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) sw_off[ks] = ((4 * ks + kg) ^ ((l16 >> 1) & 7)) << 4;
     const int off_w = wn * (BK * 2) + frag_row;
     const int off_x = wm * (BK * 2) + frag_row;
+    // Transposed operand: the 16 rows of a sub-tile are 32 bytes of a k-line.  A
+    // transposing read (ds_read_b64_tr_b16) works per group of 16 lanes: lane i
+    // of the group points at 8 bytes = 4 rows, (k-line i / 4, rows 4 (i % 4) ..
+    // +3), and receives row i of k-lines 0 .. 3 -- half of the eight k this lane
+    // feeds to the MFMA; the k-lines four further down give the other half.
+    // Group kg of the wavefront covers k-lines 8 kg .. + 7 of the k-step.  The
+    // 32-byte unit index is XOR-ed with h(k) (see the requests): the 32 lanes
+    // served per LDS cycle read 8 different k-lines, and (k & 1, unit ^ h(k)) is
+    // distinct for each, so they cover all 64 banks.
+    const int tr_lane = (8 * kg + (l16 >> 2)) * 128 + (l16 & 3) * 8;
+    const int tr_h = (((l16 >> 3) & 1) | ((kg & 1) << 1)) << 5;
+    typedef short short4v __attribute__((ext_vector_type(4)));
+    typedef short short8v __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) short4v* lds_short4;
+    // Piece of a transposed operand tile: 16-row block `sub` of the tile, k-step ks.
+    auto read_transposed = [&](const char* tile, int sub, int ks) -> bf16x8 {
+        const char* p = tile + (sub >> 2) * 8192 + ks * (32 * 128) + (tr_lane + (((sub & 3) << 5) ^ tr_h));
+        const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4)(p));
+        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4)(p + 4 * 128));
+        const short8v both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        bf16x8 out;
+        __builtin_memcpy(&out, &both, 16);
+        return out;
+    };
+    const int sub_w = (wave / NWM) * TN, sub_x = (wave % NWM) * TM;   // first 16-row block of this wavefront in the w and x tiles
 
     // The operand with more pieces per wavefront runs in the outer loop of a
     // k-step: a piece of it is used by a few consecutive MFMAs and is dead
@@ -274,9 +340,9 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
         const int idx = r == 0 ? 0 : (r <= NI ? r - 1 : r - NI);
         const bool is_x = outer == kOuterX;
         if (is_x)
-            fb[idx] = *reinterpret_cast<const bf16x8*>(xt + off_x + idx * (16 * BK * 2) + sw);
+            fb[idx] = XT ? read_transposed(xt, sub_x + idx, ks) : *reinterpret_cast<const bf16x8*>(xt + off_x + idx * (16 * BK * 2) + sw);
         else
-            fa[idx] = *reinterpret_cast<const bf16x8*>(wt + off_w + idx * (16 * BK * 2) + sw);
+            fa[idx] = WT ? read_transposed(wt, sub_w + idx, ks) : *reinterpret_cast<const bf16x8*>(wt + off_w + idx * (16 * BK * 2) + sw);
     };
 
     // Request instructions go behind even MFMAs (the fragment reads take the odd
@@ -317,8 +383,8 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
         const char* xn1 = lds + unit_off(s0 + 3);
         const int w2_off = unit_off(s0 + 4);   // slot of X(t-1), free since the barrier of tile t-1
         const int x2_off = unit_off(s0);       // slot of W(t), free after this tile's barrier
-        if (!STEADY && t + 2 < ktiles) request_unit(buf_w, base_w, off_gw, t + 2, w2_off);
-        k_step(0, wt, xt, 1, kGapW - 2, kGapW, STEADY ? JW_W : 0, [&](int j) { request_part(buf_w, off_gw, t + 2, w2_off, j); });
+        if (!STEADY && t + 2 < ktiles) request_unit(w_kind, buf_w, base_w, off_gw, step_w, t + 2, w2_off);
+        k_step(0, wt, xt, 1, kGapW - 2, kGapW, STEADY ? JW_W : 0, [&](int j) { request_part(w_kind, buf_w, off_gw, step_w, t + 2, w2_off, j); });
         // Own requests of W(t+1), X(t+1) have landed (W(t+2)'s may still be in
         // flight) and every LDS read issued so far -- all of tile t's -- has
         // returned; the barrier extends both to the workgroup, so tile t+1 may
@@ -326,17 +392,17 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
         __builtin_amdgcn_s_waitcnt(STEADY ? wait_vm_lgkm0(JW_W) : wait_vm_lgkm0(0));
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        if (!STEADY && t + 2 < ktiles) request_unit(buf_x, base_x, off_gx, t + 2, x2_off);
+        if (!STEADY && t + 2 < ktiles) request_unit(x_kind, buf_x, base_x, off_gx, step_x, t + 2, x2_off);
         // Past the last tile the reads of this k-step fetch stale LDS contents that are never used.
-        k_step(1, wn1, xn1, 0, 0, 2, STEADY ? JW_X : 0, [&](int j) { request_part(buf_x, off_gx, t + 2, x2_off, j); });
+        k_step(1, wn1, xn1, 0, 0, 2, STEADY ? JW_X : 0, [&](int j) { request_part(x_kind, buf_x, off_gx, step_x, t + 2, x2_off, j); });
         s0 = s0 + 2 >= kUnits ? s0 + 2 - kUnits : s0 + 2;
     };
 
-    request_unit(buf_w, base_w, off_gw, 0, 0);
-    request_unit(buf_x, base_x, off_gx, 0, kUnitBytes);
+    request_unit(w_kind, buf_w, base_w, off_gw, step_w, 0, 0);
+    request_unit(x_kind, buf_x, base_x, off_gx, step_x, 0, kUnitBytes);
     if (ktiles > 1) {
-        request_unit(buf_w, base_w, off_gw, 1, 2 * kUnitBytes);
-        request_unit(buf_x, base_x, off_gx, 1, 3 * kUnitBytes);
+        request_unit(w_kind, buf_w, base_w, off_gw, step_w, 1, 2 * kUnitBytes);
+        request_unit(x_kind, buf_x, base_x, off_gx, step_x, 1, 3 * kUnitBytes);
     }
     // Tile 0 complete and visible, then its first fragments.
     __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
@@ -455,65 +521,77 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
 constexpr int kThreads = 512;
 
 // 256 x 256 tiles: 2 x 4 wavefronts of 128 x 64.
-template <bool F16>
-__global__ __launch_bounds__(kThreads) void linear16_wide(const Part part) {
+template <bool F16, bool XT, bool WT>
+__global__ __launch_bounds__(kThreads) void gemm16_wide(const Part part) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
-    gemm_tile<F16, 2, 4, 8, 4>(part, blockIdx.x, lds);
+    gemm_tile<F16, XT, WT, 2, 4, 8, 4>(part, blockIdx.x, lds);
 }
 
 // 256 x 192 tiles: 4 x 2 wavefronts of 64 x 96.
-template <bool F16>
-__global__ __launch_bounds__(kThreads) void linear16_narrow(const Part part) {
+template <bool F16, bool XT, bool WT>
+__global__ __launch_bounds__(kThreads) void gemm16_narrow(const Part part) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
-    gemm_tile<F16, 4, 2, 4, 6>(part, blockIdx.x, lds);
+    gemm_tile<F16, XT, WT, 4, 2, 4, 6>(part, blockIdx.x, lds);
 }
+
+typedef void (*Kernel)(const Part);
+// index: 8 fp16 + 4 (x transposed) + 2 (w transposed) + narrow
+const Kernel kKernels[16] = {
+    gemm16_wide<false, false, false>, gemm16_narrow<false, false, false>, gemm16_wide<false, false, true>, gemm16_narrow<false, false, true>,
+    gemm16_wide<false, true, false>,  gemm16_narrow<false, true, false>,  gemm16_wide<false, true, true>,  gemm16_narrow<false, true, true>,
+    gemm16_wide<true, false, false>,  gemm16_narrow<true, false, false>,  gemm16_wide<true, false, true>,  gemm16_narrow<true, false, true>,
+    gemm16_wide<true, true, false>,   gemm16_narrow<true, true, false>,   gemm16_wide<true, true, true>,   gemm16_narrow<true, true, true>,
+};
 
 // Per-device state, set on first use by whichever thread gets there (the
 // values are the same for all of them).
 constexpr int kMaxDevices = 64;
-std::atomic<bool> lds_reserved[kMaxDevices][4];   // the dynamic LDS size of kernel (fp16 ? 2 : 0) + (narrow ? 1 : 0) has been raised
+std::atomic<bool> lds_reserved[kMaxDevices][16];  // the dynamic LDS size of kKernels[i] has been raised
 std::atomic<int> cu_count[kMaxDevices];           // 0: not asked yet
 
-}  // namespace
-}  // namespace ddl
+// One operand of the product: element (row, k) at p[row * row_stride + k * k_stride],
+// one of the strides being 1.
+struct Operand {
+    const uint16_t* p;
+    int64_t row_stride, k_stride;
+    bool transposed() const { return row_stride == 1 && k_stride != 1; }
+    int64_t ld() const { return transposed() ? k_stride : row_stride; }
+};
 
-extern "C" int ddl_gemm_f32(const float* a, int64_t a_row_stride, int64_t a_k_stride, const float* b, int64_t b_row_stride,
-                            int64_t b_k_stride, const float* bias, float* y, int64_t ldy, int64_t M, int64_t N, int64_t K,
-                            void* stream);
-
-extern "C" int ddl_linear_bf16(const void* x, const void* w, const void* bias, void* y, int64_t M, int64_t N, int64_t K,
-                               int64_t ldx, int64_t ldw, int64_t ldy, void* stream) {
-    return ddl_linear(x, w, bias, y, DDL_DT_BF16, M, N, K, ldx, ldw, ldy, stream);
+// What the kernel asks of an operand with `rows` rows; 0 or an error code.
+int check_operand(const char* who, const char* name, const Operand& o, int64_t rows, int64_t K) {
+    if (o.row_stride != 1 && o.k_stride != 1)
+        return fail(DDL_E_UNSUPP, "%s: operand %s has no unit stride (row stride %lld, k stride %lld)", who, name, (long long)o.row_stride,
+                    (long long)o.k_stride);
+    const int64_t ld = o.ld();
+    if (!aligned_to(o.p, 16) || ld % 8 != 0) return fail(DDL_E_ALIGN, "%s: operand %s must be 16-byte aligned with a pitch that is a multiple of 8", who, name);
+    if (ld > 0x3FFFFF) return fail(DDL_E_UNSUPP, "%s: pitch of %s above 2^22 elements", who, name);   // 32-bit byte offsets inside a tile
+    if (o.transposed()) {
+        if (ld < rows) return fail(DDL_E_ARG, "%s: pitch %lld of %s below its %lld rows", who, (long long)ld, name, (long long)rows);
+        if (rows % 8 != 0) return fail(DDL_E_ALIGN, "%s: %s is read along its rows, whose number must be a multiple of 8", who, name);
+        if ((K + BK) * ld > 0x3FFFFFFF) return fail(DDL_E_UNSUPP, "%s: %s spans more than 2^31 bytes along k", who, name);
+    } else {
+        if (ld < K) return fail(DDL_E_ARG, "%s: pitch %lld of %s below K=%lld", who, (long long)ld, name, (long long)K);
+        if (K % 8 != 0) return fail(DDL_E_ALIGN, "%s: %s is read along k, so K must be a multiple of 8", who, name);
+        if (K > 0x3FFFFFFF) return fail(DDL_E_UNSUPP, "%s: K above 2^30", who);
+    }
+    return 0;
 }
 
-extern "C" int ddl_linear(const void* x, const void* w, const void* bias, void* y, int dtype, int64_t M, int64_t N, int64_t K,
-                          int64_t ldx, int64_t ldw, int64_t ldy, void* stream) {
-    using namespace ddl;
-    if (dtype != DDL_DT_BF16 && dtype != DDL_DT_F16 && dtype != DDL_DT_F32)
-        return fail(DDL_E_UNSUPP, "linear: dtype %d (bf16, f16 and f32 only)", dtype);
-    if (dtype == DDL_DT_F32) {
-        if (ldx < K || ldw < K) return fail(DDL_E_ARG, "linear: ldx=%lld ldw=%lld below K=%lld", (long long)ldx, (long long)ldw, (long long)K);
-        return ddl_gemm_f32(static_cast<const float*>(x), ldx, 1, static_cast<const float*>(w), ldw, 1, static_cast<const float*>(bias),
-                            static_cast<float*>(y), ldy, M, N, K, stream);
-    }
-    const bool f16 = dtype == DDL_DT_F16;
-    if (M < 0 || N < 0 || K < 0 || ldx < K || ldw < K || ldy < N)
-        return fail(DDL_E_ARG, "linear: M=%lld N=%lld K=%lld ldx=%lld ldw=%lld ldy=%lld", (long long)M, (long long)N,
-                    (long long)K, (long long)ldx, (long long)ldw, (long long)ldy);
+// y[M, N] = a[M, K] . b[N, K]^T + bias in 16-bit elements.
+int gemm16(const char* who, bool f16, Operand a, Operand b, const uint16_t* bias, uint16_t* y, int64_t ldy, int64_t M, int64_t N, int64_t K,
+           void* stream) {
+    if (M < 0 || N < 0 || K < 0 || ldy < N)
+        return fail(DDL_E_ARG, "%s: M=%lld N=%lld K=%lld ldy=%lld", who, (long long)M, (long long)N, (long long)K, (long long)ldy);
     if (M == 0 || N == 0) return 0;
-    if (!x || !w || !y) return fail(DDL_E_ARG, "linear: null pointer");
-    if (K == 0) return fail(DDL_E_UNSUPP, "linear: K = 0");
-    if (K % 8 != 0 || ldx % 8 != 0 || ldw % 8 != 0 || !aligned_to(x, 16) || !aligned_to(w, 16))
-        return fail(DDL_E_ALIGN, "linear: K, ldx, ldw must be multiples of 8 and x, w 16-byte aligned");
-    if (!aligned_to(y, 2) || (bias && !aligned_to(bias, 2))) return fail(DDL_E_ALIGN, "linear: y / bias misaligned");
-    if (ldx > 0x3FFFFF || ldw > 0x3FFFFF || K > 0x3FFFFFFF)
-        return fail(DDL_E_UNSUPP, "linear: row pitch above 2^22 elements or K above 2^30");   // 32-bit byte offsets inside a tile
+    if (!a.p || !b.p || !y) return fail(DDL_E_ARG, "%s: null pointer", who);
+    if (K == 0) return fail(DDL_E_UNSUPP, "%s: K = 0", who);
+    if (int rc = check_operand(who, "a", a, M, K)) return rc;
+    if (int rc = check_operand(who, "b", b, N, K)) return rc;
+    if (!aligned_to(y, 2) || (bias && !aligned_to(bias, 2))) return fail(DDL_E_ALIGN, "%s: y / bias misaligned", who);
     // 2: rows of y can be stored 16 bytes at a time, 1: 8 bytes, 0: element by element
     const int vec_store = (ldy % 8 == 0 && aligned_to(y, 16)) ? 2 : (ldy % 4 == 0 && aligned_to(y, 8)) ? 1 : 0;
-    const uint16_t* const xp = static_cast<const uint16_t*>(x);
-    const uint16_t* const wp = static_cast<const uint16_t*>(w);
-    const uint16_t* const bp = static_cast<const uint16_t*>(bias);
-    uint16_t* const yp = static_cast<uint16_t*>(y);
+    const bool at = a.transposed(), bt = b.transposed();
 
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
@@ -524,18 +602,16 @@ extern "C" int ddl_linear(const void* x, const void* w, const void* bias, void* 
         cus = n;
         cu_count[dev].store(n, std::memory_order_relaxed);
     }
-    auto launch = [&](int which, const Part& p) -> int {
-        typedef void (*Kernel)(const Part);
-        const Kernel kernels[4] = {linear16_wide<false>, linear16_narrow<false>, linear16_wide<true>, linear16_narrow<true>};
-        const int k = (f16 ? 2 : 0) + which;
+    auto launch = [&](int narrow, const Part& p) -> int {
+        const int k = (f16 ? 8 : 0) + (at ? 4 : 0) + (bt ? 2 : 0) + narrow;
         if (!lds_reserved[dev][k].load(std::memory_order_acquire)) {   // the attribute sticks to the function on this device
-            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernels[k]), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-            if (e != hipSuccess) return fail(static_cast<int>(e), "linear: cannot reserve %d bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kKernels[k]), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+            if (e != hipSuccess) return fail(static_cast<int>(e), "%s: cannot reserve %d bytes of LDS: %s", who, kLdsBytes, hipGetErrorString(e));
             lds_reserved[dev][k].store(true, std::memory_order_release);
         }
         const dim3 grid(static_cast<uint32_t>(static_cast<int64_t>(p.tiles_m) * p.tiles_n));
-        hipLaunchKernelGGL(kernels[k], grid, dim3(kThreads), kLdsBytes, static_cast<hipStream_t>(stream), p);
-        return check_launch(which == 0 ? "linear16_wide" : "linear16_narrow");
+        hipLaunchKernelGGL(kKernels[k], grid, dim3(kThreads), kLdsBytes, static_cast<hipStream_t>(stream), p);
+        return check_launch(narrow ? "gemm16_narrow" : "gemm16_wide");
     };
 
     // How many 256-column strips go to the wide tiles: whole rounds of them,
@@ -554,13 +630,13 @@ extern "C" int ddl_linear(const void* x, const void* w, const void* bias, void* 
     // Columns [n_begin, n_begin + n_count) of the output with tiles of 256 x bn.
     auto part = [&](int bn, int64_t n_begin, int64_t n_count) {
         Part p{};
-        p.x = xp, p.w = wp + n_begin * ldw, p.bias = bp ? bp + n_begin : nullptr, p.y = yp + n_begin;
-        p.M = M, p.N = n_count, p.K = K, p.ldx = ldx, p.ldw = ldw, p.ldy = ldy;
+        p.x = a.p, p.w = b.p + n_begin * b.row_stride, p.bias = bias ? bias + n_begin : nullptr, p.y = y + n_begin;
+        p.M = M, p.N = n_count, p.K = K, p.ldx = a.ld(), p.ldw = b.ld(), p.ldy = ldy;
         p.tiles_m = static_cast<int>(tiles_m), p.tiles_n = static_cast<int>((n_count + bn - 1) / bn), p.vec_store = vec_store;
         return p;
     };
     if (tiles_m > 0x7FFFFFll || cols > 0x7FFFFFll || tiles_m * (cols + 1) > 0x7FFFFFFFll)
-        return fail(DDL_E_UNSUPP, "linear: too many output tiles");
+        return fail(DDL_E_UNSUPP, "%s: too many output tiles", who);
     const int64_t wide_cols = best_split == cols ? N : best_split * 256;
     if (wide_cols > 0) {
         const int rc = launch(0, part(256, 0, wide_cols));
@@ -568,4 +644,38 @@ extern "C" int ddl_linear(const void* x, const void* w, const void* bias, void* 
     }
     if (wide_cols < N) return launch(1, part(192, wide_cols, N - wide_cols));
     return 0;
+}
+
+}  // namespace
+}  // namespace ddl
+
+extern "C" int ddl_gemm_f32(const float* a, int64_t a_row_stride, int64_t a_k_stride, const float* b, int64_t b_row_stride,
+                            int64_t b_k_stride, const float* bias, float* y, int64_t ldy, int64_t M, int64_t N, int64_t K,
+                            void* stream);
+
+extern "C" int ddl_linear_bf16(const void* x, const void* w, const void* bias, void* y, int64_t M, int64_t N, int64_t K,
+                               int64_t ldx, int64_t ldw, int64_t ldy, void* stream) {
+    return ddl_linear(x, w, bias, y, DDL_DT_BF16, M, N, K, ldx, ldw, ldy, stream);
+}
+
+extern "C" int ddl_linear(const void* x, const void* w, const void* bias, void* y, int dtype, int64_t M, int64_t N, int64_t K,
+                          int64_t ldx, int64_t ldw, int64_t ldy, void* stream) {
+    using namespace ddl;
+    if (dtype != DDL_DT_BF16 && dtype != DDL_DT_F16 && dtype != DDL_DT_F32)
+        return fail(DDL_E_UNSUPP, "linear: dtype %d (bf16, f16 and f32 only)", dtype);
+    if (ldx < K || ldw < K) return fail(DDL_E_ARG, "linear: ldx=%lld ldw=%lld below K=%lld", (long long)ldx, (long long)ldw, (long long)K);
+    // A pitch of 1 would read as "contiguous along the rows" below; it can only belong to a K = 1 operand, which the 16-bit kernel refuses anyway.
+    return ddl_gemm(x, ldx, 1, w, ldw, 1, bias, y, dtype, ldy, M, N, K, stream);
+}
+
+extern "C" int ddl_gemm(const void* a, int64_t a_row_stride, int64_t a_k_stride, const void* b, int64_t b_row_stride, int64_t b_k_stride,
+                        const void* bias, void* y, int dtype, int64_t ldy, int64_t M, int64_t N, int64_t K, void* stream) {
+    using namespace ddl;
+    if (dtype == DDL_DT_F32)
+        return ddl_gemm_f32(static_cast<const float*>(a), a_row_stride, a_k_stride, static_cast<const float*>(b), b_row_stride, b_k_stride,
+                            static_cast<const float*>(bias), static_cast<float*>(y), ldy, M, N, K, stream);
+    if (dtype != DDL_DT_BF16 && dtype != DDL_DT_F16) return fail(DDL_E_UNSUPP, "gemm: dtype %d (bf16, f16 and f32 only)", dtype);
+    const Operand oa{static_cast<const uint16_t*>(a), a_row_stride, a_k_stride};
+    const Operand ob{static_cast<const uint16_t*>(b), b_row_stride, b_k_stride};
+    return gemm16("gemm", dtype == DDL_DT_F16, oa, ob, static_cast<const uint16_t*>(bias), static_cast<uint16_t*>(y), ldy, M, N, K, stream);
 }

@@ -574,11 +574,12 @@ def colsum_bf16(a):
 
 def linear_backward(x, weight, grad_output, need_input=True, need_weight=True, need_bias=True):
     """Adjoint of :func:`linear`: ``(dx, dw, db)`` for ``y = x @ weight.T + bias``
-    (entries not asked for are None).  float32 operands go through the strided
-    product, which reads them where they lie.  For the 16-bit types the operands
-    that are not contiguous along the reduction dimension are transposed into
-    temporaries whose row pitch is padded to a multiple of 8 with zeros, then the
-    forward kernel runs."""
+    (entries not asked for are None).  Both products read their operands where
+    they lie: the float32 one through strides, the 16-bit one through
+    transposing LDS reads, which need row counts and pitches that are multiples
+    of 8; 16-bit operands that do not qualify are transposed into temporaries
+    whose row pitch is padded to a multiple of 8 with zeros, and the forward
+    kernel runs on those."""
     _require_gpu(x, weight, grad_output)
     dt = _LINEAR_DTYPES.get(x.dtype)
     if dt is None or weight.dtype != x.dtype or grad_output.dtype != x.dtype:
@@ -617,23 +618,54 @@ def linear_backward(x, weight, grad_output, need_input=True, need_weight=True, n
         if need_bias:
             db = colsum(dy)
         return dx, dw, db
+    if x2.stride(1) != 1 and k > 1:
+        x2 = x2.contiguous()
+    if weight.stride(1) != 1 and k > 1:
+        weight = weight.contiguous()
+    ld_dy, ld_x, ld_w = (dy.stride(0) if m > 1 else n), (x2.stride(0) if m > 1 else k), (weight.stride(0) if n > 1 else k)
     if need_input:
-        # dx[m, k] = sum_n dy[m, n] w[n, k]: operands dy[M, N] and wT[K, N]
-        np8 = _round_up(n, 8)
-        w_t = transpose_2d(weight, np8)                       # [K, np8], padding columns zero
-        dy_p = dy
-        if np8 != n or (m > 1 and dy.stride(0) % 8 != 0) or dy.data_ptr() % 16 != 0:
-            dy_p = _padded_k(dy, np8)
-        dx = _linear_padded(dy_p, w_t, m, k, np8, dt).reshape(x.shape)
+        # dx[m, j] = sum_n dy[m, n] w[n, j]: dy is read along n, w down its columns
+        if m and n and k and _along_k_ok(dy, ld_dy, n) and _along_rows_ok(weight, ld_w, k, n):
+            dx = torch.empty((m, k), dtype=x.dtype, device=x.device)
+            rc = _lib.load().ddl_gemm(dy.data_ptr(), ld_dy, 1, weight.data_ptr(), 1, ld_w, None, dx.data_ptr(), dt, k, m, k, n,
+                                      _stream())
+            _lib.check(rc, "ddl_gemm")
+            dx = dx.reshape(x.shape)
+        else:   # operands dy[M, N] and wT[K, N], padded
+            np8 = _round_up(n, 8)
+            w_t = transpose_2d(weight, np8)                       # [K, np8], padding columns zero
+            dy_p = dy
+            if np8 != n or (m > 1 and dy.stride(0) % 8 != 0) or dy.data_ptr() % 16 != 0:
+                dy_p = _padded_k(dy, np8)
+            dx = _linear_padded(dy_p, w_t, m, k, np8, dt).reshape(x.shape)
     if need_weight:
-        # dw[n, k] = sum_m dy[m, n] x[m, k]: operands dyT[N, M] and xT[K, M]
-        mp8 = _round_up(m, 8)
-        dy_t = transpose_2d(dy, mp8)                          # [N, mp8]
-        x_t = transpose_2d(x2, mp8)                           # [K, mp8]
-        dw = _linear_padded(dy_t, x_t, n, k, mp8, dt)
+        # dw[i, j] = sum_m dy[m, i] x[m, j]: both operands are read down their columns
+        if m and n and k and _along_rows_ok(dy, ld_dy, n, m) and _along_rows_ok(x2, ld_x, k, m):
+            dw = torch.empty((n, k), dtype=x.dtype, device=x.device)
+            rc = _lib.load().ddl_gemm(dy.data_ptr(), 1, ld_dy, x2.data_ptr(), 1, ld_x, None, dw.data_ptr(), dt, k, n, k, m,
+                                      _stream())
+            _lib.check(rc, "ddl_gemm")
+        else:   # operands dyT[N, M] and xT[K, M], padded
+            mp8 = _round_up(m, 8)
+            dy_t = transpose_2d(dy, mp8)                          # [N, mp8]
+            x_t = transpose_2d(x2, mp8)                           # [K, mp8]
+            dw = _linear_padded(dy_t, x_t, n, k, mp8, dt)
     if need_bias:
         db = colsum(dy)
     return dx, dw, db
+
+
+def _along_k_ok(t, pitch, depth):
+    """Can the 16-bit product read ``t`` (rows contiguous along the reduction
+    dimension of length ``depth``) where it lies?"""
+    return depth % 8 == 0 and pitch % 8 == 0 and pitch <= 0x3FFFFF and t.data_ptr() % 16 == 0
+
+
+def _along_rows_ok(t, pitch, rows, depth):
+    """Can the 16-bit product read ``t`` down its columns (``rows`` of them, each
+    of length ``depth`` along the reduction dimension) where it lies?"""
+    return (rows % 8 == 0 and pitch % 8 == 0 and pitch <= 0x3FFFFF and t.data_ptr() % 16 == 0
+            and (depth + 64) * pitch <= 0x3FFFFFFF)
 
 
 def linear_bf16_backward(x, weight, grad_output, need_input=True, need_weight=True, need_bias=True):

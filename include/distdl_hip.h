@@ -375,26 +375,37 @@ int ddl_linear_bf16(const void* x, const void* w, const void* bias, void* y,
                     int64_t M, int64_t N, int64_t K,
                     int64_t ldx, int64_t ldw, int64_t ldy, void* stream);
 
-/* The fp32 product with both operands addressed by two strides each (elements):
+/* The product with both operands addressed by two strides each (elements):
  *   y[m, n] = sum_k a[m a_row_stride + k a_k_stride] b[n b_row_stride + k b_k_stride] + bias[n]
- * so that the adjoint of the fp32 shard (what autograd runs for the two calls
- * above: dx = dy . w, dw = dy^T . x) needs no transposed copies:
+ * so that the adjoint of the shard (what autograd runs for ddl_linear:
+ * dx = dy . w, dw = dy^T . x, torch's linear backward behind nn/linear.py:103)
+ * needs no transposed copies:
  *   dx[M,K] = gemm(a = dy (N, 1),  b = w (1, K))       reduction over N
- *   dw[N,K] = gemm(a = dy (1, N),  b = x (1, K))       reduction over M */
+ *   dw[N,K] = gemm(a = dy (1, N),  b = x (1, K))       reduction over M
+ * a, b, bias and y are of `dtype`; y is row-major with pitch ldy.
+ * fp32: any strides.  bf16 / fp16 (the MFMA kernel of ddl_linear, which reads an
+ * operand that is contiguous along its rows through transposing LDS reads): each
+ * operand needs one stride equal to 1, the other (its pitch) a multiple of 8, and
+ * 16-byte alignment; an operand contiguous along k needs K % 8 == 0, one
+ * contiguous along its rows needs a row count (M for a, N for b) that is a
+ * multiple of 8 (DDL_E_ALIGN otherwise) and (K + 64) * pitch < 2^30 elements
+ * (DDL_E_UNSUPP otherwise: transpose it with ddl_transpose_2d instead).
+ * ddl_gemm_f32 is the fp32 form. */
+int ddl_gemm(const void* a, int64_t a_row_stride, int64_t a_k_stride,
+             const void* b, int64_t b_row_stride, int64_t b_k_stride,
+             const void* bias, void* y, int dtype, int64_t ldy,
+             int64_t M, int64_t N, int64_t K, void* stream);
 int ddl_gemm_f32(const float* a, int64_t a_row_stride, int64_t a_k_stride,
                  const float* b, int64_t b_row_stride, int64_t b_k_stride,
                  const float* bias, float* y, int64_t ldy,
                  int64_t M, int64_t N, int64_t K, void* stream);
 
-/* Adjoint of the 16-bit shard GEMM:
- *   dx = dy . w,   dw = dy^T . x,   db = column sums of dy.
- * The 16-bit kernel multiplies operands that are contiguous along the reduction
- * dimension, so the host transposes w (for dx), dy and x (for dw) with
- * ddl_transpose_2d into caller-provided buffers and calls ddl_linear again:
- *   dx[M,K] = linear(dy[M,N],   wT[K,N])      dw[N,K] = linear(dyT[N,M], xT[K,M]).
- *
- * ddl_transpose_2d:  dst[c, r] = src[r, c] for r < rows, c < cols; 2-byte
- * elements only (elem_size = 2); ld_src >= cols, ld_dst >= rows. */
+/* dst[c, r] = src[r, c] for r < rows, c < cols; 2-byte elements only
+ * (elem_size = 2); ld_src >= cols, ld_dst >= rows.  For the operands of the
+ * adjoint that ddl_gemm cannot read where they lie (row counts that are not
+ * multiples of 8): transposed into a buffer whose pitch is padded with zeros,
+ * they go through ddl_linear,
+ *   dx[M,K] = linear(dy[M,N],   wT[K,N])      dw[N,K] = linear(dyT[N,M], xT[K,M]). */
 int ddl_transpose_2d(const void* src, void* dst, int64_t rows, int64_t cols,
                      int64_t ld_src, int64_t ld_dst, int elem_size, void* stream);
 

@@ -906,6 +906,87 @@ def test_linear_layers_run_in_float32_like_the_reference_tests(ops):
     assert torch.allclose(y3.cpu(), want, rtol=1e-5, atol=1e-5)
 
 
+def _gemm_operand(values, transposed, pad):
+    """Device tensor holding ``values[rows, k]`` contiguous along k, or (transposed)
+    along the rows, with `pad` unused elements at the end of each line; returns
+    (tensor, row_stride, k_stride)."""
+    rows, k = values.shape
+    if transposed:
+        store = torch.full((k, rows + pad), 3.0, dtype=values.dtype)
+        store[:, :rows] = values.T
+        return store.cuda(), 1, rows + pad
+    store = torch.full((rows, k + pad), 3.0, dtype=values.dtype)
+    store[:, :k] = values
+    return store.cuda(), k + pad, 1
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("a_t,b_t", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("M,N,K,pad", [(8, 8, 8, 0), (16, 24, 72, 8), (304, 200, 136, 0), (264, 40, 64, 16), (520, 776, 200, 8),
+                                       (4096, 4352, 136, 0), (64, 192, 4104, 0)])
+def test_gemm_16_bit_reads_operands_where_they_lie(ops, dtype, a_t, b_t, M, N, K, pad):
+    """ddl_gemm on every combination of operand layouts (contiguous along k or
+    along the rows), with small integers so that the result must be the exact
+    integer: tiles that straddle M, N and K, pitched operands, one k-tile and
+    many, and a shape that is split between wide and narrow tiles."""
+    from distdl_amd import _lib
+    gen = torch.Generator().manual_seed(M * 7 + N * 3 + K + 2 * a_t + b_t)
+    a = torch.randint(-1, 2, (M, K), generator=gen).to(dtype)
+    b = torch.randint(-1, 2, (N, K), generator=gen).to(dtype)
+    b = b * (torch.rand(N, K, generator=gen) < min(1.0, 64.0 / K)).to(dtype)
+    bias = torch.randint(-3, 4, (N,), generator=gen).to(dtype)
+    ag, a_rs, a_ks = _gemm_operand(a, a_t, pad)
+    bg, b_rs, b_ks = _gemm_operand(b, b_t, pad)
+    ldy = N + 8
+    out = torch.full((M, ldy), 77.0, dtype=dtype, device="cuda")
+    dt = _lib.DDL_DT_BF16 if dtype == torch.bfloat16 else _lib.DDL_DT_F16
+    rc = _lib.load().ddl_gemm(ag.data_ptr(), a_rs, a_ks, bg.data_ptr(), b_rs, b_ks, bias.cuda().data_ptr(), out.data_ptr(), dt, ldy,
+                              M, N, K, torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "ddl_gemm")
+    want = a.double() @ b.double().T + bias.double()
+    assert want.abs().max() <= 256
+    got = out.cpu().double()
+    assert torch.equal(got[:, :N], want)
+    assert (got[:, N:] == 77.0).all()
+
+
+@pytest.mark.parametrize("a_t,b_t", [(False, True), (True, True)])
+def test_gemm_16_bit_random_within_tolerance_and_ragged_depth(ops, a_t, b_t):
+    """Random operands, a reduction length that is no multiple of the k-tile
+    (and, with both operands read down their columns, of nothing at all)."""
+    from distdl_amd import _lib
+    M, N, K = 328, 272, (1000 if not a_t else 1003)
+    gen = torch.Generator().manual_seed(K)
+    a = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    b = (0.02 * torch.randn(N, K, generator=gen)).to(torch.bfloat16)
+    ag, a_rs, a_ks = _gemm_operand(a, a_t, 0)
+    bg, b_rs, b_ks = _gemm_operand(b, b_t, 0)
+    out = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    rc = _lib.load().ddl_gemm(ag.data_ptr(), a_rs, a_ks, bg.data_ptr(), b_rs, b_ks, None, out.data_ptr(), _lib.DDL_DT_BF16, N,
+                              M, N, K, torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "ddl_gemm")
+    _lin_check(bits16(out), a, b, None)
+
+
+def test_gemm_16_bit_refuses_what_it_cannot_read_in_place(ops):
+    from distdl_amd import _lib
+    lib = _lib.load()
+    a = torch.zeros(64, 64, dtype=torch.bfloat16, device="cuda")
+    y = torch.zeros(64, 64, dtype=torch.bfloat16, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    bf16 = _lib.DDL_DT_BF16
+    # an operand read down its columns whose row count is no multiple of 8
+    assert lib.ddl_gemm(a.data_ptr(), 1, 64, a.data_ptr(), 64, 1, None, y.data_ptr(), bf16, 64, 60, 64, 64, stream) == -3
+    # no unit stride
+    assert lib.ddl_gemm(a.data_ptr(), 2, 64, a.data_ptr(), 64, 1, None, y.data_ptr(), bf16, 64, 16, 64, 16, stream) == -5
+    # reduction length that an operand read along k cannot take
+    assert lib.ddl_gemm(a.data_ptr(), 64, 1, a.data_ptr(), 1, 64, None, y.data_ptr(), bf16, 64, 64, 64, 60, stream) == -3
+    # pitch below the row count
+    assert lib.ddl_gemm(a.data_ptr(), 1, 8, a.data_ptr(), 64, 1, None, y.data_ptr(), bf16, 64, 64, 64, 8, stream) == -1
+    assert b"rows" in lib.ddl_last_error()
+    torch.cuda.synchronize()
+
+
 def test_linear_layers_forward(ops):
     """DistributedLinear and DistributedLinearAllGather (solo rank 0 of 8,
     weights split on out_features) call the same kernel."""
