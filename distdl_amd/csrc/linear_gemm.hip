@@ -375,8 +375,14 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
     // are in fa[0] / fb[0] or on their way, W(t+1) and X(t+1) have been
     // requested.  STEADY: tile t+2 exists and is a full tile; its request
     // instructions are spread between the MFMAs.
-    auto k_tile = [&](int t, auto steady) {
+    // `slot` is the ring slot of W(t): the running s0, or a compile-time constant
+    // (the steady loop is unrolled over the five positions of the ring, so
+    // that LDS addresses are immediates instead of scalar arithmetic that all
+    // wavefronts of a SIMD would run at the same moment, right after a barrier,
+    // with the matrix cores idle).
+    auto k_tile = [&](int t, auto steady, auto slot) {
         constexpr bool STEADY = decltype(steady)::value;
+        const int s0 = slot;
         const char* wt = lds + unit_off(s0);
         const char* xt = lds + unit_off(s0 + 1);
         const char* wn1 = lds + unit_off(s0 + 2);
@@ -395,8 +401,8 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
         if (!STEADY && t + 2 < ktiles) request_unit(x_kind, buf_x, base_x, off_gx, step_x, t + 2, x2_off);
         // Past the last tile the reads of this k-step fetch stale LDS contents that are never used.
         k_step(1, wn1, xn1, 0, 0, 2, STEADY ? JW_X : 0, [&](int j) { request_part(x_kind, buf_x, off_gx, step_x, t + 2, x2_off, j); });
-        s0 = s0 + 2 >= kUnits ? s0 + 2 - kUnits : s0 + 2;
     };
+    auto advance = [&]() { s0 = s0 + 2 >= kUnits ? s0 + 2 - kUnits : s0 + 2; };
 
     request_unit(w_kind, buf_w, base_w, off_gw, step_w, 0, 0);
     request_unit(x_kind, buf_x, base_x, off_gx, step_x, 0, kUnitBytes);
@@ -414,9 +420,17 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
     const int steady_end = full_tiles - 2 > 0 ? full_tiles - 2 : 0;
     int t = 0;
 #pragma unroll 1
-    for (; t < steady_end; ++t) k_tile(t, std::true_type{});
+    for (; t + kUnits <= steady_end; t += kUnits) {   // s0 == 0 here: five tiles bring the ring back to where it was
+        k_tile(t, std::true_type{}, std::integral_constant<int, 0>{});
+        k_tile(t + 1, std::true_type{}, std::integral_constant<int, 2>{});
+        k_tile(t + 2, std::true_type{}, std::integral_constant<int, 4>{});
+        k_tile(t + 3, std::true_type{}, std::integral_constant<int, 1>{});
+        k_tile(t + 4, std::true_type{}, std::integral_constant<int, 3>{});
+    }
 #pragma unroll 1
-    for (; t < ktiles; ++t) k_tile(t, std::false_type{});
+    for (; t < steady_end; ++t, advance()) k_tile(t, std::true_type{}, s0);
+#pragma unroll 1
+    for (; t < ktiles; ++t, advance()) k_tile(t, std::false_type{}, s0);
 
     // The last MFMAs must have left the pipeline before acc is read by anything
     // else (18 wait states cover every case; these are 32).
