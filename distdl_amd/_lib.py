@@ -74,6 +74,17 @@ SIGNATURES = {
     "ddl_ln_normalize_affine_f32": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int, POINTER(c_int64),
                                             c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_void_p,
                                             c_void_p]),
+    "ddl_ln_bwd_partial": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
+                                   c_void_p, c_void_p]),
+    "ddl_ln_bwd_input": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
+                                 c_void_p, c_int, c_float, c_void_p, c_int64, c_void_p]),
+    "ddl_ln_bwd_params": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
+                                  c_void_p, c_void_p, c_int64, c_void_p]),
+    "ddl_ln_bwd_partial_params": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
+                                          c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
+    "ddl_ln_bwd_input_params": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
+                                        c_void_p, c_void_p, c_int, c_float, c_void_p, c_int64, c_void_p, c_int64,
+                                        c_void_p, c_void_p, c_void_p]),
     "ddl_ln_bwd_partial_f32": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
                                        c_void_p, c_void_p]),
     "ddl_ln_bwd_input_f32": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,

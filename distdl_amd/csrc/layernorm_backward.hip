@@ -1,4 +1,4 @@
-// Backward of the DistributedLayerNorm shard, fp32: what autograd derives from
+// Backward of the DistributedLayerNorm shard: what autograd derives from
 // the reference's forward (nn/layernorm.py:230-247, 295-309)
 //
 //   mean = allreduce(local mean) / P        var = allreduce(local mean((x-mean)^2)) / P
@@ -18,9 +18,12 @@
 //   ln_bwd_input     sums the gathered pairs, writes dx      (one read of dy, x)
 //   ln_bwd_params    column sums over the local rows, in row splits through a
 //                    workspace, for dgamma and dbeta
-// One wavefront owns a row and strides over its columns (float4 when the row is
-// aligned); nothing is kept between passes, so rows of any length work.
-#include "ddl_common.h"
+// One wavefront owns a row and strides over its columns (four elements at a time
+// when the row is aligned); nothing is kept between passes, so rows of any length
+// work.  dy, x, gamma, dx, dgamma and dbeta are float, bf16 or fp16 (one type per
+// call); the arithmetic, the saved mean and rstd, the row sums and the workspace
+// are fp32.
+#include "ln_elements.h"
 
 namespace ddl {
 namespace {
@@ -36,33 +39,33 @@ __device__ inline float wave_sum(float v) {
     return v;
 }
 
-template <bool VEC>
-__global__ __launch_bounds__(kBlock) void ln_bwd_partial(const float* __restrict__ dy, const float* __restrict__ x, int64_t rows,
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kBlock) void ln_bwd_partial(const T* __restrict__ dy, const T* __restrict__ x, int64_t rows,
                                                          int64_t cols, int64_t ld_dy, int64_t ld_x,
                                                          const float* __restrict__ mean, const float* __restrict__ rstd,
-                                                         const float* __restrict__ gamma, float* __restrict__ sums) {
+                                                         const T* __restrict__ gamma, float* __restrict__ sums) {
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t r = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + threadIdx.x / kWave;
     if (r >= rows) return;
     const float m = mean[r], rs = rstd[r];
-    const float* dyr = dy + r * ld_dy;
-    const float* xr = x + r * ld_x;
+    const T* dyr = dy + r * ld_dy;
+    const T* xr = x + r * ld_x;
     float s1 = 0.f, s2 = 0.f;
     if (VEC) {
         for (int64_t c = lane * 4; c < cols; c += kWave * 4) {
-            const float4 d = *reinterpret_cast<const float4*>(dyr + c);
-            const float4 v = *reinterpret_cast<const float4*>(xr + c);
+            const float4 d = load4(dyr + c);
+            const float4 v = load4(xr + c);
             float4 g = make_float4(1.f, 1.f, 1.f, 1.f);
-            if (gamma) g = *reinterpret_cast<const float4*>(gamma + c);
+            if (gamma) g = load4(gamma + c);
             const float g0 = d.x * g.x, g1 = d.y * g.y, g2 = d.z * g.z, g3 = d.w * g.w;
             s1 += (g0 + g1) + (g2 + g3);
             s2 += (g0 * ((v.x - m) * rs) + g1 * ((v.y - m) * rs)) + (g2 * ((v.z - m) * rs) + g3 * ((v.w - m) * rs));
         }
     } else {
         for (int64_t c = lane; c < cols; c += kWave) {
-            const float g = dyr[c] * (gamma ? gamma[c] : 1.f);
+            const float g = load1(dyr + c) * (gamma ? load1(gamma + c) : 1.f);
             s1 += g;
-            s2 += g * ((xr[c] - m) * rs);
+            s2 += g * ((load1(xr + c) - m) * rs);
         }
     }
     s1 = wave_sum(s1);
@@ -70,11 +73,11 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_partial(const float* __restrict
     if (lane == 0) reinterpret_cast<float2*>(sums)[r] = make_float2(s1, s2);
 }
 
-template <bool VEC>
-__device__ inline void ln_bwd_input_body(uint32_t block, const float* __restrict__ dy, const float* __restrict__ x, int64_t rows,
+template <typename T, bool VEC>
+__device__ inline void ln_bwd_input_body(uint32_t block, const T* __restrict__ dy, const T* __restrict__ x, int64_t rows,
                                          int64_t cols, int64_t ld_dy, int64_t ld_x, const float* __restrict__ mean,
-                                         const float* __restrict__ rstd, const float* __restrict__ gamma,
-                                         const float* __restrict__ part_sums, int nparts, float weight, float* __restrict__ dx,
+                                         const float* __restrict__ rstd, const T* __restrict__ gamma,
+                                         const float* __restrict__ part_sums, int nparts, float weight, T* __restrict__ dx,
                                          int64_t ld_dx) {
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t r = static_cast<int64_t>(block) * kWavesPerBlock + threadIdx.x / kWave;
@@ -88,46 +91,44 @@ __device__ inline void ln_bwd_input_body(uint32_t block, const float* __restrict
     }
     const float m = mean[r], rs = rstd[r];
     const float S1 = wave_sum(p1) * weight, S2 = wave_sum(p2) * weight;   // already times a_p
-    const float* dyr = dy + r * ld_dy;
-    const float* xr = x + r * ld_x;
-    float* dxr = dx + r * ld_dx;
+    const T* dyr = dy + r * ld_dy;
+    const T* xr = x + r * ld_x;
+    T* dxr = dx + r * ld_dx;
     if (VEC) {
         for (int64_t c = lane * 4; c < cols; c += kWave * 4) {
-            const float4 d = *reinterpret_cast<const float4*>(dyr + c);
-            const float4 v = *reinterpret_cast<const float4*>(xr + c);
+            const float4 d = load4(dyr + c);
+            const float4 v = load4(xr + c);
             float4 g = make_float4(1.f, 1.f, 1.f, 1.f);
-            if (gamma) g = *reinterpret_cast<const float4*>(gamma + c);
+            if (gamma) g = load4(gamma + c);
             float4 o;
             o.x = rs * (d.x * g.x - (S1 + ((v.x - m) * rs) * S2));
             o.y = rs * (d.y * g.y - (S1 + ((v.y - m) * rs) * S2));
             o.z = rs * (d.z * g.z - (S1 + ((v.z - m) * rs) * S2));
             o.w = rs * (d.w * g.w - (S1 + ((v.w - m) * rs) * S2));
-            typedef float f32x4 __attribute__((ext_vector_type(4)));   // dx is not read again here: streaming store
-            f32x4 ov;
-            ov[0] = o.x, ov[1] = o.y, ov[2] = o.z, ov[3] = o.w;
-            __builtin_nontemporal_store(ov, reinterpret_cast<f32x4*>(dxr + c));
+            store4(dxr + c, o);   // dx is not read again here: streaming store
         }
     } else {
         for (int64_t c = lane; c < cols; c += kWave) {
-            const float g = dyr[c] * (gamma ? gamma[c] : 1.f);
-            dxr[c] = rs * (g - (S1 + ((xr[c] - m) * rs) * S2));
+            const float g = load1(dyr + c) * (gamma ? load1(gamma + c) : 1.f);
+            store1(dxr + c, rs * (g - (S1 + ((load1(xr + c) - m) * rs) * S2)));
         }
     }
 }
 
-template <bool VEC>
-__global__ __launch_bounds__(kBlock) void ln_bwd_input(const float* __restrict__ dy, const float* __restrict__ x, int64_t rows,
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kBlock) void ln_bwd_input(const T* __restrict__ dy, const T* __restrict__ x, int64_t rows,
                                                        int64_t cols, int64_t ld_dy, int64_t ld_x,
                                                        const float* __restrict__ mean, const float* __restrict__ rstd,
-                                                       const float* __restrict__ gamma, const float* __restrict__ part_sums,
-                                                       int nparts, float weight, float* __restrict__ dx, int64_t ld_dx) {
-    ln_bwd_input_body<VEC>(blockIdx.x, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, part_sums, nparts, weight, dx, ld_dx);
+                                                       const T* __restrict__ gamma, const float* __restrict__ part_sums,
+                                                       int nparts, float weight, T* __restrict__ dx, int64_t ld_dx) {
+    ln_bwd_input_body<T, VEC>(blockIdx.x, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, part_sums, nparts, weight, dx, ld_dx);
 }
 
 // Workgroup (strip, split): rows [split * rows_per_split, ...) of a 64-column
 // strip; lane group t / 64 takes every fourth row, thread t % 64 one column.
 // partial[split, 0, c] = sum dy xhat, partial[split, 1, c] = sum dy.
-__global__ __launch_bounds__(kBlock) void ln_bwd_params_partial(const float* __restrict__ dy, const float* __restrict__ x,
+template <typename T>
+__global__ __launch_bounds__(kBlock) void ln_bwd_params_partial(const T* __restrict__ dy, const T* __restrict__ x,
                                                                 int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
                                                                 const float* __restrict__ mean, const float* __restrict__ rstd,
                                                                 int64_t rows_per_split, float* __restrict__ partial, int strips) {
@@ -140,8 +141,8 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_params_partial(const float* __r
     float a = 0.f, b = 0.f;
     if (c < cols) {
         for (int64_t r = r_begin + g; r < r_end; r += kWavesPerBlock) {
-            const float d = dy[r * ld_dy + c];
-            a += d * ((x[r * ld_x + c] - mean[r]) * rstd[r]);
+            const float d = load1(dy + r * ld_dy + c);
+            a += d * ((load1(x + r * ld_x + c) - mean[r]) * rstd[r]);
             b += d;
         }
     }
@@ -160,8 +161,9 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_params_partial(const float* __r
 // Workgroup per 64-column strip: lane group g = t / 64 adds the splits g, g+4,
 // ... of column t % 64 (independent loads, eight in flight), LDS folds the four
 // groups.
+template <typename T>
 __device__ inline void ln_bwd_params_final_body(uint32_t block, const float* __restrict__ partial, int64_t cols, int splits,
-                                                float* __restrict__ dgamma, float* __restrict__ dbeta) {
+                                                T* __restrict__ dgamma, T* __restrict__ dbeta) {
     __shared__ float fold[2][kWavesPerBlock][kStrip];
     const int g = threadIdx.x / kStrip, t = threadIdx.x % kStrip;
     const int64_t c = static_cast<int64_t>(block) * kStrip + t;
@@ -194,32 +196,33 @@ __device__ inline void ln_bwd_params_final_body(uint32_t block, const float* __r
         float s = 0.f;
 #pragma unroll
         for (int k = 0; k < kWavesPerBlock; ++k) s += fold[which][k][t];
-        float* out = which == 0 ? dgamma : dbeta;
-        if (out) out[c] = s;
+        T* out = which == 0 ? dgamma : dbeta;
+        if (out) store1(out + c, s);
     }
 }
 
+template <typename T>
 __global__ __launch_bounds__(kBlock) void ln_bwd_params_final(const float* __restrict__ partial, int64_t cols, int splits,
-                                                              float* __restrict__ dgamma, float* __restrict__ dbeta) {
-    ln_bwd_params_final_body(blockIdx.x, partial, cols, splits, dgamma, dbeta);
+                                                              T* __restrict__ dgamma, T* __restrict__ dbeta) {
+    ln_bwd_params_final_body<T>(blockIdx.x, partial, cols, splits, dgamma, dbeta);
 }
 
 // dx and the final parameter sums in one launch: the first final_blocks
 // workgroups (one per 64-column strip) add up the partial column sums -- a chain
 // of dependent loads, so they start first -- and the rest write dx.  The two
 // parts are independent.
-template <bool VEC>
-__global__ __launch_bounds__(kBlock) void ln_bwd_input_final(const float* __restrict__ dy, const float* __restrict__ x, int64_t rows,
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kBlock) void ln_bwd_input_final(const T* __restrict__ dy, const T* __restrict__ x, int64_t rows,
                                                              int64_t cols, int64_t ld_dy, int64_t ld_x,
                                                              const float* __restrict__ mean, const float* __restrict__ rstd,
-                                                             const float* __restrict__ gamma, const float* __restrict__ part_sums,
-                                                             int nparts, float weight, float* __restrict__ dx, int64_t ld_dx,
+                                                             const T* __restrict__ gamma, const float* __restrict__ part_sums,
+                                                             int nparts, float weight, T* __restrict__ dx, int64_t ld_dx,
                                                              uint32_t final_blocks, const float* __restrict__ partial, int splits,
-                                                             float* __restrict__ dgamma, float* __restrict__ dbeta) {
+                                                             T* __restrict__ dgamma, T* __restrict__ dbeta) {
     if (blockIdx.x < final_blocks)
-        ln_bwd_params_final_body(blockIdx.x, partial, cols, splits, dgamma, dbeta);
+        ln_bwd_params_final_body<T>(blockIdx.x, partial, cols, splits, dgamma, dbeta);
     else
-        ln_bwd_input_body<VEC>(blockIdx.x - final_blocks, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, part_sums, nparts,
+        ln_bwd_input_body<T, VEC>(blockIdx.x - final_blocks, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, part_sums, nparts,
                                weight, dx, ld_dx);
 }
 
@@ -230,11 +233,11 @@ constexpr int kFusedWaves = kFusedBlock / kWave;
 // pass over dy and x: workgroup = split, its wavefronts take every eighth row
 // and each lane keeps the columns (lane + 64 k) * 4 .. + 3, k < NV, in registers.
 // partial has the layout of ln_bwd_params_partial.
-template <int NV>
-__global__ __launch_bounds__(kFusedBlock) void ln_bwd_partial_cols(const float* __restrict__ dy, const float* __restrict__ x, int64_t rows,
+template <typename T, int NV>
+__global__ __launch_bounds__(kFusedBlock) void ln_bwd_partial_cols(const T* __restrict__ dy, const T* __restrict__ x, int64_t rows,
                                                               int64_t cols, int64_t ld_dy, int64_t ld_x,
                                                               const float* __restrict__ mean, const float* __restrict__ rstd,
-                                                              const float* __restrict__ gamma, float* __restrict__ sums,
+                                                              const T* __restrict__ gamma, float* __restrict__ sums,
                                                               int64_t rows_per_split, float* __restrict__ partial) {
     __shared__ float fold[2][kFusedWaves][NV * kWave * 4];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
@@ -246,7 +249,7 @@ __global__ __launch_bounds__(kFusedBlock) void ln_bwd_partial_cols(const float* 
     for (int k = 0; k < NV; ++k) {
         const int c = lane + k * kWave;
         g[k] = make_float4(1.f, 1.f, 1.f, 1.f);
-        if (gamma && c < nv) g[k] = reinterpret_cast<const float4*>(gamma)[c];
+        if (gamma && c < nv) g[k] = load4(gamma + 4 * c);
         ca[k] = cb[k] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
     constexpr int RU = NV <= 2 ? 4 : 2;   // rows whose loads are in flight together
@@ -264,8 +267,8 @@ __global__ __launch_bounds__(kFusedBlock) void ln_bwd_partial_cols(const float* 
                 const int c = lane + k * kWave;
                 d[u][k] = v[u][k] = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (on && c < nv) {
-                    d[u][k] = reinterpret_cast<const float4*>(dy + r * ld_dy)[c];
-                    v[u][k] = reinterpret_cast<const float4*>(x + r * ld_x)[c];
+                    d[u][k] = load4(dy + r * ld_dy + 4 * c);
+                    v[u][k] = load4(x + r * ld_x + 4 * c);
                 }
             }
         }
@@ -306,12 +309,13 @@ __global__ __launch_bounds__(kFusedBlock) void ln_bwd_partial_cols(const float* 
     }
 }
 
-bool vectorizable(int64_t cols, std::initializer_list<int64_t> lds, std::initializer_list<const void*> ptrs) {
+// Can rows be read four elements at a time?  elem = bytes per element.
+bool vectorizable(int elem, int64_t cols, std::initializer_list<int64_t> lds, std::initializer_list<const void*> ptrs) {
     if (cols % 4 != 0) return false;
     for (int64_t ld : lds)
         if (ld % 4 != 0) return false;
     for (const void* p : ptrs)
-        if (p && !aligned_to(p, 16)) return false;
+        if (p && !aligned_to(p, 4 * elem)) return false;
     return true;
 }
 
@@ -321,6 +325,15 @@ int check_rows(const char* what, int64_t rows, int64_t cols, int64_t ld_dy, int6
                     (long long)ld_dy, (long long)ld_x);
     if (rows > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "%s: more than 2^31 rows", what);
     return 0;
+}
+
+int elem_bytes(int dtype) { return dtype == DDL_DT_F32 ? 4 : (dtype == DDL_DT_BF16 || dtype == DDL_DT_F16) ? 2 : 0; }
+
+// Elements aligned to their own size, fp32 side arrays to 4 bytes, pairs to 8.
+bool elems_aligned(int elem, std::initializer_list<const void*> ptrs) {
+    for (const void* p : ptrs)
+        if (p && !aligned_to(p, elem)) return false;
+    return true;
 }
 
 // Row splits of the parameter gradients: as many as the workspace holds, at most
@@ -334,134 +347,198 @@ int64_t param_splits(int64_t rows, int64_t cols, int64_t workspace_elems) {
     return splits;
 }
 
+template <typename T>
+const T* as(const void* p) { return static_cast<const T*>(p); }
+template <typename T>
+T* as(void* p) { return static_cast<T*>(p); }
+
 }  // namespace
 }  // namespace ddl
 
-extern "C" int ddl_ln_bwd_partial_f32(const float* dy, const float* x, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
-                                      const float* mean, const float* rstd, const float* gamma, float* sums, void* stream) {
+extern "C" int ddl_ln_bwd_partial(const void* dy, const void* x, int dtype, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                  const float* mean, const float* rstd, const void* gamma, float* sums, void* stream) {
     using namespace ddl;
+    const int elem = elem_bytes(dtype);
+    if (!elem) return fail(DDL_E_UNSUPP, "ln backward sums: dtype %d (f32, bf16, f16 only)", dtype);
     if (int rc = check_rows("ln backward sums", rows, cols, ld_dy, ld_x)) return rc;
     if (rows == 0) return 0;
     if (!dy || !x || !mean || !rstd || !sums) return fail(DDL_E_ARG, "ln backward sums: null pointer");
-    if (!aligned_to(dy, 4) || !aligned_to(x, 4) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) || !aligned_to(gamma, 4) || !aligned_to(sums, 8))
-        return fail(DDL_E_ALIGN, "ln backward sums: pointers must be 4-byte aligned, the sums 8-byte");
+    if (!elems_aligned(elem, {dy, x, gamma}) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) || !aligned_to(sums, 8))
+        return fail(DDL_E_ALIGN, "ln backward sums: elements must be aligned to their size, mean and rstd to 4 bytes, the sums to 8");
     const uint32_t blocks = static_cast<uint32_t>((rows + kWavesPerBlock - 1) / kWavesPerBlock);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (vectorizable(cols, {ld_dy, ld_x}, {dy, x, gamma}))
-        hipLaunchKernelGGL(ln_bwd_partial<true>, dim3(blocks), dim3(kBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, sums);
-    else
-        hipLaunchKernelGGL(ln_bwd_partial<false>, dim3(blocks), dim3(kBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, sums);
+    const bool vec = vectorizable(elem, cols, {ld_dy, ld_x}, {dy, x, gamma});
+    with_ln_element(dtype, [&](auto* tag) {
+        using T = std::remove_pointer_t<decltype(tag)>;
+        if (vec)
+            hipLaunchKernelGGL((ln_bwd_partial<T, true>), dim3(blocks), dim3(kBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd, as<T>(gamma), sums);
+        else
+            hipLaunchKernelGGL((ln_bwd_partial<T, false>), dim3(blocks), dim3(kBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd, as<T>(gamma), sums);
+    });
     return check_launch("ln_bwd_partial");
 }
 
-extern "C" int ddl_ln_bwd_input_f32(const float* dy, const float* x, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
-                                    const float* mean, const float* rstd, const float* gamma, const float* part_sums,
-                                    int nparts, float weight, float* dx, int64_t ld_dx, void* stream) {
+extern "C" int ddl_ln_bwd_input(const void* dy, const void* x, int dtype, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                const float* mean, const float* rstd, const void* gamma, const float* part_sums, int nparts,
+                                float weight, void* dx, int64_t ld_dx, void* stream) {
     using namespace ddl;
+    const int elem = elem_bytes(dtype);
+    if (!elem) return fail(DDL_E_UNSUPP, "ln backward input: dtype %d (f32, bf16, f16 only)", dtype);
     if (int rc = check_rows("ln backward input", rows, cols, ld_dy, ld_x)) return rc;
     if (ld_dx < cols || nparts < 1) return fail(DDL_E_ARG, "ln backward input: ld_dx=%lld nparts=%d", (long long)ld_dx, nparts);
     if (rows == 0) return 0;
     if (!dy || !x || !mean || !rstd || !part_sums || !dx) return fail(DDL_E_ARG, "ln backward input: null pointer");
-    if (!aligned_to(dy, 4) || !aligned_to(x, 4) || !aligned_to(dx, 4) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) ||
-        !aligned_to(gamma, 4) || !aligned_to(part_sums, 8))
-        return fail(DDL_E_ALIGN, "ln backward input: pointers must be 4-byte aligned, the sums 8-byte");
+    if (!elems_aligned(elem, {dy, x, gamma, dx}) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) || !aligned_to(part_sums, 8))
+        return fail(DDL_E_ALIGN, "ln backward input: elements must be aligned to their size, mean and rstd to 4 bytes, the sums to 8");
     const uint32_t blocks = static_cast<uint32_t>((rows + kWavesPerBlock - 1) / kWavesPerBlock);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (vectorizable(cols, {ld_dy, ld_x, ld_dx}, {dy, x, gamma, dx}))
-        hipLaunchKernelGGL(ln_bwd_input<true>, dim3(blocks), dim3(kBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma,
-                           part_sums, nparts, weight, dx, ld_dx);
-    else
-        hipLaunchKernelGGL(ln_bwd_input<false>, dim3(blocks), dim3(kBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma,
-                           part_sums, nparts, weight, dx, ld_dx);
+    const bool vec = vectorizable(elem, cols, {ld_dy, ld_x, ld_dx}, {dy, x, gamma, dx});
+    with_ln_element(dtype, [&](auto* tag) {
+        using T = std::remove_pointer_t<decltype(tag)>;
+        if (vec)
+            hipLaunchKernelGGL((ln_bwd_input<T, true>), dim3(blocks), dim3(kBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd,
+                               as<T>(gamma), part_sums, nparts, weight, as<T>(dx), ld_dx);
+        else
+            hipLaunchKernelGGL((ln_bwd_input<T, false>), dim3(blocks), dim3(kBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd,
+                               as<T>(gamma), part_sums, nparts, weight, as<T>(dx), ld_dx);
+    });
     return check_launch("ln_bwd_input");
 }
 
-extern "C" int ddl_ln_bwd_params_f32(const float* dy, const float* x, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
-                                     const float* mean, const float* rstd, float* dgamma, float* dbeta, float* workspace,
-                                     int64_t workspace_elems, void* stream) {
+extern "C" int ddl_ln_bwd_params(const void* dy, const void* x, int dtype, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                 const float* mean, const float* rstd, void* dgamma, void* dbeta, float* workspace,
+                                 int64_t workspace_elems, void* stream) {
     using namespace ddl;
+    const int elem = elem_bytes(dtype);
+    if (!elem) return fail(DDL_E_UNSUPP, "ln backward parameters: dtype %d (f32, bf16, f16 only)", dtype);
     if (int rc = check_rows("ln backward parameters", rows, cols, ld_dy, ld_x)) return rc;
     if (!dgamma && !dbeta) return 0;
     if (!workspace || (rows > 0 && (!dy || !x || !mean || !rstd))) return fail(DDL_E_ARG, "ln backward parameters: null pointer");
-    if (!aligned_to(dy, 4) || !aligned_to(x, 4) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) || !aligned_to(dgamma, 4) ||
-        !aligned_to(dbeta, 4) || !aligned_to(workspace, 4))
-        return fail(DDL_E_ALIGN, "ln backward parameters: pointers must be 4-byte aligned");
+    if (!elems_aligned(elem, {dy, x, dgamma, dbeta}) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) || !aligned_to(workspace, 4))
+        return fail(DDL_E_ALIGN, "ln backward parameters: elements must be aligned to their size, fp32 arrays to 4 bytes");
     const int64_t splits = param_splits(rows, cols, workspace_elems);
     if (splits < 1) return fail(DDL_E_ARG, "ln backward parameters: workspace of %lld floats is smaller than 2 x %lld", (long long)workspace_elems, (long long)cols);
     const int64_t rows_per_split = rows > 0 ? (rows + splits - 1) / splits : 1;
     const int64_t strips = (cols + kStrip - 1) / kStrip;
     if (strips * splits > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "ln backward parameters: too many workgroups");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(ln_bwd_params_partial, dim3(static_cast<uint32_t>(strips * splits)), dim3(kBlock), 0, s, dy, x, rows, cols,
-                       ld_dy, ld_x, mean, rstd, rows_per_split, workspace, static_cast<int>(strips));
-    if (int rc = check_launch("ln_bwd_params_partial")) return rc;
-    hipLaunchKernelGGL(ln_bwd_params_final, dim3(static_cast<uint32_t>(strips)), dim3(kBlock), 0, s, workspace, cols,
-                       static_cast<int>(splits), dgamma, dbeta);
-    return check_launch("ln_bwd_params_final");
+    int rc = 0;
+    with_ln_element(dtype, [&](auto* tag) {
+        using T = std::remove_pointer_t<decltype(tag)>;
+        hipLaunchKernelGGL(ln_bwd_params_partial<T>, dim3(static_cast<uint32_t>(strips * splits)), dim3(kBlock), 0, s, as<T>(dy), as<T>(x), rows,
+                           cols, ld_dy, ld_x, mean, rstd, rows_per_split, workspace, static_cast<int>(strips));
+        rc = check_launch("ln_bwd_params_partial");
+        if (rc) return;
+        hipLaunchKernelGGL(ln_bwd_params_final<T>, dim3(static_cast<uint32_t>(strips)), dim3(kBlock), 0, s, workspace, cols,
+                           static_cast<int>(splits), as<T>(dgamma), as<T>(dbeta));
+        rc = check_launch("ln_bwd_params_final");
+    });
+    return rc;
 }
 
-extern "C" int ddl_ln_bwd_partial_params_f32(const float* dy, const float* x, int64_t rows, int64_t cols, int64_t ld_dy,
-                                             int64_t ld_x, const float* mean, const float* rstd, const float* gamma, float* sums,
-                                             float* workspace, int64_t workspace_elems, void* stream) {
+extern "C" int ddl_ln_bwd_partial_params(const void* dy, const void* x, int dtype, int64_t rows, int64_t cols, int64_t ld_dy,
+                                         int64_t ld_x, const float* mean, const float* rstd, const void* gamma, float* sums,
+                                         float* workspace, int64_t workspace_elems, void* stream) {
     using namespace ddl;
+    const int elem = elem_bytes(dtype);
+    if (!elem) return fail(DDL_E_UNSUPP, "ln backward sums: dtype %d (f32, bf16, f16 only)", dtype);
     if (int rc = check_rows("ln backward sums", rows, cols, ld_dy, ld_x)) return rc;
     if (!workspace) return fail(DDL_E_ARG, "ln backward sums: null workspace");
     const int64_t splits = param_splits(rows, cols, workspace_elems);
     if (splits < 1) return fail(DDL_E_ARG, "ln backward sums: workspace of %lld floats is smaller than 2 x %lld", (long long)workspace_elems, (long long)cols);
     if (rows > 0 && (!dy || !x || !mean || !rstd || !sums)) return fail(DDL_E_ARG, "ln backward sums: null pointer");
-    if (!aligned_to(dy, 4) || !aligned_to(x, 4) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) || !aligned_to(gamma, 4) ||
-        !aligned_to(sums, 8) || !aligned_to(workspace, 4))
-        return fail(DDL_E_ALIGN, "ln backward sums: pointers must be 4-byte aligned, the sums 8-byte");
+    if (!elems_aligned(elem, {dy, x, gamma}) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) || !aligned_to(sums, 8) || !aligned_to(workspace, 4))
+        return fail(DDL_E_ALIGN, "ln backward sums: elements must be aligned to their size, fp32 arrays to 4 bytes, the sums to 8");
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t rows_per_split = rows > 0 ? (rows + splits - 1) / splits : 1;
-    if (rows > 0 && cols <= 4 * kWave * 4 && vectorizable(cols, {ld_dy, ld_x}, {dy, x, gamma})) {
+    if (rows > 0 && cols <= 4 * kWave * 4 && vectorizable(elem, cols, {ld_dy, ld_x}, {dy, x, gamma})) {
         const dim3 grid(static_cast<uint32_t>(splits));
-        if (cols <= kWave * 4)
-            hipLaunchKernelGGL(ln_bwd_partial_cols<1>, grid, dim3(kFusedBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, sums, rows_per_split, workspace);
-        else if (cols <= 2 * kWave * 4)
-            hipLaunchKernelGGL(ln_bwd_partial_cols<2>, grid, dim3(kFusedBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, sums, rows_per_split, workspace);
-        else
-            hipLaunchKernelGGL(ln_bwd_partial_cols<4>, grid, dim3(kFusedBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, sums, rows_per_split, workspace);
+        with_ln_element(dtype, [&](auto* tag) {
+            using T = std::remove_pointer_t<decltype(tag)>;
+            if (cols <= kWave * 4)
+                hipLaunchKernelGGL((ln_bwd_partial_cols<T, 1>), grid, dim3(kFusedBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd, as<T>(gamma), sums, rows_per_split, workspace);
+            else if (cols <= 2 * kWave * 4)
+                hipLaunchKernelGGL((ln_bwd_partial_cols<T, 2>), grid, dim3(kFusedBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd, as<T>(gamma), sums, rows_per_split, workspace);
+            else
+                hipLaunchKernelGGL((ln_bwd_partial_cols<T, 4>), grid, dim3(kFusedBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd, as<T>(gamma), sums, rows_per_split, workspace);
+        });
         return check_launch("ln_bwd_partial_cols");
     }
     // long or unaligned rows: the two passes separately, same results in the same places
     if (rows > 0) {
-        if (int rc = ddl_ln_bwd_partial_f32(dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, sums, stream)) return rc;
+        if (int rc = ddl_ln_bwd_partial(dy, x, dtype, rows, cols, ld_dy, ld_x, mean, rstd, gamma, sums, stream)) return rc;
     }
     const int64_t strips = (cols + kStrip - 1) / kStrip;
     if (strips * splits > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "ln backward sums: too many workgroups");
-    hipLaunchKernelGGL(ln_bwd_params_partial, dim3(static_cast<uint32_t>(strips * splits)), dim3(kBlock), 0, s, dy, x, rows, cols,
-                       ld_dy, ld_x, mean, rstd, rows_per_split, workspace, static_cast<int>(strips));
+    with_ln_element(dtype, [&](auto* tag) {
+        using T = std::remove_pointer_t<decltype(tag)>;
+        hipLaunchKernelGGL(ln_bwd_params_partial<T>, dim3(static_cast<uint32_t>(strips * splits)), dim3(kBlock), 0, s, as<T>(dy), as<T>(x), rows,
+                           cols, ld_dy, ld_x, mean, rstd, rows_per_split, workspace, static_cast<int>(strips));
+    });
     return check_launch("ln_bwd_params_partial");
 }
 
-extern "C" int ddl_ln_bwd_input_params_f32(const float* dy, const float* x, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
-                                           const float* mean, const float* rstd, const float* gamma, const float* part_sums,
-                                           int nparts, float weight, float* dx, int64_t ld_dx, const float* workspace,
-                                           int64_t workspace_elems, float* dgamma, float* dbeta, void* stream) {
+extern "C" int ddl_ln_bwd_input_params(const void* dy, const void* x, int dtype, int64_t rows, int64_t cols, int64_t ld_dy,
+                                       int64_t ld_x, const float* mean, const float* rstd, const void* gamma, const float* part_sums,
+                                       int nparts, float weight, void* dx, int64_t ld_dx, const float* workspace,
+                                       int64_t workspace_elems, void* dgamma, void* dbeta, void* stream) {
     using namespace ddl;
+    const int elem = elem_bytes(dtype);
+    if (!elem) return fail(DDL_E_UNSUPP, "ln backward input: dtype %d (f32, bf16, f16 only)", dtype);
     if (int rc = check_rows("ln backward input", rows, cols, ld_dy, ld_x)) return rc;
     if (ld_dx < cols || nparts < 1) return fail(DDL_E_ARG, "ln backward input: ld_dx=%lld nparts=%d", (long long)ld_dx, nparts);
     if (!workspace) return fail(DDL_E_ARG, "ln backward input: null workspace");
     const int64_t splits = param_splits(rows, cols, workspace_elems);
     if (splits < 1) return fail(DDL_E_ARG, "ln backward input: workspace of %lld floats is smaller than 2 x %lld", (long long)workspace_elems, (long long)cols);
     if (rows > 0 && (!dy || !x || !mean || !rstd || !part_sums || !dx)) return fail(DDL_E_ARG, "ln backward input: null pointer");
-    if (!aligned_to(dy, 4) || !aligned_to(x, 4) || !aligned_to(dx, 4) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) ||
-        !aligned_to(gamma, 4) || !aligned_to(part_sums, 8) || !aligned_to(workspace, 4) || !aligned_to(dgamma, 4) || !aligned_to(dbeta, 4))
-        return fail(DDL_E_ALIGN, "ln backward input: pointers must be 4-byte aligned, the sums 8-byte");
+    if (!elems_aligned(elem, {dy, x, gamma, dx, dgamma, dbeta}) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) || !aligned_to(part_sums, 8) ||
+        !aligned_to(workspace, 4))
+        return fail(DDL_E_ALIGN, "ln backward input: elements must be aligned to their size, fp32 arrays to 4 bytes, the sums to 8");
     const int64_t input_blocks = (rows + kWavesPerBlock - 1) / kWavesPerBlock;
     const int64_t strips = (dgamma || dbeta) ? (cols + kStrip - 1) / kStrip : 0;
     if (input_blocks + strips == 0) return 0;
     if (input_blocks + strips > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "ln backward input: too many workgroups");
     hipStream_t s = static_cast<hipStream_t>(stream);
     const dim3 grid(static_cast<uint32_t>(input_blocks + strips));
-    if (vectorizable(cols, {ld_dy, ld_x, ld_dx}, {dy, x, gamma, dx}))
-        hipLaunchKernelGGL(ln_bwd_input_final<true>, grid, dim3(kBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma,
-                           part_sums, nparts, weight, dx, ld_dx, static_cast<uint32_t>(strips), workspace,
-                           static_cast<int>(splits), dgamma, dbeta);
-    else
-        hipLaunchKernelGGL(ln_bwd_input_final<false>, grid, dim3(kBlock), 0, s, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma,
-                           part_sums, nparts, weight, dx, ld_dx, static_cast<uint32_t>(strips), workspace,
-                           static_cast<int>(splits), dgamma, dbeta);
+    const bool vec = vectorizable(elem, cols, {ld_dy, ld_x, ld_dx}, {dy, x, gamma, dx});
+    with_ln_element(dtype, [&](auto* tag) {
+        using T = std::remove_pointer_t<decltype(tag)>;
+        if (vec)
+            hipLaunchKernelGGL((ln_bwd_input_final<T, true>), grid, dim3(kBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd,
+                               as<T>(gamma), part_sums, nparts, weight, as<T>(dx), ld_dx, static_cast<uint32_t>(strips), workspace,
+                               static_cast<int>(splits), as<T>(dgamma), as<T>(dbeta));
+        else
+            hipLaunchKernelGGL((ln_bwd_input_final<T, false>), grid, dim3(kBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd,
+                               as<T>(gamma), part_sums, nparts, weight, as<T>(dx), ld_dx, static_cast<uint32_t>(strips), workspace,
+                               static_cast<int>(splits), as<T>(dgamma), as<T>(dbeta));
+    });
     return check_launch("ln_bwd_input_final");
+}
+
+// The float32 forms.
+extern "C" int ddl_ln_bwd_partial_f32(const float* dy, const float* x, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                      const float* mean, const float* rstd, const float* gamma, float* sums, void* stream) {
+    return ddl_ln_bwd_partial(dy, x, DDL_DT_F32, rows, cols, ld_dy, ld_x, mean, rstd, gamma, sums, stream);
+}
+extern "C" int ddl_ln_bwd_input_f32(const float* dy, const float* x, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                    const float* mean, const float* rstd, const float* gamma, const float* part_sums,
+                                    int nparts, float weight, float* dx, int64_t ld_dx, void* stream) {
+    return ddl_ln_bwd_input(dy, x, DDL_DT_F32, rows, cols, ld_dy, ld_x, mean, rstd, gamma, part_sums, nparts, weight, dx, ld_dx, stream);
+}
+extern "C" int ddl_ln_bwd_params_f32(const float* dy, const float* x, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                     const float* mean, const float* rstd, float* dgamma, float* dbeta, float* workspace,
+                                     int64_t workspace_elems, void* stream) {
+    return ddl_ln_bwd_params(dy, x, DDL_DT_F32, rows, cols, ld_dy, ld_x, mean, rstd, dgamma, dbeta, workspace, workspace_elems, stream);
+}
+extern "C" int ddl_ln_bwd_partial_params_f32(const float* dy, const float* x, int64_t rows, int64_t cols, int64_t ld_dy,
+                                             int64_t ld_x, const float* mean, const float* rstd, const float* gamma, float* sums,
+                                             float* workspace, int64_t workspace_elems, void* stream) {
+    return ddl_ln_bwd_partial_params(dy, x, DDL_DT_F32, rows, cols, ld_dy, ld_x, mean, rstd, gamma, sums, workspace, workspace_elems, stream);
+}
+extern "C" int ddl_ln_bwd_input_params_f32(const float* dy, const float* x, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                           const float* mean, const float* rstd, const float* gamma, const float* part_sums,
+                                           int nparts, float weight, float* dx, int64_t ld_dx, const float* workspace,
+                                           int64_t workspace_elems, float* dgamma, float* dbeta, void* stream) {
+    return ddl_ln_bwd_input_params(dy, x, DDL_DT_F32, rows, cols, ld_dy, ld_x, mean, rstd, gamma, part_sums, nparts, weight, dx, ld_dx,
+                                   workspace, workspace_elems, dgamma, dbeta, stream);
 }

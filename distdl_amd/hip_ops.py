@@ -316,20 +316,30 @@ def layer_norm(x2d, gamma, beta, eps, want_stats=False):
 
 
 def _rows2d(t, name):
-    if t.dtype != torch.float32 or t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
-        raise ValueError(f"{name}: need a 2-D fp32 tensor with unit column stride")
+    if t.dtype not in _LN_DTYPES or t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise ValueError(f"{name}: need a 2-D float32, bfloat16 or float16 tensor with unit column stride")
     return t.stride(0) if t.shape[0] > 1 else t.shape[1]
+
+
+def _ln_bwd_dtype(name, dy2d, x2d, gamma):
+    """The element type of a LayerNorm backward call: dy, x and gamma must share it."""
+    if dy2d.dtype != x2d.dtype or (gamma is not None and gamma.dtype != x2d.dtype):
+        raise ValueError(f"{name}: dy, x and gamma must have one dtype")
+    if dy2d.shape != x2d.shape:
+        raise ValueError(f"{name}: dy {tuple(dy2d.shape)} and x {tuple(x2d.shape)} differ in shape")
+    return _LN_DTYPES[x2d.dtype]
 
 
 def ln_backward_partial(dy2d, x2d, mean, rstd, gamma):
     """Local {sum g, sum g xhat} per row, g = dy gamma: a [rows, 2] fp32 tensor."""
     _require_gpu(dy2d, x2d, mean, rstd, gamma)
     ld_dy, ld_x = _rows2d(dy2d, "ln_backward_partial"), _rows2d(x2d, "ln_backward_partial")
+    dt = _ln_bwd_dtype("ln_backward_partial", dy2d, x2d, gamma)
     rows, cols = x2d.shape
     sums = torch.empty((rows, 2), dtype=torch.float32, device=x2d.device)
-    rc = _lib.load().ddl_ln_bwd_partial_f32(dy2d.data_ptr(), x2d.data_ptr(), rows, cols, ld_dy, ld_x, mean.data_ptr(),
-                                            rstd.data_ptr(), _ptr(gamma), sums.data_ptr(), _stream())
-    _lib.check(rc, "ddl_ln_bwd_partial_f32")
+    rc = _lib.load().ddl_ln_bwd_partial(dy2d.data_ptr(), x2d.data_ptr(), dt, rows, cols, ld_dy, ld_x, mean.data_ptr(),
+                                        rstd.data_ptr(), _ptr(gamma), sums.data_ptr(), _stream())
+    _lib.check(rc, "ddl_ln_bwd_partial")
     return sums
 
 
@@ -341,11 +351,12 @@ def ln_backward_input(dy2d, x2d, mean, rstd, gamma, part_sums, weight):
     if part_sums.dtype != torch.float32 or part_sums.dim() != 3 or tuple(part_sums.shape[1:]) != (rows, 2) or \
        not part_sums.is_contiguous():
         raise ValueError(f"ln_backward_input: part_sums must be contiguous fp32 [P, {rows}, 2]")
-    dx = torch.empty((rows, cols), dtype=torch.float32, device=x2d.device)
-    rc = _lib.load().ddl_ln_bwd_input_f32(dy2d.data_ptr(), x2d.data_ptr(), rows, cols, ld_dy, ld_x, mean.data_ptr(),
-                                          rstd.data_ptr(), _ptr(gamma), part_sums.data_ptr(), part_sums.shape[0],
-                                          float(weight), dx.data_ptr(), cols, _stream())
-    _lib.check(rc, "ddl_ln_bwd_input_f32")
+    dt = _ln_bwd_dtype("ln_backward_input", dy2d, x2d, gamma)
+    dx = torch.empty((rows, cols), dtype=x2d.dtype, device=x2d.device)
+    rc = _lib.load().ddl_ln_bwd_input(dy2d.data_ptr(), x2d.data_ptr(), dt, rows, cols, ld_dy, ld_x, mean.data_ptr(),
+                                      rstd.data_ptr(), _ptr(gamma), part_sums.data_ptr(), part_sums.shape[0],
+                                      float(weight), dx.data_ptr(), cols, _stream())
+    _lib.check(rc, "ddl_ln_bwd_input")
     return dx
 
 
@@ -354,12 +365,13 @@ def ln_backward_params(dy2d, x2d, mean, rstd, want_gamma=True, want_beta=True):
     _require_gpu(dy2d, x2d, mean, rstd)
     ld_dy, ld_x = _rows2d(dy2d, "ln_backward_params"), _rows2d(x2d, "ln_backward_params")
     rows, cols = x2d.shape
-    dg = torch.empty(cols, dtype=torch.float32, device=x2d.device) if want_gamma else None
-    db = torch.empty(cols, dtype=torch.float32, device=x2d.device) if want_beta else None
+    dt = _ln_bwd_dtype("ln_backward_params", dy2d, x2d, None)
+    dg = torch.empty(cols, dtype=x2d.dtype, device=x2d.device) if want_gamma else None
+    db = torch.empty(cols, dtype=x2d.dtype, device=x2d.device) if want_beta else None
     work = _ln_param_workspace(rows, cols, x2d.device)
-    rc = _lib.load().ddl_ln_bwd_params_f32(dy2d.data_ptr(), x2d.data_ptr(), rows, cols, ld_dy, ld_x, mean.data_ptr(),
-                                           rstd.data_ptr(), _ptr(dg), _ptr(db), work.data_ptr(), work.numel(), _stream())
-    _lib.check(rc, "ddl_ln_bwd_params_f32")
+    rc = _lib.load().ddl_ln_bwd_params(dy2d.data_ptr(), x2d.data_ptr(), dt, rows, cols, ld_dy, ld_x, mean.data_ptr(),
+                                       rstd.data_ptr(), _ptr(dg), _ptr(db), work.data_ptr(), work.numel(), _stream())
+    _lib.check(rc, "ddl_ln_bwd_params")
     return dg, db
 
 
@@ -377,10 +389,11 @@ def ln_backward_partial_params(dy2d, x2d, mean, rstd, gamma):
     rows, cols = x2d.shape
     sums = torch.empty((rows, 2), dtype=torch.float32, device=x2d.device)
     work = _ln_param_workspace(rows, cols, x2d.device)
-    rc = _lib.load().ddl_ln_bwd_partial_params_f32(dy2d.data_ptr(), x2d.data_ptr(), rows, cols, ld_dy, ld_x,
-                                                   mean.data_ptr(), rstd.data_ptr(), _ptr(gamma), sums.data_ptr(),
-                                                   work.data_ptr(), work.numel(), _stream())
-    _lib.check(rc, "ddl_ln_bwd_partial_params_f32")
+    dt = _ln_bwd_dtype("ln_backward_partial_params", dy2d, x2d, gamma)
+    rc = _lib.load().ddl_ln_bwd_partial_params(dy2d.data_ptr(), x2d.data_ptr(), dt, rows, cols, ld_dy, ld_x,
+                                               mean.data_ptr(), rstd.data_ptr(), _ptr(gamma), sums.data_ptr(),
+                                               work.data_ptr(), work.numel(), _stream())
+    _lib.check(rc, "ddl_ln_bwd_partial_params")
     return sums, work
 
 
@@ -395,14 +408,15 @@ def ln_backward_input_params(dy2d, x2d, mean, rstd, gamma, part_sums, weight, wo
         raise ValueError(f"ln_backward_input_params: part_sums must be contiguous fp32 [P, {rows}, 2]")
     if work.dtype != torch.float32 or not work.is_contiguous():
         raise ValueError("ln_backward_input_params: the workspace must be a contiguous fp32 tensor")
-    dx = torch.empty((rows, cols), dtype=torch.float32, device=x2d.device)
-    dg = torch.empty(cols, dtype=torch.float32, device=x2d.device) if want_gamma else None
-    db = torch.empty(cols, dtype=torch.float32, device=x2d.device) if want_beta else None
-    rc = _lib.load().ddl_ln_bwd_input_params_f32(dy2d.data_ptr(), x2d.data_ptr(), rows, cols, ld_dy, ld_x, mean.data_ptr(),
-                                                 rstd.data_ptr(), _ptr(gamma), part_sums.data_ptr(), part_sums.shape[0],
-                                                 float(weight), dx.data_ptr(), cols, work.data_ptr(), work.numel(),
-                                                 _ptr(dg), _ptr(db), _stream())
-    _lib.check(rc, "ddl_ln_bwd_input_params_f32")
+    dt = _ln_bwd_dtype("ln_backward_input_params", dy2d, x2d, gamma)
+    dx = torch.empty((rows, cols), dtype=x2d.dtype, device=x2d.device)
+    dg = torch.empty(cols, dtype=x2d.dtype, device=x2d.device) if want_gamma else None
+    db = torch.empty(cols, dtype=x2d.dtype, device=x2d.device) if want_beta else None
+    rc = _lib.load().ddl_ln_bwd_input_params(dy2d.data_ptr(), x2d.data_ptr(), dt, rows, cols, ld_dy, ld_x, mean.data_ptr(),
+                                             rstd.data_ptr(), _ptr(gamma), part_sums.data_ptr(), part_sums.shape[0],
+                                             float(weight), dx.data_ptr(), cols, work.data_ptr(), work.numel(),
+                                             _ptr(dg), _ptr(db), _stream())
+    _lib.check(rc, "ddl_ln_bwd_input_params")
     return dx, dg, db
 
 

@@ -8,8 +8,8 @@ per-row ``{mean, M2}`` pairs; the combination rule reproduces the reference's
 mean of local means and mean of local variances exactly.  When the normalised
 dimensions are not partitioned the reference calls
 ``torch.nn.functional.layer_norm`` (:310-319); here that is one HIP kernel.
-Inputs may be float32, bfloat16 or float16 (sums are float32); the backward
-kernels are float32 only.
+Inputs may be float32, bfloat16 or float16, forward and backward; sums, means
+and reciprocal deviations are float32 and results are rounded once.
 """
 
 import numbers
@@ -70,9 +70,6 @@ class _LayerNormShard(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, weight, bias, P_reduce, part_cols, eps, part_cols_arr=None, stats_buffers=None):
-        if input.dtype != torch.float32:
-            raise NotImplementedError(f"DistributedLayerNorm backward kernels are fp32 only, got {input.dtype}; "
-                                      "run the forward under torch.no_grad() or in float32")
         y, x2d, mean, rstd, gamma = _shard_forward(input, weight, bias, P_reduce, part_cols, eps, part_cols_arr,
                                                    {} if stats_buffers is None else stats_buffers, True)
         ctx.save_for_backward(x2d, mean, rstd, gamma)
@@ -85,6 +82,8 @@ class _LayerNormShard(torch.autograd.Function):
         x2d, mean, rstd, gamma = ctx.saved_tensors
         need_x, need_w, need_b = ctx.needs_input_grad[:3]
         dy2d = grad_output.detach().reshape(-1, ctx.cols)
+        if dy2d.dtype != x2d.dtype:
+            dy2d = dy2d.to(x2d.dtype)
         if dy2d.shape[1] > 1 and dy2d.stride(1) != 1:
             dy2d = dy2d.contiguous()
         dx = dw = db = None

@@ -238,20 +238,40 @@ int ddl_ln_normalize_affine_f32(const float* x, int64_t rows, int64_t cols,
 /* Backward of the LayerNorm shard: what autograd derives from the reference's
  * forward (nn/layernorm.py:230-247, 295-309, all-reduces included).  With
  * g = dy * gamma (gamma NULL = 1), xhat = (x - mean) * rstd (mean, rstd as
- * ddl_ln_normalize_affine_f32 returned them) and a = 1 / (P * columns of this
+ * ddl_ln_normalize_affine returned them) and a = 1 / (P * columns of this
  * worker), P = workers sharing a row:
  *
- *   ddl_ln_bwd_partial_f32   sums[r] = { sum_c g[r,c], sum_c g[r,c] xhat[r,c] }
- *                            over the LOCAL columns; the caller gathers the
- *                            pairs of the P workers into part_sums[P, rows, 2]
- *   ddl_ln_bwd_input_f32     dx[r,c] = rstd[r] * ( g[r,c] - weight * (S1[r] +
- *                            xhat[r,c] * S2[r]) ), S = sum over the P pairs,
- *                            weight = a
- *   ddl_ln_bwd_params_f32    dgamma[c] = sum_r dy[r,c] xhat[r,c],
- *                            dbeta[c]  = sum_r dy[r,c]   (either may be NULL);
- *                            `workspace`: device memory for at least 2 * cols
- *                            floats (up to 512 * cols are used), contents on
- *                            entry do not matter. */
+ *   ddl_ln_bwd_partial   sums[r] = { sum_c g[r,c], sum_c g[r,c] xhat[r,c] }
+ *                        over the LOCAL columns; the caller gathers the
+ *                        pairs of the P workers into part_sums[P, rows, 2]
+ *   ddl_ln_bwd_input     dx[r,c] = rstd[r] * ( g[r,c] - weight * (S1[r] +
+ *                        xhat[r,c] * S2[r]) ), S = sum over the P pairs,
+ *                        weight = a
+ *   ddl_ln_bwd_params    dgamma[c] = sum_r dy[r,c] xhat[r,c],
+ *                        dbeta[c]  = sum_r dy[r,c]   (either may be NULL);
+ *                        `workspace`: device memory for at least 2 * cols
+ *                        floats (up to 512 * cols are used), contents on
+ *                        entry do not matter.
+ *
+ * dy, x, gamma, dx, dgamma and dbeta are of `dtype` (DDL_DT_F32, DDL_DT_BF16 or
+ * DDL_DT_F16: autograd hands gradients over in the type of the tensors); mean,
+ * rstd, the sums and the workspace are fp32, as is all arithmetic, and results
+ * are rounded once when stored.  The _f32 forms are the same calls with
+ * dtype = DDL_DT_F32. */
+int ddl_ln_bwd_partial(const void* dy, const void* x, int dtype, int64_t rows,
+                       int64_t cols, int64_t ld_dy, int64_t ld_x,
+                       const float* mean, const float* rstd,
+                       const void* gamma, float* sums, void* stream);
+int ddl_ln_bwd_input(const void* dy, const void* x, int dtype, int64_t rows,
+                     int64_t cols, int64_t ld_dy, int64_t ld_x,
+                     const float* mean, const float* rstd,
+                     const void* gamma, const float* part_sums, int nparts,
+                     float weight, void* dx, int64_t ld_dx, void* stream);
+int ddl_ln_bwd_params(const void* dy, const void* x, int dtype, int64_t rows,
+                      int64_t cols, int64_t ld_dy, int64_t ld_x,
+                      const float* mean, const float* rstd, void* dgamma,
+                      void* dbeta, float* workspace,
+                      int64_t workspace_elems, void* stream);
 int ddl_ln_bwd_partial_f32(const float* dy, const float* x, int64_t rows,
                            int64_t cols, int64_t ld_dy, int64_t ld_x,
                            const float* mean, const float* rstd,
@@ -268,19 +288,32 @@ int ddl_ln_bwd_params_f32(const float* dy, const float* x, int64_t rows,
                           int64_t workspace_elems, void* stream);
 
 /* The same three results in two launches instead of four, for a caller that
- * wants dx and the parameter gradients (rows of a few hundred floats are
+ * wants dx and the parameter gradients (rows of a few hundred elements are
  * launch-bound, so this halves the time):
  *
- *   ddl_ln_bwd_partial_params_f32   sums[] as ddl_ln_bwd_partial_f32, and in the
- *                                   same pass over dy and x the row-split
- *                                   partial column sums, left in `workspace`
- *   ddl_ln_bwd_input_params_f32     dx as ddl_ln_bwd_input_f32, and in the same
- *                                   launch dgamma / dbeta (either may be NULL)
- *                                   from the partial sums in `workspace`
+ *   ddl_ln_bwd_partial_params   sums[] as ddl_ln_bwd_partial, and in the
+ *                               same pass over dy and x the row-split
+ *                               partial column sums, left in `workspace`
+ *   ddl_ln_bwd_input_params     dx as ddl_ln_bwd_input, and in the same
+ *                               launch dgamma / dbeta (either may be NULL)
+ *                               from the partial sums in `workspace`
  *
  * Both calls take the same rows, cols, workspace and workspace_elems (at least
  * 2 * cols floats, up to 512 * cols are used); the second must follow the first
- * on the same stream. */
+ * on the same stream.  Element types as above; _f32 forms likewise. */
+int ddl_ln_bwd_partial_params(const void* dy, const void* x, int dtype,
+                              int64_t rows, int64_t cols, int64_t ld_dy,
+                              int64_t ld_x, const float* mean,
+                              const float* rstd, const void* gamma,
+                              float* sums, float* workspace,
+                              int64_t workspace_elems, void* stream);
+int ddl_ln_bwd_input_params(const void* dy, const void* x, int dtype,
+                            int64_t rows, int64_t cols, int64_t ld_dy,
+                            int64_t ld_x, const float* mean, const float* rstd,
+                            const void* gamma, const float* part_sums,
+                            int nparts, float weight, void* dx, int64_t ld_dx,
+                            const float* workspace, int64_t workspace_elems,
+                            void* dgamma, void* dbeta, void* stream);
 int ddl_ln_bwd_partial_params_f32(const float* dy, const float* x, int64_t rows,
                                   int64_t cols, int64_t ld_dy, int64_t ld_x,
                                   const float* mean, const float* rstd,

@@ -171,7 +171,7 @@ def test_layernorm_16_bit_elements(ops, dtype, cols):
 
 def test_layernorm_layer_single_worker_and_bf16(ops):
     """The layer on one worker takes the single-launch kernel (the reference's
-    F.layer_norm branch) and is differentiable in fp32; in bf16 it runs forward."""
+    F.layer_norm branch) and is differentiable; a bf16 forward beside it."""
     from distdl_amd.backends.stub_hip import SimWorld
     from distdl_amd.nn import DistributedLayerNorm
     torch.manual_seed(3)
@@ -337,6 +337,103 @@ def test_layernorm_backward_kernels_match_oracle(ops, cols, affine):
         dx3, dg3, db3 = ops.ln_backward_input_params(dy2d, x2d, mean, rstd, g, torch.stack(gathered).contiguous(),
                                                      1.0 / (P * cols[live]), work, want_gamma=False, want_beta=True)
         assert dg3 is None and torch.equal(db3, db2) and torch.equal(dx3, dx2)
+
+
+@pytest.mark.parametrize("dtype,ulp", [(torch.bfloat16, 2.0 ** -8), (torch.float16, 2.0 ** -11)])
+@pytest.mark.parametrize("cols", [[256, 256], [300, 212], [7, 9], [2048], [1030]])
+def test_layernorm_backward_16_bit_elements(ops, dtype, ulp, cols):
+    """The backward kernels on bf16 / fp16 tensors: arithmetic in fp32 on the
+    16-bit values, one rounding when dx, dgamma and dbeta are stored -- so the
+    results must be the fp64 closed form of the same 16-bit inputs to within one
+    rounding of the result type (plus fp32 summation noise)."""
+    rng = np.random.default_rng(sum(cols) + 5)
+    rows, eps = 45, 1e-5
+    def q(a):   # through the 16-bit type and back
+        return torch.from_numpy(a.astype(np.float32)).to(dtype)
+    shards = [q(rng.standard_normal((rows, c)) * 2 + 0.5) for c in cols]
+    dys = [q(rng.standard_normal((rows, c))) for c in cols]
+    gammas = [q(1 + 0.1 * rng.standard_normal(c)) for c in cols]
+    f64 = lambda t: t.double().numpy()
+    want_dx, want_dg, want_db = o_ln.backward_shards([f64(t) for t in shards], [f64(t) for t in gammas], [f64(t) for t in dys], eps)
+    P = len(cols)
+    m64 = sum(f64(s).mean(axis=1) for s in shards) / P
+    v64 = sum(((f64(s) - m64[:, None]) ** 2).mean(axis=1) for s in shards) / P
+    r64 = 1.0 / np.sqrt(v64 + eps)
+    live = P - 1
+    x2d, dy2d, g = shards[live].cuda(), dys[live].cuda(), gammas[live].cuda()
+    parts = [torch.from_numpy(o_ln.partial_stats(f64(s)).astype(np.float32)).cuda() for s in shards]
+    parts[live] = ops.ln_partial_stats(x2d)
+    _, mean, rstd = ops.ln_normalize_affine(x2d, torch.stack(parts).contiguous(), cols, g, g, eps, want_stats=True)
+    assert mean.dtype == torch.float32 and rstd.dtype == torch.float32
+    gathered = []
+    for p in range(P):
+        gp = f64(dys[p]) * f64(gammas[p])
+        xh = (f64(shards[p]) - m64[:, None]) * r64[:, None]
+        gathered.append(torch.from_numpy(np.stack([gp.sum(axis=1), (gp * xh).sum(axis=1)], axis=1).astype(np.float32)).cuda())
+    sums = ops.ln_backward_partial(dy2d, x2d, mean, rstd, g)
+    scale = np.abs(f64(dys[live]) * f64(gammas[live])).sum(axis=1).max()
+    assert np.allclose(sums.cpu().numpy(), gathered[live].cpu().numpy(), rtol=1e-4, atol=2e-5 * scale)
+    gathered[live] = sums
+    stack = torch.stack(gathered).contiguous()
+    weight = 1.0 / (P * cols[live])
+    dx = ops.ln_backward_input(dy2d, x2d, mean, rstd, g, stack, weight)
+    dg, db = ops.ln_backward_params(dy2d, x2d, mean, rstd)
+    sums2, work = ops.ln_backward_partial_params(dy2d, x2d, mean, rstd, g)
+    gathered[live] = sums2
+    dx2, dg2, db2 = ops.ln_backward_input_params(dy2d, x2d, mean, rstd, g, torch.stack(gathered).contiguous(), weight, work)
+    torch.cuda.synchronize()
+    for got_dx, got_dg, got_db in ((dx, dg, db), (dx2, dg2, db2)):
+        assert got_dx.dtype == dtype and got_dg.dtype == dtype and got_db.dtype == dtype
+        for got, want in ((got_dx, want_dx[live]), (got_dg, want_dg[live]), (got_db, want_db[live])):
+            err = np.abs(got.double().cpu().numpy() - want)
+            assert (err <= ulp * np.abs(want) + 1e-4 * max(1.0, np.abs(want).max())).all(), float(err.max())
+    # misaligned rows (odd pitch) take the element-wise kernels: same values
+    pitch = cols[live] + 3
+    xp = torch.zeros((rows, pitch), dtype=dtype, device="cuda")
+    dyp = torch.zeros((rows, pitch), dtype=dtype, device="cuda")
+    xp[:, :cols[live]] = x2d
+    dyp[:, :cols[live]] = dy2d
+    dx3 = ops.ln_backward_input(dyp[:, :cols[live]], xp[:, :cols[live]], mean, rstd, g, stack, weight)
+    err = np.abs(dx3.double().cpu().numpy() - want_dx[live])
+    assert (err <= ulp * np.abs(want_dx[live]) + 1e-4 * max(1.0, np.abs(want_dx[live]).max())).all()
+
+
+def test_layernorm_layer_backward_in_bfloat16():
+    """The layer in bfloat16 on two workers that share the rows, forward and
+    backward through autograd, against torch's layer norm in float64 on the
+    same bfloat16 values."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedLayerNorm
+    torch.manual_seed(11)
+    P, shape, norm = [1, 1, 2], [4, 6, 128], [128]
+    x = torch.randn(shape).to(torch.bfloat16)
+    dy = torch.randn(shape).to(torch.bfloat16)
+    gamma = (1 + 0.1 * torch.randn(norm)).to(torch.bfloat16)
+    beta = (0.1 * torch.randn(norm)).to(torch.bfloat16)
+
+    def body(P_world):
+        P_x = P_world.create_partition_inclusive([0, 1]).create_cartesian_topology_partition(P)
+        layer = DistributedLayerNorm(P_x, norm, dtype=torch.bfloat16)
+        half = slice(64 * P_x.rank, 64 * P_x.rank + 64)
+        with torch.no_grad():
+            layer.weight.copy_(gamma[half].reshape(1, 1, 64))
+            layer.bias.copy_(beta[half].reshape(1, 1, 64))
+        xin = x[..., half].contiguous().cuda().requires_grad_(True)
+        y = layer(xin)
+        y.backward(dy[..., half].contiguous().cuda())
+        torch.cuda.synchronize()
+        assert y.dtype == torch.bfloat16 and xin.grad.dtype == torch.bfloat16 and layer.weight.grad.dtype == torch.bfloat16
+        return y.detach().cpu(), xin.grad.cpu(), layer.weight.grad.cpu().reshape(-1), layer.bias.grad.cpu().reshape(-1)
+
+    outs = SimWorld(2).run(body)
+    xr, gr, br = x.double().requires_grad_(True), gamma.double().requires_grad_(True), beta.double().requires_grad_(True)
+    yr = F.layer_norm(xr, tuple(norm), gr, br, 1e-5)
+    yr.backward(dy.double())
+    for rank, (y, dx, dw, db) in enumerate(outs):
+        half = slice(64 * rank, 64 * rank + 64)
+        for got, want in ((y, yr.detach()[..., half]), (dx, xr.grad[..., half]), (dw, gr.grad[half]), (db, br.grad[half])):
+            err = (got.double() - want).abs()
+            assert (err <= 2.0 ** -8 * want.abs() + 1e-3 * max(1.0, float(want.abs().max()))).all(), float(err.max())
 
 
 def test_layernorm_backward_two_launch_variant_many_rows(ops):
