@@ -45,13 +45,17 @@
 //              one per CU and a last round that is only partly filled costs as
 //              much as a full one; when it pays, the columns are split between
 //              256-wide tiles (whole rounds) and 192-wide tiles (4 x 2
-//              wavefronts of 64 x 96), whose rounds are shorter, in a launch of
-//              their own.  (Both kinds in one grid, so that a CU starts on a
-//              narrow tile the moment its wide one is stored, measured 2 %
-//              slower: the workgroups of an XCD then drift apart in k and share
-//              fewer operand lines in its L2.)  Workgroup ids are regrouped so
-//              that the 32 workgroups resident on one XCD cover a compact patch
-//              of the tile grid and share their operand panels in that XCD's L2
+//              wavefronts of 64 x 96), whose rounds are shorter.  One launch:
+//              workgroup b computes wide tile b and then narrow tile b, so the
+//              stores of its first tile drain while it computes the second and
+//              the workgroups of an XCD stay in step.  (Both kinds as separate
+//              workgroups of one grid, so that a CU starts on a narrow tile the
+//              moment its wide one is stored, measured 2 % slower: the
+//              workgroups of an XCD then drift apart in k and share fewer
+//              operand lines in its L2; two launches measured 1 % slower.)
+//              Workgroup ids are regrouped so that the 32 workgroups resident on
+//              one XCD cover a compact patch of the tile grid and share their
+//              operand panels in that XCD's L2
 #include "ddl_common.h"
 #include <hip/hip_fp16.h>
 #include <atomic>
@@ -534,33 +538,38 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
 
 constexpr int kThreads = 512;
 
-// 256 x 256 tiles: 2 x 4 wavefronts of 128 x 64.
+// The two kinds of tiles of one product.
+struct Parts {
+    Part wide;     // 256 x 256 tiles: 2 x 4 wavefronts of 128 x 64
+    Part narrow;   // 256 x 192 tiles: 4 x 2 wavefronts of 64 x 96
+};
+
+// Workgroup b computes wide tile b and then narrow tile b (where they exist):
+// the stores of the first tile drain while the second is computed, and there
+// is no kernel boundary between the two rounds.
 template <bool F16, bool XT, bool WT>
-__global__ __launch_bounds__(kThreads) void gemm16_wide(const Part part) {
+__global__ __launch_bounds__(kThreads) void gemm16_tiles(const Parts parts) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
-    gemm_tile<F16, XT, WT, 2, 4, 8, 4>(part, blockIdx.x, lds);
+    const int b = static_cast<int>(blockIdx.x);
+    const bool has_wide = b < parts.wide.tiles_m * parts.wide.tiles_n;
+    if (has_wide) gemm_tile<F16, XT, WT, 2, 4, 8, 4>(parts.wide, b, lds);
+    if (b < parts.narrow.tiles_m * parts.narrow.tiles_n) {
+        if (has_wide) __syncthreads();   // every wavefront has read its part of the first tile out of LDS
+        gemm_tile<F16, XT, WT, 4, 2, 4, 6>(parts.narrow, b, lds);
+    }
 }
 
-// 256 x 192 tiles: 4 x 2 wavefronts of 64 x 96.
-template <bool F16, bool XT, bool WT>
-__global__ __launch_bounds__(kThreads) void gemm16_narrow(const Part part) {
-    extern __shared__ __attribute__((aligned(16))) char lds[];
-    gemm_tile<F16, XT, WT, 4, 2, 4, 6>(part, blockIdx.x, lds);
-}
-
-typedef void (*Kernel)(const Part);
-// index: 8 fp16 + 4 (x transposed) + 2 (w transposed) + narrow
-const Kernel kKernels[16] = {
-    gemm16_wide<false, false, false>, gemm16_narrow<false, false, false>, gemm16_wide<false, false, true>, gemm16_narrow<false, false, true>,
-    gemm16_wide<false, true, false>,  gemm16_narrow<false, true, false>,  gemm16_wide<false, true, true>,  gemm16_narrow<false, true, true>,
-    gemm16_wide<true, false, false>,  gemm16_narrow<true, false, false>,  gemm16_wide<true, false, true>,  gemm16_narrow<true, false, true>,
-    gemm16_wide<true, true, false>,   gemm16_narrow<true, true, false>,   gemm16_wide<true, true, true>,   gemm16_narrow<true, true, true>,
+typedef void (*Kernel)(const Parts);
+// index: 4 fp16 + 2 (x transposed) + (w transposed)
+const Kernel kKernels[8] = {
+    gemm16_tiles<false, false, false>, gemm16_tiles<false, false, true>, gemm16_tiles<false, true, false>, gemm16_tiles<false, true, true>,
+    gemm16_tiles<true, false, false>,  gemm16_tiles<true, false, true>,  gemm16_tiles<true, true, false>,  gemm16_tiles<true, true, true>,
 };
 
 // Per-device state, set on first use by whichever thread gets there (the
 // values are the same for all of them).
 constexpr int kMaxDevices = 64;
-std::atomic<bool> lds_reserved[kMaxDevices][16];  // the dynamic LDS size of kKernels[i] has been raised
+std::atomic<bool> lds_reserved[kMaxDevices][8];   // the dynamic LDS size of kKernels[i] has been raised
 std::atomic<int> cu_count[kMaxDevices];           // 0: not asked yet
 
 // One operand of the product: element (row, k) at p[row * row_stride + k * k_stride],
@@ -616,18 +625,6 @@ int gemm16(const char* who, bool f16, Operand a, Operand b, const uint16_t* bias
         cus = n;
         cu_count[dev].store(n, std::memory_order_relaxed);
     }
-    auto launch = [&](int narrow, const Part& p) -> int {
-        const int k = (f16 ? 8 : 0) + (at ? 4 : 0) + (bt ? 2 : 0) + narrow;
-        if (!lds_reserved[dev][k].load(std::memory_order_acquire)) {   // the attribute sticks to the function on this device
-            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kKernels[k]), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-            if (e != hipSuccess) return fail(static_cast<int>(e), "%s: cannot reserve %d bytes of LDS: %s", who, kLdsBytes, hipGetErrorString(e));
-            lds_reserved[dev][k].store(true, std::memory_order_release);
-        }
-        const dim3 grid(static_cast<uint32_t>(static_cast<int64_t>(p.tiles_m) * p.tiles_n));
-        hipLaunchKernelGGL(kKernels[k], grid, dim3(kThreads), kLdsBytes, static_cast<hipStream_t>(stream), p);
-        return check_launch(narrow ? "gemm16_narrow" : "gemm16_wide");
-    };
-
     // How many 256-column strips go to the wide tiles: whole rounds of them,
     // the rest of the columns to 192-wide tiles, if that shortens the last round.
     const int64_t tiles_m = (M + 255) / 256, cols = (N + 255) / 256;
@@ -652,12 +649,19 @@ int gemm16(const char* who, bool f16, Operand a, Operand b, const uint16_t* bias
     if (tiles_m > 0x7FFFFFll || cols > 0x7FFFFFll || tiles_m * (cols + 1) > 0x7FFFFFFFll)
         return fail(DDL_E_UNSUPP, "%s: too many output tiles", who);
     const int64_t wide_cols = best_split == cols ? N : best_split * 256;
-    if (wide_cols > 0) {
-        const int rc = launch(0, part(256, 0, wide_cols));
-        if (rc) return rc;
+    Parts parts{};
+    if (wide_cols > 0) parts.wide = part(256, 0, wide_cols);
+    if (wide_cols < N) parts.narrow = part(192, wide_cols, N - wide_cols);
+    const int n_wide = parts.wide.tiles_m * parts.wide.tiles_n, n_narrow = parts.narrow.tiles_m * parts.narrow.tiles_n;
+    const int k = (f16 ? 4 : 0) + (at ? 2 : 0) + (bt ? 1 : 0);
+    if (!lds_reserved[dev][k].load(std::memory_order_acquire)) {   // the attribute sticks to the function on this device
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kKernels[k]), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+        if (e != hipSuccess) return fail(static_cast<int>(e), "%s: cannot reserve %d bytes of LDS: %s", who, kLdsBytes, hipGetErrorString(e));
+        lds_reserved[dev][k].store(true, std::memory_order_release);
     }
-    if (wide_cols < N) return launch(1, part(192, wide_cols, N - wide_cols));
-    return 0;
+    hipLaunchKernelGGL(kKernels[k], dim3(static_cast<uint32_t>(n_wide > n_narrow ? n_wide : n_narrow)), dim3(kThreads), kLdsBytes,
+                       static_cast<hipStream_t>(stream), parts);
+    return check_launch("gemm16_tiles");
 }
 
 }  // namespace
