@@ -44,6 +44,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+MFMA_F32_PEAK_TFLOPS = 157.3    # MI355X dense fp32 matrix, published
 MIN_SECONDARY_STEPS, MIN_SECONDARY_WARMUP = 100, 20
 
 
@@ -495,6 +496,55 @@ def build_linear(torch, lib, _lib, nsets):
     return steps, keep, 2 * 8192 * 3584 * 8192
 
 
+def _build_linear_f32(library):
+    def build(torch, lib, _lib, nsets):
+        M, N, K = 8192, 3584, 8192
+        gen = torch.Generator(device="cuda").manual_seed(7004)
+        w = 0.02 * torch.randn(N, K, generator=gen, device="cuda")
+        b = 0.02 * torch.randn(N, generator=gen, device="cuda")
+        keep, steps = [w, b], []
+        for s in range(nsets):
+            x = torch.randn(M, K, generator=gen, device="cuda")
+            if library:
+                keep.append(x)
+
+                def gemm(x=x):
+                    torch.nn.functional.linear(x, w, b)
+                steps.append([gemm])
+            else:
+                y = torch.empty(M, N, device="cuda")
+                keep.append((x, y))
+                steps.append([_call(lib, _lib, "ddl_linear", (x.data_ptr(), w.data_ptr(), b.data_ptr(), y.data_ptr(), _lib.DDL_DT_F32,
+                                                              M, N, K, K, K, N))])
+        return steps, keep, 2 * M * N * K
+    build.__doc__ = ("Config 4's shape in float32, the default dtype of the reference's layers: M=8192 N=3584 K=8192, bias, "
+                     + ("through torch.nn.functional.linear (the vendor GEMM library), for comparison." if library else
+                        "through ddl_linear (fp32 MFMA kernel)."))
+    return build
+
+
+def build_linear_f32_bwd(torch, lib, _lib, nsets):
+    """Backward of the float32 shard of config 4's shape: dx = dy w and dw = dy^T x through ddl_gemm_f32 on the
+    operands where they lie, db = column sums of dy.  Work: 2 x 2 M N K flop."""
+    M, N, K = 8192, 3584, 8192
+    gen = torch.Generator(device="cuda").manual_seed(7005)
+    w = 0.02 * torch.randn(N, K, generator=gen, device="cuda")
+    work = torch.empty(64 * N, device="cuda")
+    keep, steps = [w, work], []
+    f32 = _lib.DDL_DT_F32
+    for s in range(nsets):
+        x = torch.randn(M, K, generator=gen, device="cuda")
+        dy = torch.randn(M, N, generator=gen, device="cuda")
+        dx, dw, db = torch.empty(M, K, device="cuda"), torch.empty(N, K, device="cuda"), torch.empty(N, device="cuda")
+        keep.append((x, dy, dx, dw, db))
+        steps.append([
+            _call(lib, _lib, "ddl_gemm_f32", (dy.data_ptr(), N, 1, w.data_ptr(), 1, K, None, dx.data_ptr(), K, M, K, N)),
+            _call(lib, _lib, "ddl_gemm_f32", (dy.data_ptr(), 1, N, x.data_ptr(), 1, K, None, dw.data_ptr(), K, N, K, M)),
+            _call(lib, _lib, "ddl_colsum", (dy.data_ptr(), f32, M, N, N, db.data_ptr(), work.data_ptr(), work.numel())),
+        ])
+    return steps, keep, 2 * 2 * M * N * K
+
+
 def build_linear_library(torch, lib, _lib, nsets):
     """The same product on the same operands through torch.nn.functional.linear
     (the vendor GEMM library): the comparison figure for the hand-written
@@ -860,6 +910,8 @@ WORKLOADS = {
     "layernorm_bwd": (build_layernorm_bwd, 32, 2, "hbm", None, None, None, None),
     "embedding_bwd": (build_embedding_bwd, 4, 1, "hbm", None, None, None, None),
     "linear_bwd": (_build_linear_bwd(True), 2, 1, "mfma", None, None, None, None),
+    "linear_f32": (_build_linear_f32(False), 2, 1, "mfma_f32", None, None, None, None),
+    "linear_f32_bwd": (build_linear_f32_bwd, 2, 1, "mfma_f32", None, None, None, None),
     "launch_floor": (build_launch_floor, 8, 2, "hbm", None, None, None, None),
     "mfma_32x32x16_constant": (_build_mfma_probe(0, 0), 1, 1, "mfma", None, None, None, None),
     "mfma_32x32x16_random": (_build_mfma_probe(0, 1), 1, 1, "mfma", None, None, None, None),
@@ -868,9 +920,10 @@ WORKLOADS = {
     # only with --only:
     "linear_library": (build_linear_library, 4, 1, "mfma", None, None, None, None),
     "linear_bwd_transposed": (_build_linear_bwd(False), 2, 1, "mfma", None, None, None, None),
+    "linear_f32_library": (_build_linear_f32(True), 2, 1, "mfma_f32", None, None, None, None),
     "calib": (build_calib, 4, 1, "hbm", None, None, None, None),
 }
-ONLY_ON_REQUEST = ("linear_library", "linear_bwd_transposed", "calib")
+ONLY_ON_REQUEST = ("linear_library", "linear_bwd_transposed", "linear_f32_library", "calib")
 
 
 def cpu_host():
@@ -924,7 +977,8 @@ def main():
             achieved, peak, unit = per_launch / m["launch_s"] / 1e9, HBM_PEAK_GBS, "GB/s"
             value = work * m["steps"] / m["wall_s"] / 1e9
         else:
-            achieved, peak, unit = per_launch / m["launch_s"] / 1e12, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
+            peak = MFMA_F32_PEAK_TFLOPS if bound == "mfma_f32" else MFMA_BF16_PEAK_TFLOPS
+            achieved, unit, bound = per_launch / m["launch_s"] / 1e12, "TFLOP/s", "mfma"
             value = work * m["steps"] / m["wall_s"] / 1e12
         traffic = profile_traffic(name, combine) if combine else None
         results[name] = {

@@ -20,11 +20,16 @@
 //              registers (the next tile's, while the current one is multiplied)
 //              and stores them to the other stage
 //
-// This is the compatibility path for fp32 layers, not the tuned one: the bf16 /
-// fp16 kernel is the one sized against the matrix-core roofline.
+// This kernel takes any strides, alignment and size; products large enough to
+// fill the chip with 256 x 256 tiles whose operands have a unit stride and
+// 16-byte alignment go to the tiled kernel of linear_f32_tiles.hip instead.
 #include "ddl_common.h"
 
 namespace ddl {
+
+bool gemm_f32_tiled(const float* a, int64_t a_rs, int64_t a_ks, const float* b, int64_t b_rs, int64_t b_ks, const float* bias, float* y,
+                    int64_t ldy, int64_t M, int64_t N, int64_t K, void* stream, int* rc);
+
 namespace {
 
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
@@ -94,7 +99,23 @@ __global__ __launch_bounds__(kThreads) void gemm_f32_kernel(const Operand a, con
                                                             float* __restrict__ y, int64_t ldy, int64_t K, int tiles_m,
                                                             int a_vec, int b_vec) {
     __shared__ float lds[2][2][kTileFloats];   // [stage][a / b]
-    const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
+    // XCD-aware tile assignment: hardware deals workgroup ids round-robin over
+    // the 8 XCDs, so id % 8 names the XCD.  Each XCD gets a contiguous range of
+    // the tile sequence, which is walked in bands of 8 m-tiles, so that the
+    // workgroups resident on an XCD share operand panels in its L2.
+    const int ntiles = gridDim.x;
+    const int tiles_n = ntiles / tiles_m;
+    int id = blockIdx.x;
+    {
+        const int per = ntiles / 8, main = per * 8;
+        if (id < main) id = (id % 8) * per + id / 8;
+    }
+    constexpr int kBand = 8;
+    const int band = id / (kBand * tiles_n);
+    const int band_m0 = band * kBand;
+    const int band_h = (tiles_m - band_m0) < kBand ? (tiles_m - band_m0) : kBand;
+    const int in_band = id - band * kBand * tiles_n;
+    const int tm = band_m0 + in_band % band_h, tn = in_band / band_h;
     const int64_t m0 = static_cast<int64_t>(tm) * BM, n0 = static_cast<int64_t>(tn) * BN;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;
@@ -189,6 +210,11 @@ extern "C" int ddl_gemm_f32(const float* a, int64_t a_row_stride, int64_t a_k_st
     if (K == 0) return fail(DDL_E_UNSUPP, "gemm f32: K = 0");
     if (a_row_stride < 0 || a_k_stride < 0 || b_row_stride < 0 || b_k_stride < 0) return fail(DDL_E_ARG, "gemm f32: negative stride");
     if (!aligned_to(a, 4) || !aligned_to(b, 4) || !aligned_to(y, 4) || !aligned_to(bias, 4)) return fail(DDL_E_ALIGN, "gemm f32: pointer misaligned");
+    // At least a quarter of the CUs' worth of 256 x 256 tiles: below that, the 128 x 128 tiles here spread the work further.
+    if (((M + 255) / 256) * ((N + 255) / 256) >= 64) {
+        int rc = 0;
+        if (gemm_f32_tiled(a, a_row_stride, a_k_stride, b, b_row_stride, b_k_stride, bias, y, ldy, M, N, K, stream, &rc)) return rc;
+    }
     const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     if (tiles_m * tiles_n > 0x7FFFFFFFll || tiles_m > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "gemm f32: too many output tiles");
     const Operand oa{a, a_row_stride, a_k_stride, M}, ob{b, b_row_stride, b_k_stride, N};

@@ -56,9 +56,8 @@
 //              Workgroup ids are regrouped so that the 32 workgroups resident on
 //              one XCD cover a compact patch of the tile grid and share their
 //              operand panels in that XCD's L2
-#include "ddl_common.h"
+#include "gemm_tiles.h"
 #include <hip/hip_fp16.h>
-#include <atomic>
 #include <type_traits>
 
 namespace ddl {
@@ -67,12 +66,7 @@ namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
-constexpr int BK = 64;
-constexpr int kMaxTileRows = 256;                    // rows of an operand tile: 256 of x; 256 or 192 of w
-constexpr int kUnitBytes = kMaxTileRows * BK * 2;    // ring slot for one operand tile (rows x 128 B), 32 KiB
-constexpr int kUnits = 5;                            // ring of operand tiles: W0 X0 W1 X1 W2 | X2 W3 ...
-constexpr int kLdsBytes = kUnits * kUnitBytes;       // 160 KiB: all of a CU's LDS
-constexpr int kXcds = 8;
+constexpr int BK = kRowBytes / 2;   // 16-bit elements of a k-tile
 
 __device__ inline uint16_t f32_to_bf16_bits(float f) {
     uint32_t u = __float_as_uint(f);
@@ -82,32 +76,6 @@ __device__ inline uint16_t f32_to_bf16_bits(float f) {
 }
 
 __device__ inline float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(static_cast<uint32_t>(b) << 16); }
-
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
-// Raw buffer descriptor over all of memory from `base` on (no stride, no bounds).
-__device__ inline u32x4 raw_buffer(const void* base) {
-    const uint64_t a = reinterpret_cast<uint64_t>(base);
-    u32x4 r;
-    r[0] = static_cast<uint32_t>(a), r[1] = static_cast<uint32_t>(a >> 32) & 0xFFFFu, r[2] = 0xFFFFFFFFu, r[3] = 0x00020000u;
-    return r;
-}
-
-// One wavefront instruction: lane l copies the 16 bytes at byte (voffset +
-// soffset) of the buffer to LDS byte (dst + 16 l); dst and soffset are the same
-// for all lanes.  Written as assembly: the compiler makes every later LDS read
-// through a transposing read wait for all such copies in flight (it cannot
-// tell that they go to another ring slot), which would serialise the pipeline.
-// The kernel waits for these copies itself (s_waitcnt vmcnt in front of the
-// barriers); the compiler does not count them, which only makes its own waits
-// for ordinary loads longer, never shorter (requests complete in order).
-__device__ inline void dma16(u32x4 buffer, int voffset, int soffset, const char* dst) {
-    const uint32_t lds_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst));   // low half of a generic LDS address: the LDS offset
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :
-                 : "s"(lds_addr), "v"(voffset), "s"(buffer), "s"(soffset)
-                 : "memory", "m0");
-}
 
 // acc += a . b (16 x 16 x 32, bf16 in, fp32 accumulate).  Written as assembly
 // so that the accumulators live in the accumulation registers ("a" operands):
@@ -145,23 +113,9 @@ __device__ inline uint16_t f32_to_elem(float f) {
     return f32_to_bf16_bits(f);
 }
 
-// s_waitcnt immediate (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4,
-// lgkmcnt 11:8): wait until at most n vector-memory requests are outstanding
-// and all LDS reads have returned.
-constexpr int wait_vm_lgkm0(int n) { return 0x0070 | (n & 15) | ((n >> 4) << 14); }
-
 // NWM x NWN wavefronts, each owning TM x TN sub-tiles of 16 x 16: the workgroup
 // tile is (16 NWM TM) x (16 NWN TN).
-// The columns of the output that one kind of tile covers: operands and result
-// already offset to the first of those columns.
-struct Part {
-    const uint16_t* x;
-    const uint16_t* w;
-    const uint16_t* bias;
-    uint16_t* y;
-    int64_t M, N, K, ldx, ldw, ldy;
-    int tiles_m, tiles_n, vec_store;
-};
+typedef PartOf<uint16_t> Part;
 
 template <bool F16, bool XT, bool WT, int NWM, int NWN, int TM, int TN>
 __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* lds) {
@@ -173,22 +127,8 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
     const int64_t M = part.M, N = part.N, K = part.K, ldx = part.ldx, ldw = part.ldw, ldy = part.ldy;
     const int tiles_m = part.tiles_m, tiles_n = part.tiles_n, vec_store = part.vec_store;
 
-    // XCD-aware tile assignment: hardware deals workgroup ids round-robin over
-    // the XCDs, so id % 8 names the XCD.  Give each XCD a contiguous range of
-    // the tile sequence, and walk that sequence in bands of 8 m-tiles.
-    const int ntiles = tiles_m * tiles_n;
-    int id = tile_id;
-    {
-        const int per = ntiles / kXcds, main = per * kXcds;
-        if (id < main) id = (id % kXcds) * per + id / kXcds;
-    }
-    constexpr int kBand = 8;
-    const int band = id / (kBand * tiles_n);
-    const int band_m0 = band * kBand;
-    const int band_h = (tiles_m - band_m0) < kBand ? (tiles_m - band_m0) : kBand;
-    const int in_band = id - band * kBand * tiles_n;
-    const int tm = band_m0 + in_band % band_h;
-    const int tn = in_band / band_h;
+    int tm, tn;
+    tile_of_workgroup(tile_id, tiles_m, tiles_n, tm, tn);
 
     constexpr int BM = 16 * NWM * TM, BN = 16 * NWN * TN;
     static_assert(BM <= kMaxTileRows && BN <= kMaxTileRows, "operand tile larger than a ring slot");
@@ -538,11 +478,7 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
 
 constexpr int kThreads = 512;
 
-// The two kinds of tiles of one product.
-struct Parts {
-    Part wide;     // 256 x 256 tiles: 2 x 4 wavefronts of 128 x 64
-    Part narrow;   // 256 x 192 tiles: 4 x 2 wavefronts of 64 x 96
-};
+typedef PartsOf<uint16_t> Parts;
 
 // Workgroup b computes wide tile b and then narrow tile b (where they exist):
 // the stores of the first tile drain while the second is computed, and there
@@ -566,11 +502,7 @@ const Kernel kKernels[8] = {
     gemm16_tiles<true, false, false>,  gemm16_tiles<true, false, true>,  gemm16_tiles<true, true, false>,  gemm16_tiles<true, true, true>,
 };
 
-// Per-device state, set on first use by whichever thread gets there (the
-// values are the same for all of them).
-constexpr int kMaxDevices = 64;
-std::atomic<bool> lds_reserved[kMaxDevices][8];   // the dynamic LDS size of kKernels[i] has been raised
-std::atomic<int> cu_count[kMaxDevices];           // 0: not asked yet
+std::atomic<bool> lds_reserved[kMaxDevices][8];   // the dynamic LDS size of kKernels[i] has been raised on that device (first use, any thread)
 
 // One operand of the product: element (row, k) at p[row * row_stride + k * k_stride],
 // one of the strides being 1.
@@ -617,27 +549,11 @@ int gemm16(const char* who, bool f16, Operand a, Operand b, const uint16_t* bias
     const bool at = a.transposed(), bt = b.transposed();
 
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
-    int cus = cu_count[dev].load(std::memory_order_relaxed);
-    if (cus == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
-        cus = n;
-        cu_count[dev].store(n, std::memory_order_relaxed);
-    }
-    // How many 256-column strips go to the wide tiles: whole rounds of them,
-    // the rest of the columns to 192-wide tiles, if that shortens the last round.
+    const int cus = compute_units(dev);
     const int64_t tiles_m = (M + 255) / 256, cols = (N + 255) / 256;
-    auto rounds = [&](int64_t tiles) { return (tiles + cus - 1) / cus; };
-    int64_t best_cost = rounds(tiles_m * cols) * 256, best_split = cols;   // strips of 256 columns given to the wide tiles
-    for (int64_t c = cols - 1; c >= 0 && c >= cols - 16; --c) {
-        const int64_t rest = N - c * 256;
-        const int64_t cost = rounds(tiles_m * c) * 256 + rounds(tiles_m * ((rest + 191) / 192)) * 192;
-        if (cost < best_cost) {
-            best_cost = cost;
-            best_split = c;
-        }
-    }
+    if (tiles_m > 0x7FFFFFll || cols > 0x7FFFFFll || tiles_m * (cols + 1) > 0x7FFFFFFFll)
+        return fail(DDL_E_UNSUPP, "%s: too many output tiles", who);
+    const int64_t wide_cols = wide_tile_columns(tiles_m, N, cus);
     // Columns [n_begin, n_begin + n_count) of the output with tiles of 256 x bn.
     auto part = [&](int bn, int64_t n_begin, int64_t n_count) {
         Part p{};
@@ -646,9 +562,6 @@ int gemm16(const char* who, bool f16, Operand a, Operand b, const uint16_t* bias
         p.tiles_m = static_cast<int>(tiles_m), p.tiles_n = static_cast<int>((n_count + bn - 1) / bn), p.vec_store = vec_store;
         return p;
     };
-    if (tiles_m > 0x7FFFFFll || cols > 0x7FFFFFll || tiles_m * (cols + 1) > 0x7FFFFFFFll)
-        return fail(DDL_E_UNSUPP, "%s: too many output tiles", who);
-    const int64_t wide_cols = best_split == cols ? N : best_split * 256;
     Parts parts{};
     if (wide_cols > 0) parts.wide = part(256, 0, wide_cols);
     if (wide_cols < N) parts.narrow = part(192, wide_cols, N - wide_cols);

@@ -1065,6 +1065,53 @@ def test_gemm_16_bit_random_within_tolerance_and_ragged_depth(ops, a_t, b_t):
     _lin_check(bits16(out), a, b, None)
 
 
+@pytest.mark.parametrize("a_t,b_t", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("M,N,K,pad", [(4060, 1000, 40, 0), (4096, 4352, 132, 4), (16384, 256, 36, 8), (4100, 1004, 288, 0)])
+def test_gemm_f32_tiled_kernel_reads_every_operand_layout(ops, a_t, b_t, M, N, K, pad):
+    """Products large enough for the 256-wide fp32 tiles (at least 64 of them), in
+    every combination of operand layouts, with integer operands: every sum is
+    exact in fp32, so the result must equal the fp64 product -- tiles that
+    straddle M, N and K, pitched operands, the wide / narrow column split."""
+    from distdl_amd import _lib
+    gen = torch.Generator().manual_seed(M + 3 * N + K + 2 * a_t + b_t)
+    a = torch.randint(-3, 4, (M, K), generator=gen).float()
+    b = torch.randint(-3, 4, (N, K), generator=gen).float()
+    bias = torch.randint(-5, 6, (N,), generator=gen).float()
+    ag, a_rs, a_ks = _gemm_operand(a, a_t, pad)
+    bg, b_rs, b_ks = _gemm_operand(b, b_t, pad)
+    ldy = N + 4
+    out = torch.full((M, ldy), 77.0, device="cuda")
+    rc = _lib.load().ddl_gemm_f32(ag.data_ptr(), a_rs, a_ks, bg.data_ptr(), b_rs, b_ks, bias.cuda().data_ptr(), out.data_ptr(), ldy,
+                                  M, N, K, torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "ddl_gemm_f32")
+    want = a.double() @ b.double().T + bias.double()
+    got = out.cpu().double()
+    assert torch.equal(got[:, :N], want)
+    assert (got[:, N:] == 77.0).all()
+
+
+def test_gemm_f32_tiled_kernel_random_and_odd_depth(ops):
+    """Random operands through the tiled fp32 kernel: both operands read along
+    their rows, so the reduction length may be anything (here 1003, no multiple
+    of the k-tile or of a vector); and the forward layout with K = 1000."""
+    from distdl_amd import _lib
+    for a_t, b_t, K in ((True, True, 1003), (False, False, 1000)):
+        M, N = 4096, 1024
+        gen = torch.Generator().manual_seed(K)
+        a = torch.randn(M, K, generator=gen)
+        b = 0.02 * torch.randn(N, K, generator=gen)
+        ag, a_rs, a_ks = _gemm_operand(a, a_t, 0)
+        bg, b_rs, b_ks = _gemm_operand(b, b_t, 0)
+        out = torch.empty((M, N), device="cuda")
+        rc = _lib.load().ddl_gemm_f32(ag.data_ptr(), a_rs, a_ks, bg.data_ptr(), b_rs, b_ks, None, out.data_ptr(), N, M, N, K,
+                                      torch.cuda.current_stream().cuda_stream)
+        _lib.check(rc, "ddl_gemm_f32")
+        want = a.double() @ b.double().T
+        err = (out.cpu().double() - want).abs()
+        # fp32 products and sums of K terms: relative to the size of the terms, a few ulp times sqrt(K)
+        assert float(err.max()) <= 1e-5 * float(a.abs().mean() * b.abs().mean()) * K
+
+
 def test_gemm_16_bit_refuses_what_it_cannot_read_in_place(ops):
     from distdl_amd import _lib
     lib = _lib.load()
