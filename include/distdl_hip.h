@@ -416,7 +416,10 @@ int ddl_linear_bf16(const void* x, const void* w, const void* bias, void* y,
  *   dx[M,K] = gemm(a = dy (N, 1),  b = w (1, K))       reduction over N
  *   dw[N,K] = gemm(a = dy (1, N),  b = x (1, K))       reduction over M
  * a, b, bias and y are of `dtype`; y is row-major with pitch ldy.
- * fp32: any strides.  bf16 / fp16 (the MFMA kernel of ddl_linear, which reads an
+ * fp32: any strides (products of at least 64 tiles of 256 x 256 whose operands
+ * have a unit stride, 16-byte alignment and a pitch that is a multiple of 4 run
+ * on the tiled MFMA kernel, everything else on a slower general one; the result
+ * is the same up to the order of the fp32 sums).  bf16 / fp16 (the MFMA kernel of ddl_linear, which reads an
  * operand that is contiguous along its rows through transposing LDS reads): each
  * operand needs one stride equal to 1, the other (its pitch) a multiple of 8, and
  * 16-byte alignment; an operand contiguous along k needs K % 8 == 0, one
