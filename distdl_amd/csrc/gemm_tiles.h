@@ -104,19 +104,21 @@ inline int compute_units(int& dev) {
 // and a last round that is only partly filled costs as much as a full one.
 // How many of the N output columns go to 256-wide tiles (whole rounds of them;
 // a multiple of 256, or N), the rest to 192-wide tiles, if that shortens the
-// last round.
-inline int64_t wide_tile_columns(int64_t tiles_m, int64_t N, int cus) {
+// last round.  *cost receives the length of the schedule in tile columns
+// (rounds of wide tiles x 256 + rounds of narrow tiles x 192).
+inline int64_t wide_tile_columns(int64_t tiles_m, int64_t N, int cus, int64_t* cost = nullptr) {
     const int64_t cols = (N + 255) / 256;
     auto rounds = [&](int64_t tiles) { return (tiles + cus - 1) / cus; };
     int64_t best_cost = rounds(tiles_m * cols) * 256, best_split = cols;   // strips of 256 columns given to the wide tiles
     for (int64_t c = cols - 1; c >= 0 && c >= cols - 16; --c) {
         const int64_t rest = N - c * 256;
-        const int64_t cost = rounds(tiles_m * c) * 256 + rounds(tiles_m * ((rest + 191) / 192)) * 192;
-        if (cost < best_cost) {
-            best_cost = cost;
+        const int64_t c_cost = rounds(tiles_m * c) * 256 + rounds(tiles_m * ((rest + 191) / 192)) * 192;
+        if (c_cost < best_cost) {
+            best_cost = c_cost;
             best_split = c;
         }
     }
+    if (cost) *cost = best_cost;
     return best_split == cols ? N : best_split * 256;
 }
 

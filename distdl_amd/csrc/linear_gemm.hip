@@ -495,6 +495,20 @@ __global__ __launch_bounds__(kThreads) void gemm16_tiles(const Parts parts) {
     }
 }
 
+// Tiles of 128 x 256 (2 x 4 wavefronts of 64 x 64), for products too small to
+// give every CU a 256 x 256 tile: twice as many workgroups, each half the work.
+template <bool F16, bool XT, bool WT>
+__global__ __launch_bounds__(kThreads) void gemm16_low_tiles(const Part part) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    gemm_tile<F16, XT, WT, 2, 4, 4, 4>(part, blockIdx.x, lds);
+}
+
+typedef void (*LowKernel)(const Part);
+const LowKernel kLowKernels[8] = {
+    gemm16_low_tiles<false, false, false>, gemm16_low_tiles<false, false, true>, gemm16_low_tiles<false, true, false>, gemm16_low_tiles<false, true, true>,
+    gemm16_low_tiles<true, false, false>,  gemm16_low_tiles<true, false, true>,  gemm16_low_tiles<true, true, false>,  gemm16_low_tiles<true, true, true>,
+};
+
 typedef void (*Kernel)(const Parts);
 // index: 4 fp16 + 2 (x transposed) + (w transposed)
 const Kernel kKernels[8] = {
@@ -502,7 +516,7 @@ const Kernel kKernels[8] = {
     gemm16_tiles<true, false, false>,  gemm16_tiles<true, false, true>,  gemm16_tiles<true, true, false>,  gemm16_tiles<true, true, true>,
 };
 
-std::atomic<bool> lds_reserved[kMaxDevices][8];   // the dynamic LDS size of kKernels[i] has been raised on that device (first use, any thread)
+std::atomic<bool> lds_reserved[kMaxDevices][16];   // the dynamic LDS size of kKernels[i] (8 + i: kLowKernels[i]) has been raised on that device (first use, any thread)
 
 // One operand of the product: element (row, k) at p[row * row_stride + k * k_stride],
 // one of the strides being 1.
@@ -553,25 +567,40 @@ int gemm16(const char* who, bool f16, Operand a, Operand b, const uint16_t* bias
     const int64_t tiles_m = (M + 255) / 256, cols = (N + 255) / 256;
     if (tiles_m > 0x7FFFFFll || cols > 0x7FFFFFll || tiles_m * (cols + 1) > 0x7FFFFFFFll)
         return fail(DDL_E_UNSUPP, "%s: too many output tiles", who);
-    const int64_t wide_cols = wide_tile_columns(tiles_m, N, cus);
-    // Columns [n_begin, n_begin + n_count) of the output with tiles of 256 x bn.
-    auto part = [&](int bn, int64_t n_begin, int64_t n_count) {
+    int64_t cost = 0;
+    const int64_t wide_cols = wide_tile_columns(tiles_m, N, cus, &cost);
+    // Columns [n_begin, n_begin + n_count) of the output with tiles of bm x bn.
+    auto part = [&](int bm, int bn, int64_t n_begin, int64_t n_count) {
         Part p{};
         p.x = a.p, p.w = b.p + n_begin * b.row_stride, p.bias = bias ? bias + n_begin : nullptr, p.y = y + n_begin;
         p.M = M, p.N = n_count, p.K = K, p.ldx = a.ld(), p.ldw = b.ld(), p.ldy = ldy;
-        p.tiles_m = static_cast<int>(tiles_m), p.tiles_n = static_cast<int>((n_count + bn - 1) / bn), p.vec_store = vec_store;
+        p.tiles_m = static_cast<int>((M + bm - 1) / bm), p.tiles_n = static_cast<int>((n_count + bn - 1) / bn), p.vec_store = vec_store;
         return p;
     };
-    Parts parts{};
-    if (wide_cols > 0) parts.wide = part(256, 0, wide_cols);
-    if (wide_cols < N) parts.narrow = part(192, wide_cols, N - wide_cols);
-    const int n_wide = parts.wide.tiles_m * parts.wide.tiles_n, n_narrow = parts.narrow.tiles_m * parts.narrow.tiles_n;
     const int k = (f16 ? 4 : 0) + (at ? 2 : 0) + (bt ? 1 : 0);
-    if (!lds_reserved[dev][k].load(std::memory_order_acquire)) {   // the attribute sticks to the function on this device
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kKernels[k]), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-        if (e != hipSuccess) return fail(static_cast<int>(e), "%s: cannot reserve %d bytes of LDS: %s", who, kLdsBytes, hipGetErrorString(e));
-        lds_reserved[dev][k].store(true, std::memory_order_release);
+    auto reserve_lds = [&](int slot, const void* kernel) -> int {
+        if (!lds_reserved[dev][slot].load(std::memory_order_acquire)) {   // the attribute sticks to the function on this device
+            const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+            if (e != hipSuccess) return fail(static_cast<int>(e), "%s: cannot reserve %d bytes of LDS: %s", who, kLdsBytes, hipGetErrorString(e));
+            lds_reserved[dev][slot].store(true, std::memory_order_release);
+        }
+        return 0;
+    };
+    // Tiles of half the height: twice the workgroups.  Taken when that shortens
+    // the schedule by more than the 10 % a smaller tile loses in efficiency.
+    const int64_t low_tiles = ((M + 127) / 128) * cols;
+    const int64_t low_cost = (low_tiles + cus - 1) / cus * 128;
+    if (low_cost * 11 < cost * 10) {
+        if (int rc = reserve_lds(8 + k, reinterpret_cast<const void*>(kLowKernels[k]))) return rc;
+        hipLaunchKernelGGL(kLowKernels[k], dim3(static_cast<uint32_t>(low_tiles)), dim3(kThreads), kLdsBytes, static_cast<hipStream_t>(stream),
+                           part(128, 256, 0, N));
+        return check_launch("gemm16_low_tiles");
     }
+    Parts parts{};
+    if (wide_cols > 0) parts.wide = part(256, 256, 0, wide_cols);
+    if (wide_cols < N) parts.narrow = part(256, 192, wide_cols, N - wide_cols);
+    const int n_wide = parts.wide.tiles_m * parts.wide.tiles_n, n_narrow = parts.narrow.tiles_m * parts.narrow.tiles_n;
+    if (int rc = reserve_lds(k, reinterpret_cast<const void*>(kKernels[k]))) return rc;
     hipLaunchKernelGGL(kKernels[k], dim3(static_cast<uint32_t>(n_wide > n_narrow ? n_wide : n_narrow)), dim3(kThreads), kLdsBytes,
                        static_cast<hipStream_t>(stream), parts);
     return check_launch("gemm16_tiles");

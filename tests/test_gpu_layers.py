@@ -1020,12 +1020,13 @@ def _gemm_operand(values, transposed, pad):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("a_t,b_t", [(False, False), (False, True), (True, False), (True, True)])
 @pytest.mark.parametrize("M,N,K,pad", [(8, 8, 8, 0), (16, 24, 72, 8), (304, 200, 136, 0), (264, 40, 64, 16), (520, 776, 200, 8),
-                                       (4096, 4352, 136, 0), (64, 192, 4104, 0)])
+                                       (4096, 4352, 136, 0), (64, 192, 4104, 0), (4096, 4096, 72, 0), (8192, 3592, 72, 8)])
 def test_gemm_16_bit_reads_operands_where_they_lie(ops, dtype, a_t, b_t, M, N, K, pad):
     """ddl_gemm on every combination of operand layouts (contiguous along k or
     along the rows), with small integers so that the result must be the exact
     integer: tiles that straddle M, N and K, pitched operands, one k-tile and
-    many, and a shape that is split between wide and narrow tiles."""
+    many; products small enough for the 128-row tiles, one that fills the chip
+    with 256 x 256 tiles, and one that is split between wide and narrow tiles."""
     from distdl_amd import _lib
     gen = torch.Generator().manual_seed(M * 7 + N * 3 + K + 2 * a_t + b_t)
     a = torch.randint(-1, 2, (M, K), generator=gen).to(dtype)
