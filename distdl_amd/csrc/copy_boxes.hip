@@ -34,6 +34,7 @@ constexpr uint32_t kTileLog = 10;  // log2(kTileVecs)
 static_assert((1u << kTileLog) == kTileVecs, "tile size must be 2^kTileLog");
 constexpr uint32_t kPersistentBlocks = 4096;  // 16 per CU
 constexpr uint64_t kMaxVecs = (1ull << 31) - kTileVecs;
+constexpr uint64_t kLongRunBytes = 64 << 10;   // boxes whose innermost runs are at least this long are interleaved within a launch
 
 enum Op { OP_COPY = 0, OP_ADD = 1, OP_ZERO = 2 };
 
@@ -70,6 +71,7 @@ struct Batch {
     uint32_t first_tile[kBatch];  // copy of box[i].first_tile, contiguous for one wide scalar load
     uint32_t nbox;
     uint32_t ntiles;
+    FastDiv rr;   // div = nbox when the launch walks its boxes round-robin (tile b belongs to box b % nbox), else 0
 };
 
 static_assert(sizeof(Batch) <= 4096, "box table must fit the kernel-argument segment");
@@ -290,12 +292,18 @@ __global__ __launch_bounds__(kThreads) void box_kernel(const Batch bt_by_value) 
     // stride of the grid, so a few thousand workgroups serve any volume.
     const uint32_t nbox = bt->nbox;
     const uint32_t ntiles = bt->ntiles;
+    const uint32_t rr_div = bt->rr.div, rr_mul = bt->rr.mul, rr_shr = bt->rr.shr;
     for (uint32_t b = blockIdx.x; b < ntiles; b += gridDim.x) {
-        uint32_t bi = 0;
+        uint32_t bi = 0, tile;
+        if (rr_div != 0) {   // boxes of equal tile counts, interleaved
+            tile = __umulhi(b, rr_mul) >> rr_shr;
+            bi = b - tile * rr_div;
+        } else {
 #pragma unroll
-        for (uint32_t i = 1; i < kBatch; ++i) bi += (i < nbox && b >= bt->first_tile[i]) ? 1u : 0u;
+            for (uint32_t i = 1; i < kBatch; ++i) bi += (i < nbox && b >= bt->first_tile[i]) ? 1u : 0u;
+            tile = b - bt->first_tile[bi];
+        }
         DevBoxPtr bx = &bt->box[bi];
-        const uint32_t tile = b - bx->first_tile;
         const uint32_t nd = bx->nd;
         switch (bx->vlog) {
             case 4: move_tile_nd<OP, T, u32x4>(bx, tile, nd); break;
@@ -462,6 +470,21 @@ int launch_batches(const std::vector<DevBox>& boxes, hipStream_t stream) {
         }
         bt.nbox = n;
         bt.ntiles = static_cast<uint32_t>(tiles);
+        // Order of the tiles.  Box after box is the default.  Boxes whose rows
+        // are long contiguous runs (the 1 MiB pieces an unpack of
+        // [8,4096,1024] bf16 from eight buffers writes into its output, 8 MiB
+        // apart) are walked round-robin instead: the few thousand tiles in
+        // flight at one moment then touch the pieces of all boxes rather than
+        // those of the first few, which spreads the accesses over address bits
+        // 20 and up -- measured 5 to 12 % faster for that unpack, depending on
+        // the machine, while the pack of the same repartition (rows of 2 KiB)
+        // loses 1 % when interleaved and stays box after box.
+        bool interleave = n >= 2 && tiles < 0x7FFFFFFFull;
+        for (uint32_t k = 0; k < n && interleave; ++k) {
+            const uint64_t own = (k + 1 < n ? bt.first_tile[k + 1] : tiles) - bt.first_tile[k];
+            interleave = own * n == tiles && (static_cast<uint64_t>(bt.box[k].cols) << bt.box[k].vlog) >= kLongRunBytes;
+        }
+        bt.rr = interleave ? make_fastdiv(n) : FastDiv{0, 0, 0, 0};
         const uint32_t blocks = tiles < kPersistentBlocks ? static_cast<uint32_t>(tiles) : kPersistentBlocks;
         hipLaunchKernelGGL((box_kernel<OP, T>), dim3(blocks), dim3(kThreads), 0, stream, bt);
         if (int rc = check_launch("box_kernel")) return rc;

@@ -173,6 +173,33 @@ def test_repartition_config2_rank0_bit_exact(ops):
     assert torch.equal(bits(y2.cpu()), bits(x_cpu))
 
 
+@pytest.mark.parametrize("nbox,rows,run", [(2, 3, 32768), (3, 5, 40960), (7, 4, 262144), (8, 2, 32768), (5, 3, 32772)])
+def test_boxes_with_long_rows_are_walked_round_robin(ops, nbox, rows, run):
+    """Boxes of equal size whose rows are long contiguous runs (64 KiB and more)
+    share a launch tile by tile in turn instead of box after box: a split of
+    dimension 1 of [rows, nbox * run] bf16, packed, unpacked and accumulated.
+    7 x 4 x 512 KiB is more tiles than the launch has workgroups; a run of
+    32772 elements leaves a ragged last tile in every row."""
+    gen = torch.Generator().manual_seed(nbox * 1000 + rows)
+    x_cpu = random_bits((rows, nbox * run), torch.bfloat16, gen)
+    x = x_cpu.cuda()
+    slices = [(slice(0, rows), slice(b * run, (b + 1) * run)) for b in range(nbox)]
+    plan = ops.BoxPlan.from_slices(x, slices)
+    bufs = [torch.empty(rows, run, dtype=torch.bfloat16, device="cuda") for _ in range(nbox)]
+    plan.pack(x, bufs)
+    for b, sl in zip(bufs, slices):
+        assert torch.equal(bits(b.cpu()), bits(x_cpu[sl]))
+    y = torch.empty_like(x)
+    plan.unpack(y, bufs)
+    assert torch.equal(bits(y.cpu()), bits(x_cpu))
+    # accumulate: every element exactly once
+    acc_cpu = torch.randint(-8, 9, (rows, nbox * run), generator=gen).to(torch.float32)
+    add_cpu = [torch.randint(-8, 9, (rows, run), generator=gen).to(torch.float32) for _ in range(nbox)]
+    acc = acc_cpu.cuda()
+    ops.BoxPlan.from_slices(acc, slices).unpack(acc, [a.cuda() for a in add_cpu], accumulate=True)
+    assert torch.equal(acc.cpu(), acc_cpu + torch.cat(add_cpu, dim=1))
+
+
 # ---------------------------------------------- Repartition layer, loopback --
 
 def _run_repartition_world(world_size, P_x_workers, P_x_shape, P_y_workers, P_y_shape, x_by_rank, dy_by_rank, dtype,
