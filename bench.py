@@ -327,6 +327,25 @@ def build_layernorm(torch, lib, _lib, nsets):
     return steps, keep, 25298944
 
 
+def build_layernorm_joined(torch, lib, _lib, nsets):
+    """Config 1 in one launch (ddl_ln_stats_normalize): the peers' statistics are
+    seeded, i.e. in memory before the launch, so the kernel that computes rank
+    0's partial sums can go on to normalise with the row still in registers.
+    `work` is what the kernel moves -- x read ONCE, y written, statistics and
+    parameters -- not config 1's three passes; the two-launch form (workload
+    `layernorm`) is what applies when peers compute at the same time."""
+    rows, cols = 16 * 512, 256
+    steps2, keep = _ln_steps(torch, lib, _lib, nsets, rows, cols, 1001, True)
+    part_cols = _lib.i64_array([cols] * 4)
+    steps = []
+    for (x, gamma, beta, gathered, y, _, _) in keep:
+        args = (x.data_ptr(), _lib.DDL_DT_F32, rows, cols, cols, gathered.data_ptr(), 4, 0, part_cols, gamma.data_ptr(),
+                beta.data_ptr(), 1e-5, y.data_ptr(), cols, None, None)
+        steps.append([_call(lib, _lib, "ddl_ln_stats_normalize", args)])
+    keep.append(part_cols)
+    return steps, keep, 2 * rows * cols * 4 + 2 * cols * 4 + 4 * rows * 8
+
+
 def build_layernorm_long(torch, lib, _lib, nsets):
     """The kernels of config 1 on 32 times its rows ([262144, 256] fp32, 268 MB):
     the streaming rate of the same code once launch ramp and memory latency no
@@ -898,6 +917,7 @@ def _build_mfma_probe(instruction, random):
 WORKLOADS = {
     "repartition": (build_repartition, 8, 2, "hbm", "mean", layer_repartition, cpu_repartition, 2),
     "layernorm": (build_layernorm, 64, 2, "hbm", "mean", layer_layernorm, cpu_layernorm, 1),
+    "layernorm_joined": (build_layernorm_joined, 64, 1, "hbm", None, None, None, None),
     "layernorm_long": (build_layernorm_long, 3, 2, "hbm", None, None, None, None),
     "layernorm_wide": (build_layernorm_wide, 4, 2, "hbm", None, None, None, None),
     "layernorm_local": (build_layernorm_local, 16, 1, "hbm", None, None, None, None),

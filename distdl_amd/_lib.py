@@ -70,6 +70,8 @@ SIGNATURES = {
                                         c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "ddl_layer_norm": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float, c_void_p, c_int64,
                                c_void_p, c_void_p, c_void_p]),
+    "ddl_ln_stats_normalize": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_int, POINTER(c_int64),
+                                       c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "ddl_ln_partial_stats_f32": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "ddl_ln_normalize_affine_f32": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int, POINTER(c_int64),
                                             c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_void_p,

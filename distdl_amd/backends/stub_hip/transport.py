@@ -119,6 +119,14 @@ class SoloTransport:
             self._seeded[tag] = (buffer.data_ptr(), tuple(buffer.shape))
         return buffer
 
+    def peers_gathered_ahead(self, P, buffer, tag=None):
+        """True when the slots of ``buffer`` other than ``P.rank`` hold the
+        peers' parts before the live rank's part exists (they were seeded, or a
+        provider has filled them on an earlier call), so that one kernel may
+        produce the live part and consume the others."""
+        fn = self._gather_providers.get(tag)
+        return fn is None or self._seeded.get(tag) == (buffer.data_ptr(), tuple(buffer.shape))
+
     def broadcast(self, P_src, P_dst, tensor, tag=None):
         if P_src.active:
             return tensor
@@ -309,6 +317,11 @@ class LoopbackTransport:
         # Nobody may overwrite its contribution before everyone has stacked it.
         self._allgather_obj(P, None, ("tgather-done", tag))
         return out
+
+    def peers_gathered_ahead(self, P, buffer, tag=None):
+        """Peers compute their parts while this worker computes its own: never
+        ahead."""
+        return False
 
     def allgather_into(self, P, buffer, tag=None):
         """In-place all-gather: ``buffer`` is ``[P.size, ...]`` and slot

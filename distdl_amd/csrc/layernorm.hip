@@ -6,6 +6,9 @@
 //                -> combined mean / var -> y = (x-mean)*rstd*gamma+beta
 //   ln_fused     both in one launch, for rows that one worker holds whole
 //                (the reference's torch.nn.functional.layer_norm branch, :310-319)
+//   ln_joined    both in one launch for rows shared with other workers whose
+//                {mean, M2} are in memory before the launch: the row stays in
+//                registers between the two halves, so x is read once
 //
 // Three ways of holding a row, chosen by its length:
 //   wavefront rows  up to 2048 columns: one wavefront owns a row, each lane
@@ -104,6 +107,7 @@ enum Mode {
     kStats = 0,   // emit {mean, M2} of the local columns
     kNorm = 1,    // statistics come from the gathered pairs
     kFused = 2,   // statistics of the local columns are the row's statistics
+    kJoined = 3,  // emit {mean, M2} of the local columns, take the other workers' pairs from memory, normalise
 };
 
 struct LnArgs {
@@ -118,6 +122,7 @@ struct LnArgs {
     int64_t rows, ld, ldy;
     int cols;
     int nparts;
+    int my_part;   // kJoined: this worker's place among the nparts
     float eps;
 };
 
@@ -150,7 +155,7 @@ __global__ __launch_bounds__(kBlock) void ln_wave_rows(const LnArgs a, const Par
     // the rows themselves.
     float2 ps[RPW];
     float inv_n = 0.f;
-    if (MODE == kNorm) {
+    if (MODE == kNorm || MODE == kJoined) {
         inv_n = lane < a.nparts ? pc.inv_n[lane] : 0.f;
 #pragma unroll
         for (int i = 0; i < RPW; ++i) {
@@ -186,11 +191,15 @@ __global__ __launch_bounds__(kBlock) void ln_wave_rows(const LnArgs a, const Par
             for (int k = 0; k < NV; ++k)
                 if (lane + k * kWave < nv) q += sq4(v[i][k], mean);
             q = wave_sum(q);
-            if (MODE == kStats) {
+            if (MODE == kStats || MODE == kJoined) {
                 if (lane == 0) reinterpret_cast<float2*>(a.stats)[r] = make_float2(mean, q);
-                continue;
+                if (MODE == kStats) continue;
             }
-            rstd = 1.0f / sqrtf(q * inv + a.eps);
+            if (MODE == kJoined)   // this worker's pair comes from the registers, the others' from memory (nparts <= 64)
+                combine_parts(a.part_stats, rows, r, a.nparts, pc, a.eps, lane, lane == a.my_part ? make_float2(mean, q) : ps[i],
+                              inv_n, &mean, &rstd);
+            else
+                rstd = 1.0f / sqrtf(q * inv + a.eps);
         }
         if (lane == 0) {
             if (a.mean_out) a.mean_out[r] = mean;
@@ -222,7 +231,7 @@ __global__ __launch_bounds__(kBlock) void ln_block_rows(const LnArgs a, const Pa
     const float inv = 1.0f / static_cast<float>(a.cols);
     for (int64_t r = blockIdx.x; r < a.rows; r += gridDim.x) {
         float2 first = make_float2(0.f, 0.f);
-        if (MODE == kNorm && lane < a.nparts) first = load_part(a.part_stats, a.rows, r, lane);
+        if ((MODE == kNorm || MODE == kJoined) && lane < a.nparts) first = load_part(a.part_stats, a.rows, r, lane);
         float4 v[NV];
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
@@ -244,11 +253,15 @@ __global__ __launch_bounds__(kBlock) void ln_block_rows(const LnArgs a, const Pa
             for (int k = 0; k < NV; ++k)
                 if (t + k * kBlock < nv) q += sq4(v[k], mean);
             q = block_sum(q, scratch);
-            if (MODE == kStats) {
+            if (MODE == kStats || MODE == kJoined) {
                 if (t == 0) reinterpret_cast<float2*>(a.stats)[r] = make_float2(mean, q);
-                continue;
+                if (MODE == kStats) continue;
             }
-            rstd = 1.0f / sqrtf(q * inv + a.eps);
+            if (MODE == kJoined)
+                combine_parts(a.part_stats, a.rows, r, a.nparts, pc, a.eps, lane, lane == a.my_part ? make_float2(mean, q) : first,
+                              lane < a.nparts ? pc.inv_n[lane] : 0.f, &mean, &rstd);
+            else
+                rstd = 1.0f / sqrtf(q * inv + a.eps);
         }
         if (t == 0) {
             if (a.mean_out) a.mean_out[r] = mean;
@@ -376,12 +389,16 @@ int launch_typed(const LnArgs& a, const PartCounts& pc, bool vec, hipStream_t s)
         else launch_block<T, MODE, AFFINE, 16>(a, pc, s);
         return check_launch("ln_block_rows");
     }
-    const uint32_t blocks = static_cast<uint32_t>(a.rows < 65536 ? a.rows : 65536);
-    if (vec)
-        hipLaunchKernelGGL((ln_stream_rows<T, MODE, true>), dim3(blocks), dim3(kBlock), 0, s, a, pc);
-    else
-        hipLaunchKernelGGL((ln_stream_rows<T, MODE, false>), dim3(blocks), dim3(kBlock), 0, s, a, pc);
-    return check_launch("ln_stream_rows");
+    if constexpr (MODE == kJoined) {
+        return fail(DDL_E_UNSUPP, "ln stats+normalize: rows of more than %d columns take the two-launch form", kBlockRowCols);
+    } else {
+        const uint32_t blocks = static_cast<uint32_t>(a.rows < 65536 ? a.rows : 65536);
+        if (vec)
+            hipLaunchKernelGGL((ln_stream_rows<T, MODE, true>), dim3(blocks), dim3(kBlock), 0, s, a, pc);
+        else
+            hipLaunchKernelGGL((ln_stream_rows<T, MODE, false>), dim3(blocks), dim3(kBlock), 0, s, a, pc);
+        return check_launch("ln_stream_rows");
+    }
 }
 
 template <int MODE>
@@ -476,6 +493,37 @@ int ddl_layer_norm(const void* x, int dtype, int64_t rows, int64_t cols, int64_t
     const bool vec = quad_access(x, es, cols, ld) && quad_access(y, es, cols, ldy) &&
                      (!gamma || (aligned_to(gamma, 4 * es) && aligned_to(beta, 4 * es)));
     return launch_mode<kFused>(dtype, a, pc, vec, static_cast<hipStream_t>(stream));
+}
+
+int ddl_ln_stats_normalize(const void* x, int dtype, int64_t rows, int64_t cols, int64_t ld, float* part_stats, int nparts,
+                           int my_part, const int64_t* part_cols, const void* gamma, const void* beta, float eps, void* y,
+                           int64_t ldy, float* mean_out, float* rstd_out, void* stream) {
+    using namespace ddl;
+    if (const int rc = check_common("ln stats+normalize", dtype, rows, cols, ld)) return rc;
+    if (ldy < cols) return fail(DDL_E_ARG, "ln stats+normalize: ldy=%lld below cols=%lld", (long long)ldy, (long long)cols);
+    if (nparts < 1 || nparts > kWave) return fail(DDL_E_UNSUPP, "ln stats+normalize: nparts=%d outside [1,%d]", nparts, kWave);
+    if (my_part < 0 || my_part >= nparts) return fail(DDL_E_ARG, "ln stats+normalize: my_part=%d outside [0,%d)", my_part, nparts);
+    if ((gamma == nullptr) != (beta == nullptr)) return fail(DDL_E_ARG, "ln stats+normalize: gamma and beta must both be given or both be NULL");
+    if (rows == 0) return 0;
+    if (!x || !y || !part_stats || !part_cols) return fail(DDL_E_ARG, "ln stats+normalize: null pointer");
+    const int es = elem_size_of(dtype);
+    if (!aligned_to(x, es) || !aligned_to(y, es) || !aligned_to(gamma, es) || !aligned_to(beta, es) || !aligned_to(part_stats, 8))
+        return fail(DDL_E_ALIGN, "ln stats+normalize: x, y, gamma, beta must be element-aligned and the statistics 8-byte aligned");
+    PartCounts pc{};
+    for (int p = 0; p < nparts; ++p) {
+        if (part_cols[p] < 1) return fail(DDL_E_ARG, "ln stats+normalize: worker %d holds %lld columns", p, (long long)part_cols[p]);
+        pc.inv_n[p] = 1.0f / static_cast<float>(part_cols[p]);
+    }
+    if (part_cols[my_part] != cols) return fail(DDL_E_ARG, "ln stats+normalize: worker %d holds %lld columns, x has %lld", my_part, (long long)part_cols[my_part], (long long)cols);
+    LnArgs a{};
+    a.x = x, a.y = y, a.gamma = gamma, a.beta = beta, a.part_stats = part_stats;
+    a.stats = part_stats + static_cast<int64_t>(my_part) * rows * 2;
+    a.mean_out = mean_out, a.rstd_out = rstd_out;
+    a.rows = rows, a.ld = ld, a.ldy = ldy, a.cols = static_cast<int>(cols), a.nparts = nparts, a.my_part = my_part, a.eps = eps;
+    const bool vec = quad_access(x, es, cols, ld) && quad_access(y, es, cols, ldy) &&
+                     (!gamma || (aligned_to(gamma, 4 * es) && aligned_to(beta, 4 * es)));
+    if (!vec) return fail(DDL_E_UNSUPP, "ln stats+normalize: rows must allow four-element accesses (columns and pitches multiples of 4, aligned)");
+    return launch_mode<kJoined>(dtype, a, pc, vec, static_cast<hipStream_t>(stream));
 }
 
 int ddl_ln_partial_stats_f32(const float* x, int64_t rows, int64_t cols, int64_t ld, float* stats, void* stream) {

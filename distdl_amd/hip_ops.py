@@ -298,6 +298,45 @@ def ln_normalize_affine(x2d, part_stats, part_cols, gamma, beta, eps, want_stats
     return (y, mean, rstd) if want_stats else y
 
 
+def ln_joined_supported(x2d, nparts, gamma=None, beta=None):
+    """Whether ``ln_stats_normalize`` takes these rows: at most 64 workers, rows
+    of at most 16384 columns, columns and row pitch multiples of 4, x and the
+    parameters aligned to four elements."""
+    rows, cols = x2d.shape
+    quad = 4 * x2d.element_size()
+    return (nparts <= 64 and cols <= 16384 and cols % 4 == 0 and (rows <= 1 or x2d.stride(0) % 4 == 0) and
+            x2d.data_ptr() % quad == 0 and
+            (gamma is None or (gamma.data_ptr() % quad == 0 and beta.data_ptr() % quad == 0)))
+
+
+def ln_stats_normalize(x2d, part_stats, my_part, part_cols, gamma, beta, eps, want_stats=False, part_cols_arr=None):
+    """``ln_partial_stats`` into slot ``my_part`` of ``part_stats`` [P, rows, 2]
+    and ``ln_normalize_affine`` on the completed table, in one launch and one
+    read of x2d: for a worker whose peers' slots are filled before the call.
+    Returns y (and mean, rstd), bit-equal to the two calls.  Rows the single
+    launch does not take (see ``ln_joined_supported``) raise ``RuntimeError``."""
+    _require_gpu(x2d, part_stats, gamma, beta)
+    dt, ld = _ln_rows(x2d, "ln_stats_normalize")
+    rows, cols = x2d.shape
+    nparts = len(part_cols)
+    if part_stats.dtype != torch.float32 or tuple(part_stats.shape) != (nparts, rows, 2) or \
+       not part_stats.is_contiguous():
+        raise ValueError(f"ln_stats_normalize: part_stats must be contiguous fp32 [{nparts}, {rows}, 2]")
+    _ln_params(x2d, gamma, beta, "ln_stats_normalize")
+    y = torch.empty((rows, cols), dtype=x2d.dtype, device=x2d.device)
+    mean = rstd = None
+    if want_stats:
+        mean = torch.empty((rows,), dtype=torch.float32, device=x2d.device)
+        rstd = torch.empty((rows,), dtype=torch.float32, device=x2d.device)
+    if part_cols_arr is None:
+        part_cols_arr = _lib.i64_array(part_cols)
+    rc = _lib.load().ddl_ln_stats_normalize(x2d.data_ptr(), dt, rows, cols, ld, part_stats.data_ptr(), nparts, int(my_part),
+                                            part_cols_arr, _ptr(gamma), _ptr(beta), float(eps), y.data_ptr(), cols,
+                                            _ptr(mean), _ptr(rstd), _stream())
+    _lib.check(rc, "ddl_ln_stats_normalize")
+    return (y, mean, rstd) if want_stats else y
+
+
 def layer_norm(x2d, gamma, beta, eps, want_stats=False):
     """Layer norm of rows held whole by this worker, one launch; returns y (and mean, rstd)."""
     _require_gpu(x2d, gamma, beta)

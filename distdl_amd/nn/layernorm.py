@@ -51,10 +51,17 @@ def _shard_forward(input, weight, bias, P_reduce, part_cols, eps, part_cols_arr,
         gathered = stats_buffers.get(rows)
         if gathered is None or gathered.device != x2d.device:
             gathered = stats_buffers[rows] = torch.zeros((nparts, rows, 2), dtype=torch.float32, device=x2d.device)
-        hip_ops.ln_partial_stats(x2d, out=gathered[P_reduce.rank])
-        P_reduce._world.transport.allgather_into(P_reduce, gathered, tag=STATS_TAG)
-        res = hip_ops.ln_normalize_affine(x2d, gathered, part_cols, gamma, beta, eps, want_stats=keep,
-                                          part_cols_arr=part_cols_arr)
+        transport = P_reduce._world.transport
+        if transport.peers_gathered_ahead(P_reduce, gathered, tag=STATS_TAG) and \
+           hip_ops.ln_joined_supported(x2d, nparts, gamma, beta):
+            # The peers' statistics are there already: one launch, one read of x.
+            res = hip_ops.ln_stats_normalize(x2d, gathered, P_reduce.rank, part_cols, gamma, beta, eps, want_stats=keep,
+                                             part_cols_arr=part_cols_arr)
+        else:
+            hip_ops.ln_partial_stats(x2d, out=gathered[P_reduce.rank])
+            transport.allgather_into(P_reduce, gathered, tag=STATS_TAG)
+            res = hip_ops.ln_normalize_affine(x2d, gathered, part_cols, gamma, beta, eps, want_stats=keep,
+                                              part_cols_arr=part_cols_arr)
     else:
         res = hip_ops.layer_norm(x2d, gamma, beta, eps, want_stats=keep)
     if not keep:
@@ -217,7 +224,9 @@ class DistributedLayerNorm(Module):
         gradient is recorded: everything that only depends on the input's
         shape (row and column counts, the gathered-statistics buffer and the
         address of this worker's slot in it) is worked out once per shape, and a
-        call is the two entry points with the transport's gather between."""
+        call is the two entry points with the transport's gather between -- or
+        the single-launch entry point when the peers' statistics are in the
+        buffer beforehand."""
         plan = self._call_plan
         if plan is None or plan[0] != input.shape or plan[1] != input.dtype or plan[2] != input.device:
             P_reduce = self.allreduce.P_allreduce
@@ -231,9 +240,10 @@ class DistributedLayerNorm(Module):
                     gathered = self._stats_buffers[rows] = torch.zeros((nparts, rows, 2), dtype=torch.float32,
                                                                        device=input.device)
                 own = gathered.data_ptr() + P_reduce.rank * rows * 8
+            joinable = 1 < nparts <= 64 and cols <= 16384 and cols % 4 == 0     # what ddl_ln_stats_normalize takes
             plan = self._call_plan = (input.shape, input.dtype, input.device, rows, cols, hip_ops._LN_DTYPES[input.dtype],
-                                      nparts, gathered, own, P_reduce, _lib.load())
-        _, _, _, rows, cols, dt, nparts, gathered, own, P_reduce, lib = plan
+                                      nparts, gathered, own, P_reduce, _lib.load(), joinable, 4 * input.element_size())
+        _, _, _, rows, cols, dt, nparts, gathered, own, P_reduce, lib, joinable, quad = plan
         if weight is not None and (weight.numel() != cols or bias.numel() != cols):
             raise ValueError(f"DistributedLayerNorm parameters hold {weight.numel()} / {bias.numel()} elements, "
                              f"the local rows hold {cols}")
@@ -241,7 +251,15 @@ class DistributedLayerNorm(Module):
         stream = hip_ops._stream()
         gamma = None if weight is None else weight.data_ptr()
         beta = None if bias is None else bias.data_ptr()
-        if nparts > 1:
+        if nparts > 1 and joinable and input.data_ptr() % quad == 0 and \
+           (weight is None or (weight.data_ptr() % quad == 0 and bias.data_ptr() % quad == 0)) and \
+           P_reduce._world.transport.peers_gathered_ahead(P_reduce, gathered, tag=STATS_TAG):
+            rc = lib.ddl_ln_stats_normalize(input.data_ptr(), dt, rows, cols, cols, gathered.data_ptr(), nparts, P_reduce.rank,
+                                            self._part_cols_arr, gamma, beta, self.eps, y.data_ptr(), cols, None, None,
+                                            stream)
+            if rc:
+                _lib.check(rc, "ddl_ln_stats_normalize")
+        elif nparts > 1:
             rc = lib.ddl_ln_partial_stats(input.data_ptr(), dt, rows, cols, cols, own, stream)
             if rc:
                 _lib.check(rc, "ddl_ln_partial_stats")

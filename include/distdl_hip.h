@@ -223,6 +223,26 @@ int ddl_layer_norm(const void* x, int dtype, int64_t rows, int64_t cols, int64_t
                    void* y, int64_t ldy, float* mean_out, float* rstd_out,
                    void* stream);
 
+/* ddl_ln_partial_stats and ddl_ln_normalize_affine in ONE launch, for a worker
+ * whose peers' statistics are in memory before the launch: slots p != my_part
+ * of part_stats[nparts][rows][2] are read, slot my_part is written (the pair
+ * ddl_ln_partial_stats would store), and y, mean_out, rstd_out are what
+ * ddl_ln_normalize_affine would return for the completed table, bit for bit.
+ * The row stays in registers between the two halves, so x is read once.
+ * The same reference lines, nn/layernorm.py:230-233, :246-247, :298-302, :309;
+ * which of the two forms applies is decided by where the all-reduces of
+ * :231 and :247 stand in time: a peer whose pair can only arrive after this
+ * worker's own has been sent needs the two launches.
+ * Limits: nparts <= 64; rows of at most 16384 columns, columns and pitches
+ * multiples of 4, 4-element-aligned pointers (else DDL_E_UNSUPP: take the two
+ * launches).  part_cols[my_part] must equal cols. */
+int ddl_ln_stats_normalize(const void* x, int dtype, int64_t rows, int64_t cols,
+                           int64_t ld, float* part_stats, int nparts,
+                           int my_part, const int64_t* part_cols,
+                           const void* gamma, const void* beta, float eps,
+                           void* y, int64_t ldy, float* mean_out,
+                           float* rstd_out, void* stream);
+
 /* The fp32 forms of the first two (dtype = DDL_DT_F32). */
 int ddl_ln_partial_stats_f32(const float* x, int64_t rows, int64_t cols,
                              int64_t ld, float* stats /*[rows][2]*/,

@@ -56,6 +56,7 @@ def _ln_case(ops, shards_cpu, gamma_full, beta_full, eps, live=0, strict=True):
     b = None if beta_full is None else torch.from_numpy(beta_full[offs[live]:offs[live + 1]].copy()).cuda()
     y, mean, rstd = ops.ln_normalize_affine(x2d, gathered, cols, g, b, eps, want_stats=True)
     torch.cuda.synchronize()
+    _ln_joined_equals_two_launches(ops, x2d, gathered, live, cols, g, b, eps, y, mean, rstd)
     gs = [None if gamma_full is None else gamma_full[offs[p]:offs[p + 1]] for p in range(len(cols))]
     bs = [None if beta_full is None else beta_full[offs[p]:offs[p + 1]] for p in range(len(cols))]
     exact = o_ln.forward_shards(shards_cpu, gs, bs, eps, dtype=np.float64)[live].reshape(-1, cols[live])
@@ -67,6 +68,24 @@ def _ln_case(ops, shards_cpu, gamma_full, beta_full, eps, live=0, strict=True):
     # and no worse than the reference's own fp32 op sequence
     assert np.abs(got - exact).max() <= max(4 * np.abs(ref32 - exact).max(), 3e-6)
     return got, exact
+
+
+def _ln_joined_equals_two_launches(ops, x2d, gathered, live, cols, g, b, eps, y, mean=None, rstd=None):
+    """The single launch that writes this worker's statistics and consumes the
+    peers' (already in the table) gives the bits of the two launches: y, the
+    combined mean and rstd, and the worker's own slot of the table."""
+    if not ops.ln_joined_supported(x2d, len(cols), g, b):
+        with pytest.raises(RuntimeError, match="code -5"):      # DDL_E_UNSUPP
+            ops.ln_stats_normalize(x2d, gathered.clone(), live, cols, g, b, eps)
+        return
+    table = gathered.clone()
+    table[live] = float("nan")          # the launch must produce this slot itself
+    y2, mean2, rstd2 = ops.ln_stats_normalize(x2d, table, live, cols, g, b, eps, want_stats=True)
+    torch.cuda.synchronize()
+    assert torch.equal(table, gathered)
+    assert torch.equal(y2.view(torch.uint8), y.view(torch.uint8))
+    if mean is not None:
+        assert torch.equal(mean2, mean) and torch.equal(rstd2, rstd)
 
 
 def test_layernorm_config1_rank0(ops):
@@ -163,10 +182,70 @@ def test_layernorm_16_bit_elements(ops, dtype, cols):
             assert np.allclose(stats.cpu().numpy()[:, 0], want_stats[:, 0], rtol=1e-5, atol=1e-5)
             parts = [stats if p == live else torch.from_numpy(o_ln.partial_stats(shards64[p]).astype(np.float32)).cuda()
                      for p in range(len(cols))]
-            y = ops.ln_normalize_affine(x2d, torch.stack(parts).contiguous(), cols, g, b, 1e-5)
+            gathered = torch.stack(parts).contiguous()
+            y = ops.ln_normalize_affine(x2d, gathered, cols, g, b, 1e-5)
+            _ln_joined_equals_two_launches(ops, x2d, gathered, live, cols, g, b, 1e-5, y)
         assert y.dtype == dtype
         got = y.cpu().double().numpy()
         assert (np.abs(got - exact[live]) <= tol * np.maximum(np.abs(exact[live]), 1.0)).all()
+
+
+def test_layernorm_layer_takes_one_launch_once_the_peers_are_seeded(ops):
+    """One live rank of four: the first forward runs stats, gather, normalize
+    and leaves the peers' statistics in the layer's table; from then on the
+    transport reports them as present beforehand and the layer needs a single
+    launch.  Both give the oracle's result; the gradient path does the same."""
+    from distdl_amd import _lib
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedLayerNorm
+    from distdl_amd.nn.layernorm import STATS_TAG
+    world = SimWorld(4)
+    P_x = world.partition(0).create_partition_inclusive(list(range(4))).create_cartesian_topology_partition([1, 1, 4])
+    layer = DistributedLayerNorm(P_x, [512])
+    gen = torch.Generator().manual_seed(77)
+    whole = torch.randn(3, 50, 512, generator=gen)
+    shards = [np.ascontiguousarray(whole[..., 128 * p:128 * (p + 1)].numpy()) for p in range(4)]
+    peers = [None] + [torch.from_numpy(o_ln.partial_stats(shards[p]).astype(np.float32)).cuda() for p in range(1, 4)]
+    world.transport.set_gather_provider(STATS_TAG, lambda P, t: list(peers))
+    with torch.no_grad():
+        layer.weight.copy_((1 + 0.1 * torch.randn(128, generator=gen)).view(1, 1, 128))
+        layer.bias.copy_((0.1 * torch.randn(128, generator=gen)).view(1, 1, 128))
+    gs = [layer.weight.detach().cpu().numpy().reshape(-1)] + [None] * 3
+    bs = [layer.bias.detach().cpu().numpy().reshape(-1)] + [None] * 3
+    exact = o_ln.forward_shards(shards, gs, bs, 1e-5, dtype=np.float64)[0]
+    x = torch.from_numpy(shards[0]).cuda()
+    lib = _lib.load()
+    calls = []
+    real = lib.ddl_ln_stats_normalize
+
+    class Spy:
+        def __getattr__(self, name):
+            if name == "ddl_ln_stats_normalize":
+                def counted(*args):
+                    calls.append(name)
+                    return real(*args)
+                return counted
+            return getattr(lib, name)
+    saved = _lib.load
+    _lib.load = lambda: Spy()
+    try:
+        layer._call_plan = None
+        with torch.no_grad():
+            y_first = layer(x)
+            assert calls == []
+            y_second = layer(x)
+            assert calls == ["ddl_ln_stats_normalize"]
+        xg = x.clone().requires_grad_(True)
+        y_grad = layer(xg)
+        assert len(calls) == 2
+    finally:
+        _lib.load = saved
+        layer._call_plan = None
+    torch.cuda.synchronize()
+    for y in (y_first, y_second, y_grad.detach()):
+        got = y.cpu().numpy().astype(np.float64)
+        assert (np.abs(got - exact) <= LN_RTOL * np.maximum(np.abs(exact), 1.0)).all()
+    assert torch.equal(y_first, y_second) and torch.equal(y_first, y_grad.detach())
 
 
 def test_layernorm_layer_single_worker_and_bf16(ops):
