@@ -228,6 +228,72 @@ def _run_repartition_world(world_size, P_x_workers, P_x_shape, P_y_workers, P_y_
     return SimWorld(world_size).run(body)
 
 
+# The rank layouts of the reference's own adjoint test (tests/primitives/test_repartition.py:11-127):
+# (P_x ranks, P_x shape, P_y ranks, P_y shape, world size), global tensor [77, 55].
+REFERENCE_LAYOUTS = {
+    "distributed-overlap": (range(4, 8), [4, 1], range(0, 12), [3, 4], 12),
+    "distributed-disjoint": (range(0, 4), [4, 1], range(4, 16), [3, 4], 16),
+    "distributed-disjoint-inactive": (range(0, 4), [4, 1], range(5, 17), [3, 4], 17),
+    "sequential-identity": (range(0, 1), [1, 1], range(0, 1), [1, 1], 1),
+    "as_scatter-overlap": (range(4, 5), [1, 1], range(0, 12), [3, 4], 12),
+    "as_scatter-disjoint": (range(0, 1), [1, 1], range(1, 13), [3, 4], 13),
+    "as_scatter-disjoint-inactive": (range(0, 1), [1, 1], range(2, 14), [3, 4], 14),
+    "as_gather-overlap": (range(0, 12), [3, 4], range(4, 5), [1, 1], 12),
+    "as_gather-disjoint": (range(1, 13), [3, 4], range(0, 1), [1, 1], 13),
+    "as_gather-disjoint-inactive": (range(2, 14), [3, 4], range(0, 1), [1, 1], 14),
+}
+
+
+def _shard_bounds(extent, parts, balanced):
+    """[start, stop) of every part of one dimension: the balanced split, or the
+    reference test's unbalanced one (part 0 takes the whole remainder,
+    test_repartition.py:176-181)."""
+    q, r = divmod(extent, parts)
+    sizes = [q + (1 if i < r else 0) for i in range(parts)] if balanced else [q + (r if i == 0 else 0) for i in range(parts)]
+    starts = np.concatenate([[0], np.cumsum(sizes)])
+    return [(int(starts[i]), int(starts[i + 1])) for i in range(parts)]
+
+
+@pytest.mark.parametrize("balanced", [True, False])
+@pytest.mark.parametrize("layout", list(REFERENCE_LAYOUTS))
+def test_repartition_reference_adjoint_layouts(layout, balanced):
+    """The reference's test_repartition_adjoint on its own parametrisation:
+    overlapping, disjoint and partly idle teams; scatter and gather shapes;
+    balanced input shards and the unbalanced ones the reference feeds it.
+    Checked three ways: y is the balanced split of the global tensor the x
+    shards form, dx the x-shaped split of the global dy (both exact), and the
+    reference's own criterion <F x, dy> = <x, F* dy>."""
+    P_x_ranks, P_x_shape, P_y_ranks, P_y_shape, world = REFERENCE_LAYOUTS[layout]
+    shape = [77, 55]
+    gen = torch.Generator().manual_seed(len(layout) * 2 + balanced)
+    gx, gdy = torch.randn(*shape, generator=gen), torch.randn(*shape, generator=gen)
+    xb = [_shard_bounds(shape[d], P_x_shape[d], balanced) for d in range(2)]
+    yb = [_shard_bounds(shape[d], P_y_shape[d], True) for d in range(2)]
+
+    def split(t, bounds, pshape):
+        return [t[bounds[0][i][0]:bounds[0][i][1], bounds[1][j][0]:bounds[1][j][1]].contiguous()
+                for i in range(pshape[0]) for j in range(pshape[1])]       # row-major rank order
+    xs, dys = split(gx, xb, P_x_shape), split(gdy, yb, P_y_shape)
+    want_y, want_dx = split(gx, yb, P_y_shape), split(gdy, xb, P_x_shape)
+    res = _run_repartition_world(world, list(P_x_ranks), P_x_shape, list(P_y_ranks), P_y_shape, xs, dys, torch.float32)
+    ipx = ipy = 0.0
+    seen_x, seen_y = set(), set()
+    for xr, yr, y, dx, layer in res:
+        if yr is not None:
+            assert torch.equal(y, want_y[yr])
+            ipy += float((y.double() * dys[yr].double()).sum())
+            seen_y.add(yr)
+        else:
+            assert y.numel() == 0
+        if xr is not None:
+            assert torch.equal(dx, want_dx[xr])
+            ipx += float((xs[xr].double() * dx.double()).sum())
+            seen_x.add(xr)
+    assert len(seen_x) == len(xs) and len(seen_y) == len(dys)
+    d = max(float(gx.norm() * gdy.norm()), 1e-30)
+    assert np.isclose(ipx / d, ipy / d)
+
+
 def test_repartition_layer_golden_example(golden):
     g = golden("repartition_7x5.json")
     xs = [torch.tensor(a) for a in g["input_by_x_rank"]]

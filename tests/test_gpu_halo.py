@@ -83,6 +83,42 @@ def test_halo_exchange_layer_matches_oracle(P, gshape, kernel):
         assert np.array_equal(dx.numpy(), want_dx[idx])        # one add per element: bit-exact in fp32
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("P,gshape,kernel,stride", [((1, 1, 3, 3), [1, 1, 10, 7], [3, 3], [1, 1]),
+                                                    ((1, 1, 3), [1, 1, 10], [2], [2])])
+def test_halo_exchange_reference_adjoint_cases(P, gshape, kernel, stride, dtype):
+    """The reference's test_halo_exchange_adjoint on its own parametrisation
+    (tests/primitives/test_halo_exchange.py:24-88: 3 x 3 workers on [1,1,10,7]
+    with a 3 x 3 kernel, 3 workers on [1,1,10] with kernel 2 / stride 2, each
+    in float32 and float64): shards zero-padded by their halos, forward and
+    adjoint against the oracle, and the reference's criterion
+    <F x, dy> = <x, F* dy> over all workers."""
+    nf = len(kernel)
+    halo, recv, send = _world_geometry(P, gshape, kernel, stride, [1] * nf)
+    gen = torch.Generator().manual_seed(43 + nf)
+    order = pm.indices(P)
+    padded, dys = {}, {}
+    for idx in order:
+        local = torch.randn(pm.subshape(P, idx, gshape), generator=gen, dtype=dtype)
+        pad = [w for a, b in reversed(halo[idx]) for w in (a, b)]
+        padded[idx] = torch.nn.functional.pad(local, pad)
+        dys[idx] = torch.randn(padded[idx].shape, generator=gen, dtype=dtype)
+    res = _run_halo_world(P, [padded[i] for i in order], [dys[i] for i in order], halo, recv, send)
+    want_y = o_halo.forward_all({i: padded[i].numpy() for i in order}, P, recv, send)
+    want_dx = o_halo.adjoint_all({i: dys[i].numpy() for i in order}, P, recv, send)
+    ipx = ipy = nx = ny = 0.0
+    for idx, (y, dx, layer) in zip(order, res):
+        assert y.dtype == dtype and dx.dtype == dtype
+        assert np.array_equal(y.numpy(), want_y[idx])
+        assert np.array_equal(dx.numpy(), want_dx[idx])
+        ipx += float((padded[idx].double() * dx.double()).sum())
+        ipy += float((y.double() * dys[idx].double()).sum())
+        nx += float(padded[idx].double().pow(2).sum())
+        ny += float(dys[idx].double().pow(2).sum())
+    d = max(np.sqrt(nx) * np.sqrt(ny), 1e-30)
+    assert np.isclose(ipx / d, ipy / d)
+
+
 # ------------------------------------------------------------ fused kernel --
 
 @pytest.fixture(params=["rows", "lines", "default"])
