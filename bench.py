@@ -250,6 +250,15 @@ def build_repartition(torch, lib, _lib, nsets):
     return steps, keep, 268435456
 
 
+def _build_repartition_half(which):
+    def build(torch, lib, _lib, nsets):
+        """Config 2's pack (or unpack) alone, one launch per step: the two
+        halves of the headline step timed separately."""
+        steps, keep, _ = build_repartition(torch, lib, _lib, nsets)
+        return [[fns[which]] for fns in steps], keep, 134217728
+    return build
+
+
 def layer_repartition(torch):
     layer, x = repartition_layer(torch)
     rec = time_layer(torch, lambda: layer(x))
@@ -916,6 +925,8 @@ def _build_mfma_probe(instruction, random):
 #          layer timer, cpu baseline, BASELINE.json configuration number)
 WORKLOADS = {
     "repartition": (build_repartition, 8, 2, "hbm", "mean", layer_repartition, cpu_repartition, 2),
+    "repartition_pack": (_build_repartition_half(0), 8, 1, "hbm", None, None, None, None),
+    "repartition_unpack": (_build_repartition_half(1), 8, 1, "hbm", None, None, None, None),
     "layernorm": (build_layernorm, 64, 2, "hbm", "mean", layer_layernorm, cpu_layernorm, 1),
     "layernorm_joined": (build_layernorm_joined, 64, 1, "hbm", None, None, None, None),
     "layernorm_long": (build_layernorm_long, 3, 2, "hbm", None, None, None, None),
