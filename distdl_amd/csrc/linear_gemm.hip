@@ -354,8 +354,13 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
         request_unit(w_kind, buf_w, base_w, off_gw, step_w, 1, 2 * kUnitBytes);
         request_unit(x_kind, buf_x, base_x, off_gx, step_x, 1, 3 * kUnitBytes);
     }
-    // Tile 0 complete and visible, then its first fragments.
-    __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+    // Tile 0 complete and visible, then its first fragments.  The requests of
+    // tile 1 (the last JW_W + JW_X of this wavefront, when they went out as
+    // requests) may stay in flight: the wait in the middle of k-tile 0 covers them.
+    if (full_tiles > 1)
+        __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(JW_W + JW_X));
+    else
+        __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 #pragma unroll
