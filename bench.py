@@ -776,13 +776,12 @@ def cpu_halo(budget_s=4.0):
 # backward (adjoint) workloads: the same shapes as the forward configurations
 # ----------------------------------------------------------------------------
 
-def build_layernorm_bwd(torch, lib, _lib, nsets):
+def build_layernorm_bwd(torch, lib, _lib, nsets, rows=16 * 512, cols=256, nparts=4):
     """Backward of config 1 on rank 0 as the layer runs it when every gradient
     is wanted: row sums + partial column sums in one launch, then (after the
     gather of the row sums) input gradient + final parameter sums in one launch.
     Algorithmic bytes: dy and x are read twice (once per launch), dx is written
     once: 5 x 8 388 608 B, plus the small vectors and the partial column sums."""
-    rows, cols = 16 * 512, 256
     keep, steps = [], []
     for s in range(nsets):
         gen = torch.Generator(device="cuda").manual_seed(4001 + s)
@@ -791,7 +790,7 @@ def build_layernorm_bwd(torch, lib, _lib, nsets):
         gamma = 1 + 0.1 * torch.randn(cols, generator=gen, device="cuda")
         mean = 0.01 * torch.randn(rows, generator=gen, device="cuda")
         rstd = 1 + 0.01 * torch.randn(rows, generator=gen, device="cuda")
-        sums = torch.zeros(4, rows, 2, device="cuda")                     # slot 0 is written by the kernel, 1..3 seeded
+        sums = torch.zeros(nparts, rows, 2, device="cuda")                # slot 0 is written by the kernel, the others seeded
         dx = torch.empty_like(x)
         dg, db = torch.empty(cols, device="cuda"), torch.empty(cols, device="cuda")
         work = torch.empty(2 * 256 * cols, device="cuda")
@@ -799,11 +798,45 @@ def build_layernorm_bwd(torch, lib, _lib, nsets):
         a1 = (dy.data_ptr(), x.data_ptr(), rows, cols, cols, cols, mean.data_ptr(), rstd.data_ptr(), gamma.data_ptr(),
               sums.data_ptr(), work.data_ptr(), work.numel())
         a2 = (dy.data_ptr(), x.data_ptr(), rows, cols, cols, cols, mean.data_ptr(), rstd.data_ptr(), gamma.data_ptr(),
-              sums.data_ptr(), 4, 1.0 / (4 * cols), dx.data_ptr(), cols, work.data_ptr(), work.numel(), dg.data_ptr(),
+              sums.data_ptr(), nparts, 1.0 / (nparts * cols), dx.data_ptr(), cols, work.data_ptr(), work.numel(), dg.data_ptr(),
               db.data_ptr())
         steps.append([_call(lib, _lib, "ddl_ln_bwd_partial_params_f32", a1),
                       _call(lib, _lib, "ddl_ln_bwd_input_params_f32", a2)])
-    return steps, keep, 5 * rows * cols * 4 + 2 * (2 * rows * 4) + 5 * rows * 2 * 4 + 3 * cols * 4 + 2 * (2 * 256 * cols * 4)
+    return steps, keep, 5 * rows * cols * 4 + 2 * (2 * rows * 4) + (nparts + 1) * rows * 2 * 4 + 3 * cols * 4 + 2 * (2 * 256 * cols * 4)
+
+
+def build_layernorm_local_bwd_two_passes(torch, lib, _lib, nsets):
+    """The two-launch backward on rows held whole ([8192, 1024] fp32), beside
+    layernorm_local_bwd: dy and x read twice."""
+    return build_layernorm_bwd(torch, lib, _lib, nsets, 16 * 512, 1024, 1)
+
+
+def _build_layernorm_bwd_one_pass(rows, cols, nparts):
+    def build(torch, lib, _lib, nsets):
+        """LayerNorm backward with one pass over dy and x (ddl_ln_bwd_one_pass:
+        row sums, dx and partial column sums in one launch, the final parameter
+        sums in a second, small one): rows held whole (nparts 1) or the other
+        workers' row sums seeded.  `work` is what is moved: dy and x read once,
+        dx written, plus the small vectors and the partial column sums."""
+        keep, steps = [], []
+        for s in range(nsets):
+            gen = torch.Generator(device="cuda").manual_seed(4101 + s)
+            x = torch.randn(rows, cols, generator=gen, device="cuda")
+            dy = torch.randn(rows, cols, generator=gen, device="cuda")
+            gamma = 1 + 0.1 * torch.randn(cols, generator=gen, device="cuda")
+            mean = 0.01 * torch.randn(rows, generator=gen, device="cuda")
+            rstd = 1 + 0.01 * torch.randn(rows, generator=gen, device="cuda")
+            sums = torch.zeros(nparts, rows, 2, device="cuda")
+            dx = torch.empty_like(x)
+            dg, db = torch.empty(cols, device="cuda"), torch.empty(cols, device="cuda")
+            work = torch.empty(2 * 256 * cols, device="cuda")
+            keep.append((x, dy, gamma, mean, rstd, sums, dx, dg, db, work))
+            args = (dy.data_ptr(), x.data_ptr(), _lib.DDL_DT_F32, rows, cols, cols, cols, mean.data_ptr(), rstd.data_ptr(),
+                    gamma.data_ptr(), sums.data_ptr(), nparts, 0, 1.0 / (nparts * cols), dx.data_ptr(), cols, work.data_ptr(),
+                    work.numel(), dg.data_ptr(), db.data_ptr())
+            steps.append([_call(lib, _lib, "ddl_ln_bwd_one_pass", args)])
+        return steps, keep, 3 * rows * cols * 4 + 2 * rows * 4 + (nparts + 1) * rows * 2 * 4 + 3 * cols * 4 + 2 * (2 * 256 * cols * 4)
+    return build
 
 
 def build_embedding_bwd(torch, lib, _lib, nsets):
@@ -939,6 +972,8 @@ WORKLOADS = {
     "halo_slabs": (build_halo_slabs, 8, 6, "hbm", None, None, None, None),
     "halo_slabs_interior": (build_halo_slabs_interior, 8, 6, "hbm", None, None, None, None),
     "layernorm_bwd": (build_layernorm_bwd, 32, 2, "hbm", None, None, None, None),
+    "layernorm_bwd_one_pass": (_build_layernorm_bwd_one_pass(16 * 512, 256, 4), 32, 2, "hbm", None, None, None, None),
+    "layernorm_local_bwd": (_build_layernorm_bwd_one_pass(16 * 512, 1024, 1), 8, 2, "hbm", None, None, None, None),
     "embedding_bwd": (build_embedding_bwd, 4, 1, "hbm", None, None, None, None),
     "linear_bwd": (_build_linear_bwd(True), 2, 1, "mfma", None, None, None, None),
     "linear_f32": (_build_linear_f32(False), 2, 1, "mfma_f32", None, None, None, None),
@@ -949,12 +984,13 @@ WORKLOADS = {
     "mfma_16x16x32_constant": (_build_mfma_probe(1, 0), 1, 1, "mfma", None, None, None, None),
     "mfma_16x16x32_random": (_build_mfma_probe(1, 1), 1, 1, "mfma", None, None, None, None),
     # only with --only:
+    "layernorm_local_bwd_two_passes": (build_layernorm_local_bwd_two_passes, 8, 2, "hbm", None, None, None, None),
     "linear_library": (build_linear_library, 4, 1, "mfma", None, None, None, None),
     "linear_bwd_transposed": (_build_linear_bwd(False), 2, 1, "mfma", None, None, None, None),
     "linear_f32_library": (_build_linear_f32(True), 2, 1, "mfma_f32", None, None, None, None),
     "calib": (build_calib, 4, 1, "hbm", None, None, None, None),
 }
-ONLY_ON_REQUEST = ("linear_library", "linear_bwd_transposed", "linear_f32_library", "calib")
+ONLY_ON_REQUEST = ("layernorm_local_bwd_two_passes", "linear_library", "linear_bwd_transposed", "linear_f32_library", "calib")
 
 
 def cpu_host():

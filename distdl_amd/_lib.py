@@ -87,6 +87,9 @@ SIGNATURES = {
     "ddl_ln_bwd_input_params": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
                                         c_void_p, c_void_p, c_int, c_float, c_void_p, c_int64, c_void_p, c_int64,
                                         c_void_p, c_void_p, c_void_p]),
+    "ddl_ln_bwd_one_pass": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
+                                    c_void_p, c_int, c_int, c_float, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p,
+                                    c_void_p]),
     "ddl_ln_bwd_partial_f32": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
                                        c_void_p, c_void_p]),
     "ddl_ln_bwd_input_f32": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,

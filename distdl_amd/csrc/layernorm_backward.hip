@@ -73,6 +73,17 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_partial(const T* __restrict__ d
     if (lane == 0) reinterpret_cast<float2*>(sums)[r] = make_float2(s1, s2);
 }
 
+// One element of dx = rstd (g - (S1 + xhat S2)), S already times a_p.  Every
+// kernel that writes dx goes through this one sequence of roundings (no
+// contraction left to the compiler), so they agree bit for bit.
+__device__ inline float dx_value(float dyv, float gv, float xv, float m, float rs, float S1, float S2) {
+#pragma clang fp contract(off)
+    const float h = (xv - m) * rs;
+    const float t = __builtin_fmaf(h, S2, S1);
+    const float q = dyv * gv - t;
+    return rs * q;
+}
+
 template <typename T, bool VEC>
 __device__ inline void ln_bwd_input_body(uint32_t block, const T* __restrict__ dy, const T* __restrict__ x, int64_t rows,
                                          int64_t cols, int64_t ld_dy, int64_t ld_x, const float* __restrict__ mean,
@@ -101,16 +112,15 @@ __device__ inline void ln_bwd_input_body(uint32_t block, const T* __restrict__ d
             float4 g = make_float4(1.f, 1.f, 1.f, 1.f);
             if (gamma) g = load4(gamma + c);
             float4 o;
-            o.x = rs * (d.x * g.x - (S1 + ((v.x - m) * rs) * S2));
-            o.y = rs * (d.y * g.y - (S1 + ((v.y - m) * rs) * S2));
-            o.z = rs * (d.z * g.z - (S1 + ((v.z - m) * rs) * S2));
-            o.w = rs * (d.w * g.w - (S1 + ((v.w - m) * rs) * S2));
+            o.x = dx_value(d.x, g.x, v.x, m, rs, S1, S2);
+            o.y = dx_value(d.y, g.y, v.y, m, rs, S1, S2);
+            o.z = dx_value(d.z, g.z, v.z, m, rs, S1, S2);
+            o.w = dx_value(d.w, g.w, v.w, m, rs, S1, S2);
             store4(dxr + c, o);   // dx is not read again here: streaming store
         }
     } else {
         for (int64_t c = lane; c < cols; c += kWave) {
-            const float g = load1(dyr + c) * (gamma ? load1(gamma + c) : 1.f);
-            store1(dxr + c, rs * (g - (S1 + ((load1(xr + c) - m) * rs) * S2)));
+            store1(dxr + c, dx_value(load1(dyr + c), gamma ? load1(gamma + c) : 1.f, load1(xr + c), m, rs, S1, S2));
         }
     }
 }
@@ -159,9 +169,11 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_params_partial(const T* __restr
 }
 
 // Workgroup per 64-column strip: lane group g = t / 64 adds the splits g, g+4,
-// ... of column t % 64 (independent loads, eight in flight), LDS folds the four
+// ... of column t % 64 (independent loads, kInFlight of them requested together:
+// many when this is all a kernel does, few when it shares its registers with
+// the dx pass), LDS folds the four
 // groups.
-template <typename T>
+template <typename T, int kInFlight>
 __device__ inline void ln_bwd_params_final_body(uint32_t block, const float* __restrict__ partial, int64_t cols, int splits,
                                                 T* __restrict__ dgamma, T* __restrict__ dbeta) {
     __shared__ float fold[2][kWavesPerBlock][kStrip];
@@ -170,15 +182,15 @@ __device__ inline void ln_bwd_params_final_body(uint32_t block, const float* __r
     float a = 0.f, b = 0.f;
     if (c < cols) {
         int k = g;
-        for (; k + 7 * kWavesPerBlock < splits; k += 8 * kWavesPerBlock) {
-            float va[8], vb[8];
+        for (; k + (kInFlight - 1) * kWavesPerBlock < splits; k += kInFlight * kWavesPerBlock) {
+            float va[kInFlight], vb[kInFlight];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
+            for (int u = 0; u < kInFlight; ++u) {
                 va[u] = partial[(static_cast<int64_t>(k + u * kWavesPerBlock) * 2) * cols + c];
                 vb[u] = partial[(static_cast<int64_t>(k + u * kWavesPerBlock) * 2 + 1) * cols + c];
             }
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
+            for (int u = 0; u < kInFlight; ++u) {
                 a += va[u];
                 b += vb[u];
             }
@@ -204,7 +216,7 @@ __device__ inline void ln_bwd_params_final_body(uint32_t block, const float* __r
 template <typename T>
 __global__ __launch_bounds__(kBlock) void ln_bwd_params_final(const float* __restrict__ partial, int64_t cols, int splits,
                                                               T* __restrict__ dgamma, T* __restrict__ dbeta) {
-    ln_bwd_params_final_body<T>(blockIdx.x, partial, cols, splits, dgamma, dbeta);
+    ln_bwd_params_final_body<T, 32>(blockIdx.x, partial, cols, splits, dgamma, dbeta);
 }
 
 // dx and the final parameter sums in one launch: the first final_blocks
@@ -220,7 +232,7 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_input_final(const T* __restrict
                                                              uint32_t final_blocks, const float* __restrict__ partial, int splits,
                                                              T* __restrict__ dgamma, T* __restrict__ dbeta) {
     if (blockIdx.x < final_blocks)
-        ln_bwd_params_final_body<T>(blockIdx.x, partial, cols, splits, dgamma, dbeta);
+        ln_bwd_params_final_body<T, 8>(blockIdx.x, partial, cols, splits, dgamma, dbeta);
     else
         ln_bwd_input_body<T, VEC>(blockIdx.x - final_blocks, dy, x, rows, cols, ld_dy, ld_x, mean, rstd, gamma, part_sums, nparts,
                                weight, dx, ld_dx);
@@ -229,16 +241,30 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_input_final(const T* __restrict
 constexpr int kFusedBlock = 512;   // eight wavefronts: a split of 32 rows is one round of four rows per wavefront
 constexpr int kFusedWaves = kFusedBlock / kWave;
 
+// What ln_bwd_partial_cols<.., true> needs beyond the sums: the other workers'
+// row sums (already in memory), this worker's place among them, and where dx goes.
+struct DxArgs {
+    const float* part_sums;   // [nparts][rows][2]; slot my_part is not read
+    int nparts, my_part;
+    float weight;
+    void* dx;
+    int64_t ld_dx;
+};
+
 // Row sums {sum g, sum g xhat} and the partial column sums of a row split in one
 // pass over dy and x: workgroup = split, its wavefronts take every eighth row
 // and each lane keeps the columns (lane + 64 k) * 4 .. + 3, k < NV, in registers.
-// partial has the layout of ln_bwd_params_partial.
-template <typename T, int NV>
+// partial has the layout of ln_bwd_params_partial.  WITH_DX: the sums of the
+// whole row are complete once this worker's are (it holds the row whole, or the
+// other workers' pairs are in memory), so dx is written in the same pass, from
+// the registers that hold the row.
+template <typename T, int NV, bool WITH_DX>
 __global__ __launch_bounds__(kFusedBlock) void ln_bwd_partial_cols(const T* __restrict__ dy, const T* __restrict__ x, int64_t rows,
                                                               int64_t cols, int64_t ld_dy, int64_t ld_x,
                                                               const float* __restrict__ mean, const float* __restrict__ rstd,
                                                               const T* __restrict__ gamma, float* __restrict__ sums,
-                                                              int64_t rows_per_split, float* __restrict__ partial) {
+                                                              int64_t rows_per_split, float* __restrict__ partial, const DxArgs dxa) {
+#pragma clang fp contract(off)   // both instantiations round alike: sums, column sums and dx do not depend on WITH_DX
     __shared__ float fold[2][kFusedWaves][NV * kWave * 4];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int nv = static_cast<int>(cols >> 2);
@@ -290,7 +316,31 @@ __global__ __launch_bounds__(kFusedBlock) void ln_bwd_partial_cols(const T* __re
             }
             s1 = wave_sum(s1);
             s2 = wave_sum(s2);
-            if (lane == 0) reinterpret_cast<float2*>(sums)[r] = make_float2(s1, s2);
+            if (lane == 0 && sums) reinterpret_cast<float2*>(sums)[r] = make_float2(s1, s2);
+            if (WITH_DX) {
+                // the pairs of all workers of this row, one worker per lane (at most 64 workers)
+                float p1 = 0.f, p2 = 0.f;
+                if (lane == dxa.my_part) {
+                    p1 = s1, p2 = s2;
+                } else if (lane < dxa.nparts) {
+                    const float2 o = reinterpret_cast<const float2*>(dxa.part_sums)[static_cast<int64_t>(lane) * rows + r];
+                    p1 = o.x, p2 = o.y;
+                }
+                const float S1 = wave_sum(p1) * dxa.weight, S2 = wave_sum(p2) * dxa.weight;
+                T* dxr = static_cast<T*>(dxa.dx) + r * dxa.ld_dx;
+#pragma unroll
+                for (int k = 0; k < NV; ++k) {
+                    const int c = lane + k * kWave;
+                    if (c >= nv) continue;
+                    const float4 dd = d[u][k], vv = v[u][k];
+                    float4 o;
+                    o.x = dx_value(dd.x, g[k].x, vv.x, m[u], rs[u], S1, S2);
+                    o.y = dx_value(dd.y, g[k].y, vv.y, m[u], rs[u], S1, S2);
+                    o.z = dx_value(dd.z, g[k].z, vv.z, m[u], rs[u], S1, S2);
+                    o.w = dx_value(dd.w, g[k].w, vv.w, m[u], rs[u], S1, S2);
+                    store4(dxr + 4 * c, o);
+                }
+            }
         }
     }
 #pragma unroll
@@ -456,11 +506,11 @@ extern "C" int ddl_ln_bwd_partial_params(const void* dy, const void* x, int dtyp
         with_ln_element(dtype, [&](auto* tag) {
             using T = std::remove_pointer_t<decltype(tag)>;
             if (cols <= kWave * 4)
-                hipLaunchKernelGGL((ln_bwd_partial_cols<T, 1>), grid, dim3(kFusedBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd, as<T>(gamma), sums, rows_per_split, workspace);
+                hipLaunchKernelGGL((ln_bwd_partial_cols<T, 1, false>), grid, dim3(kFusedBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd, as<T>(gamma), sums, rows_per_split, workspace, DxArgs{});
             else if (cols <= 2 * kWave * 4)
-                hipLaunchKernelGGL((ln_bwd_partial_cols<T, 2>), grid, dim3(kFusedBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd, as<T>(gamma), sums, rows_per_split, workspace);
+                hipLaunchKernelGGL((ln_bwd_partial_cols<T, 2, false>), grid, dim3(kFusedBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd, as<T>(gamma), sums, rows_per_split, workspace, DxArgs{});
             else
-                hipLaunchKernelGGL((ln_bwd_partial_cols<T, 4>), grid, dim3(kFusedBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd, as<T>(gamma), sums, rows_per_split, workspace);
+                hipLaunchKernelGGL((ln_bwd_partial_cols<T, 4, false>), grid, dim3(kFusedBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd, as<T>(gamma), sums, rows_per_split, workspace, DxArgs{});
         });
         return check_launch("ln_bwd_partial_cols");
     }
@@ -513,6 +563,54 @@ extern "C" int ddl_ln_bwd_input_params(const void* dy, const void* x, int dtype,
                                static_cast<int>(splits), as<T>(dgamma), as<T>(dbeta));
     });
     return check_launch("ln_bwd_input_final");
+}
+
+extern "C" int ddl_ln_bwd_one_pass(const void* dy, const void* x, int dtype, int64_t rows, int64_t cols, int64_t ld_dy, int64_t ld_x,
+                                   const float* mean, const float* rstd, const void* gamma, float* part_sums, int nparts, int my_part,
+                                   float weight, void* dx, int64_t ld_dx, float* workspace, int64_t workspace_elems, void* dgamma,
+                                   void* dbeta, void* stream) {
+    using namespace ddl;
+    const int elem = elem_bytes(dtype);
+    if (!elem) return fail(DDL_E_UNSUPP, "ln backward (one pass): dtype %d (f32, bf16, f16 only)", dtype);
+    if (int rc = check_rows("ln backward (one pass)", rows, cols, ld_dy, ld_x)) return rc;
+    if (ld_dx < cols) return fail(DDL_E_ARG, "ln backward (one pass): ld_dx=%lld below cols=%lld", (long long)ld_dx, (long long)cols);
+    if (nparts < 1 || nparts > kWave) return fail(DDL_E_UNSUPP, "ln backward (one pass): nparts=%d outside [1,%d]", nparts, kWave);
+    if (my_part < 0 || my_part >= nparts) return fail(DDL_E_ARG, "ln backward (one pass): my_part=%d outside [0,%d)", my_part, nparts);
+    if (nparts > 1 && !part_sums) return fail(DDL_E_ARG, "ln backward (one pass): the other workers' sums are missing");
+    if (!workspace) return fail(DDL_E_ARG, "ln backward (one pass): null workspace");
+    const int64_t splits = param_splits(rows, cols, workspace_elems);
+    if (splits < 1) return fail(DDL_E_ARG, "ln backward (one pass): workspace of %lld floats is smaller than 2 x %lld", (long long)workspace_elems, (long long)cols);
+    if (rows > 0 && (!dy || !x || !mean || !rstd || !dx)) return fail(DDL_E_ARG, "ln backward (one pass): null pointer");
+    if (!elems_aligned(elem, {dy, x, gamma, dx, dgamma, dbeta}) || !aligned_to(mean, 4) || !aligned_to(rstd, 4) || !aligned_to(part_sums, 8) ||
+        !aligned_to(workspace, 4))
+        return fail(DDL_E_ALIGN, "ln backward (one pass): elements must be aligned to their size, fp32 arrays to 4 bytes, the sums to 8");
+    if (cols > 4 * kWave * 4 || !vectorizable(elem, cols, {ld_dy, ld_x, ld_dx}, {dy, x, gamma, dx}))
+        return fail(DDL_E_UNSUPP, "ln backward (one pass): rows of at most %d columns, columns and pitches multiples of 4, pointers aligned to 4 elements", 4 * kWave * 4);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t strips = (dgamma || dbeta) ? (cols + kStrip - 1) / kStrip : 0;
+    if (rows > 0) {
+        const int64_t rows_per_split = (rows + splits - 1) / splits;
+        float* sums = part_sums ? part_sums + static_cast<int64_t>(my_part) * rows * 2 : nullptr;
+        const DxArgs dxa{part_sums, nparts, my_part, weight, dx, ld_dx};
+        const dim3 grid(static_cast<uint32_t>(splits));
+        with_ln_element(dtype, [&](auto* tag) {
+            using T = std::remove_pointer_t<decltype(tag)>;
+            if (cols <= kWave * 4)
+                hipLaunchKernelGGL((ln_bwd_partial_cols<T, 1, true>), grid, dim3(kFusedBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd, as<T>(gamma), sums, rows_per_split, workspace, dxa);
+            else if (cols <= 2 * kWave * 4)
+                hipLaunchKernelGGL((ln_bwd_partial_cols<T, 2, true>), grid, dim3(kFusedBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd, as<T>(gamma), sums, rows_per_split, workspace, dxa);
+            else
+                hipLaunchKernelGGL((ln_bwd_partial_cols<T, 4, true>), grid, dim3(kFusedBlock), 0, s, as<T>(dy), as<T>(x), rows, cols, ld_dy, ld_x, mean, rstd, as<T>(gamma), sums, rows_per_split, workspace, dxa);
+        });
+        if (int rc = check_launch("ln_bwd_partial_cols")) return rc;
+    }
+    if (strips == 0) return 0;
+    with_ln_element(dtype, [&](auto* tag) {
+        using T = std::remove_pointer_t<decltype(tag)>;
+        hipLaunchKernelGGL(ln_bwd_params_final<T>, dim3(static_cast<uint32_t>(strips)), dim3(kBlock), 0, s, workspace, cols,
+                           static_cast<int>(rows > 0 ? splits : 0), as<T>(dgamma), as<T>(dbeta));
+    });
+    return check_launch("ln_bwd_params_final");
 }
 
 // The float32 forms.

@@ -459,6 +459,44 @@ def ln_backward_input_params(dy2d, x2d, mean, rstd, gamma, part_sums, weight, wo
     return dx, dg, db
 
 
+def ln_backward_one_pass_supported(dy2d, x2d, gamma, nparts=1):
+    """Whether ``ln_backward_one_pass`` takes these rows: at most 64 workers,
+    rows of at most 1024 columns, columns and pitches multiples of 4, dy, x and
+    gamma aligned to four elements."""
+    rows, cols = x2d.shape
+    quad = 4 * x2d.element_size()
+    return (nparts <= 64 and cols <= 1024 and cols % 4 == 0 and
+            (rows <= 1 or (x2d.stride(0) % 4 == 0 and dy2d.stride(0) % 4 == 0)) and
+            x2d.data_ptr() % quad == 0 and dy2d.data_ptr() % quad == 0 and (gamma is None or gamma.data_ptr() % quad == 0))
+
+
+def ln_backward_one_pass(dy2d, x2d, mean, rstd, gamma, weight, part_sums=None, my_part=0, want_gamma=True, want_beta=True):
+    """dx, (dgamma, dbeta) and this worker's row sums in one pass over dy and
+    x: for rows this worker holds whole (``part_sums`` None) or whose other
+    workers' sums are in ``part_sums`` [P, rows, 2] beforehand (slot ``my_part``
+    is written).  Results as ``ln_backward_partial_params`` followed by
+    ``ln_backward_input_params``."""
+    _require_gpu(dy2d, x2d, mean, rstd, gamma, part_sums)
+    ld_dy, ld_x = _rows2d(dy2d, "ln_backward_one_pass"), _rows2d(x2d, "ln_backward_one_pass")
+    rows, cols = x2d.shape
+    nparts = 1
+    if part_sums is not None:
+        if part_sums.dtype != torch.float32 or part_sums.dim() != 3 or tuple(part_sums.shape[1:]) != (rows, 2) or \
+           not part_sums.is_contiguous():
+            raise ValueError(f"ln_backward_one_pass: part_sums must be contiguous fp32 [P, {rows}, 2]")
+        nparts = part_sums.shape[0]
+    dt = _ln_bwd_dtype("ln_backward_one_pass", dy2d, x2d, gamma)
+    work = _ln_param_workspace(rows, cols, x2d.device)
+    dx = torch.empty((rows, cols), dtype=x2d.dtype, device=x2d.device)
+    dg = torch.empty(cols, dtype=x2d.dtype, device=x2d.device) if want_gamma else None
+    db = torch.empty(cols, dtype=x2d.dtype, device=x2d.device) if want_beta else None
+    rc = _lib.load().ddl_ln_bwd_one_pass(dy2d.data_ptr(), x2d.data_ptr(), dt, rows, cols, ld_dy, ld_x, mean.data_ptr(),
+                                         rstd.data_ptr(), _ptr(gamma), _ptr(part_sums), nparts, int(my_part), float(weight),
+                                         dx.data_ptr(), cols, work.data_ptr(), work.numel(), _ptr(dg), _ptr(db), _stream())
+    _lib.check(rc, "ddl_ln_bwd_one_pass")
+    return dx, dg, db
+
+
 def embedding_gather(weight, ids, lo, hi, out=None):
     """out[t] = weight[ids[t] - lo] if lo <= ids[t] < hi else 0."""
     _require_gpu(weight, ids)

@@ -97,7 +97,12 @@ class _LayerNormShard(torch.autograd.Function):
         w_shape, b_shape = ctx.param_shapes
         want_w, want_b = need_w and w_shape is not None, need_b and b_shape is not None
         fused = need_x and (want_w or want_b)        # two launches instead of four
-        if need_x:
+        if need_x and ctx.nparts == 1 and hip_ops.ln_backward_one_pass_supported(dy2d, x2d, gamma):
+            # rows held whole: this worker's sums are the row's sums, so dx comes out of the pass that forms them
+            dx, dw, db = hip_ops.ln_backward_one_pass(dy2d, x2d, mean, rstd, gamma, 1.0 / ctx.cols, want_gamma=want_w,
+                                                      want_beta=want_b)
+            dx = dx.view(grad_output.shape)
+        elif need_x:
             if fused:
                 sums, work = hip_ops.ln_backward_partial_params(dy2d, x2d, mean, rstd, gamma)
             else:

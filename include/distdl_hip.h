@@ -334,6 +334,24 @@ int ddl_ln_bwd_input_params(const void* dy, const void* x, int dtype,
                             int nparts, float weight, void* dx, int64_t ld_dx,
                             const float* workspace, int64_t workspace_elems,
                             void* dgamma, void* dbeta, void* stream);
+/* dx, the row sums and the parameter gradients with ONE pass over dy and x, for
+ * a worker whose share of the row sums completes them: it holds its rows whole
+ * (nparts = 1, part_sums may be NULL: the backward of the reference's
+ * torch.nn.functional.layer_norm branch, nn/layernorm.py:310-319), or the
+ * other workers' pairs are in part_sums[nparts][rows][2] before the launch
+ * (slots p != my_part are read, slot my_part is written).  Results as
+ * ddl_ln_bwd_partial_params followed by ddl_ln_bwd_input_params; the second
+ * launch only adds up the partial column sums (none when dgamma and dbeta are
+ * both NULL).  workspace as above.  Limits: nparts <= 64, rows of at most 1024
+ * columns, columns and pitches multiples of 4, pointers aligned to 4 elements
+ * (else DDL_E_UNSUPP: take the two calls). */
+int ddl_ln_bwd_one_pass(const void* dy, const void* x, int dtype, int64_t rows,
+                        int64_t cols, int64_t ld_dy, int64_t ld_x,
+                        const float* mean, const float* rstd, const void* gamma,
+                        float* part_sums, int nparts, int my_part, float weight,
+                        void* dx, int64_t ld_dx, float* workspace,
+                        int64_t workspace_elems, void* dgamma, void* dbeta,
+                        void* stream);
 int ddl_ln_bwd_partial_params_f32(const float* dy, const float* x, int64_t rows,
                                   int64_t cols, int64_t ld_dy, int64_t ld_x,
                                   const float* mean, const float* rstd,

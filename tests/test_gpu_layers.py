@@ -416,6 +416,56 @@ def test_layernorm_backward_kernels_match_oracle(ops, cols, affine):
         dx3, dg3, db3 = ops.ln_backward_input_params(dy2d, x2d, mean, rstd, g, torch.stack(gathered).contiguous(),
                                                      1.0 / (P * cols[live]), work, want_gamma=False, want_beta=True)
         assert dg3 is None and torch.equal(db3, db2) and torch.equal(dx3, dx2)
+        # one pass over dy and x, the other workers' sums in memory beforehand: the same results, own sums written in place
+        table = torch.stack(gathered).contiguous()
+        if ops.ln_backward_one_pass_supported(dy2d, x2d, g, P):
+            poisoned = table.clone()
+            poisoned[live] = float("nan")
+            dx4, dg4, db4 = ops.ln_backward_one_pass(dy2d, x2d, mean, rstd, g, 1.0 / (P * cols[live]), poisoned, live)
+            torch.cuda.synchronize()
+            assert torch.equal(poisoned, table)
+            assert torch.equal(dx4, dx2) and torch.equal(dg4, dg2) and torch.equal(db4, db2)
+        else:
+            with pytest.raises(RuntimeError, match="code -5"):
+                ops.ln_backward_one_pass(dy2d, x2d, mean, rstd, g, 1.0 / (P * cols[live]), table.clone(), live)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 4), (37, 256), (300, 1024), (1000, 300), (5000, 64), (33, 1028)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_layer_norm_backward_of_whole_rows_in_one_pass(ops, rows, cols, dtype):
+    """Rows one worker holds whole (the backward of the reference's
+    F.layer_norm branch, nn/layernorm.py:319): dx, dgamma, dbeta from one pass
+    over dy and x against torch autograd in float64, and against the two
+    launches bit for bit."""
+    gen = torch.Generator().manual_seed(rows * 7 + cols)
+    x = (torch.randn(rows, cols, generator=gen) * 2 + 0.3).to(dtype)
+    dy = torch.randn(rows, cols, generator=gen).to(dtype)
+    gamma = (1 + 0.1 * torch.randn(cols, generator=gen)).to(dtype)
+    beta = (0.1 * torch.randn(cols, generator=gen)).to(dtype)
+    xg, dyg, gg, bg = x.cuda(), dy.cuda(), gamma.cuda(), beta.cuda()
+    _, mean, rstd = ops.layer_norm(xg, gg, bg, 1e-5, want_stats=True)
+    if not ops.ln_backward_one_pass_supported(dyg, xg, gg):
+        assert cols > 1024
+        with pytest.raises(RuntimeError, match="code -5"):
+            ops.ln_backward_one_pass(dyg, xg, mean, rstd, gg, 1.0 / cols)
+        return
+    dx, dg, db = ops.ln_backward_one_pass(dyg, xg, mean, rstd, gg, 1.0 / cols)
+    sums, work = ops.ln_backward_partial_params(dyg, xg, mean, rstd, gg)
+    dx2, dg2, db2 = ops.ln_backward_input_params(dyg, xg, mean, rstd, gg, sums.unsqueeze(0).contiguous(), 1.0 / cols, work)
+    torch.cuda.synchronize()
+    assert torch.equal(dx.view(torch.uint8), dx2.view(torch.uint8))
+    assert torch.equal(dg.view(torch.uint8), dg2.view(torch.uint8)) and torch.equal(db.view(torch.uint8), db2.view(torch.uint8))
+    xr = x.double().requires_grad_(True)
+    gr, br = gamma.double().requires_grad_(True), beta.double().requires_grad_(True)
+    F.layer_norm(xr, (cols,), gr, br, 1e-5).backward(dy.double())
+    tol = 1e-5 if dtype == torch.float32 else 2.0 ** -7
+    scale = max(1.0, float(xr.grad.abs().max()))
+    assert float((dx.cpu().double() - xr.grad).abs().max()) <= 4 * tol * scale
+    assert torch.allclose(dg.cpu().double(), gr.grad, rtol=10 * tol, atol=10 * tol * max(1.0, float(gr.grad.abs().max())))
+    assert torch.allclose(db.cpu().double(), br.grad, rtol=10 * tol, atol=10 * tol * max(1.0, float(br.grad.abs().max())))
+    # without parameter gradients: dx alone, no second launch
+    dx5, dg5, db5 = ops.ln_backward_one_pass(dyg, xg, mean, rstd, gg, 1.0 / cols, want_gamma=False, want_beta=False)
+    assert dg5 is None and db5 is None and torch.equal(dx5, dx)
 
 
 @pytest.mark.parametrize("dtype,ulp", [(torch.bfloat16, 2.0 ** -8), (torch.float16, 2.0 ** -11)])
