@@ -15,6 +15,7 @@ from .halo_exchange import HaloExchange  # noqa: F401
 from .layernorm import DistributedLayerNorm  # noqa: F401
 from .linear import DistributedLinear  # noqa: F401
 from .linear_ag import DistributedLinearAllGather  # noqa: F401
+from .linear_rs import DistributedLinearReduceScatter  # noqa: F401
 from .reduce_scatter import ReduceScatter  # noqa: F401
 from .module import Module  # noqa: F401
 from .repartition import Repartition  # noqa: F401
@@ -24,6 +25,6 @@ from .transpose import DistributedTranspose  # noqa: F401
 __all__ = [
     "AllGather", "AllSumReduce", "Broadcast", "DistributedConv1d", "DistributedConv2d", "DistributedConv3d",
     "DistributedFeatureConv1d", "DistributedFeatureConv2d", "DistributedFeatureConv3d", "DistributedEmbedding",
-    "HaloExchange", "DistributedLayerNorm", "DistributedLinear", "DistributedLinearAllGather", "Module", "ReduceScatter",
+    "HaloExchange", "DistributedLayerNorm", "DistributedLinear", "DistributedLinearAllGather", "DistributedLinearReduceScatter", "Module", "ReduceScatter",
     "Repartition", "SumReduce", "DistributedTranspose",
 ]

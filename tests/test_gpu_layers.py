@@ -1288,3 +1288,62 @@ def test_linear_layers_forward(ops):
         y3 = ag(x3.cuda())
     assert y3.shape == (2, 32, 128)
     _lin_check(bits16(y3), x3, ag.weight.detach().cpu().view(128, 256), ag.bias.detach().cpu().view(128))
+
+
+@pytest.mark.parametrize("P,use_bias", [([1, 1, 4], True), ([2, 1, 2], True), ([1, 1, 3], False)])
+def test_linear_reduce_scatter_layer_matches_torch(ops, P, use_bias):
+    """DistributedLinearReduceScatter over all workers (loopback): every worker
+    multiplies its slice of the input features by its weight shard, the partial
+    products are summed and scattered along the output features.  Forward and
+    backward against torch.nn.functional.linear on the whole tensors (float32,
+    the reference's default; reference: nn/linear_rs.py:361-364)."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedLinearReduceScatter
+    from oracle import repartition as o_rep
+    D, M = P[0], P[2]
+    n = D * M
+    batch, tokens, c_in, c_out = 2 * D, 5, 26, 21          # neither feature count divides evenly among 3 or 4 workers
+    gen = torch.Generator().manual_seed(sum(P) * 10 + use_bias)
+    x = torch.randn(batch, tokens, c_in, generator=gen)
+    w = 0.2 * torch.randn(c_out, c_in, generator=gen)
+    b = 0.2 * torch.randn(c_out, generator=gen) if use_bias else None
+    dy = torch.randn(batch, tokens, c_out, generator=gen)
+    xs = o_rep.scatter(x.numpy(), P)
+    dys = o_rep.scatter(dy.numpy(), P)
+    w_shards = o_rep.scatter(w.numpy().reshape(1, c_out, c_in), [1, 1, M])
+
+    def body(P_world):
+        P_x = P_world.create_partition_inclusive(list(range(n))).create_cartesian_topology_partition(P)
+        layer = DistributedLinearReduceScatter(P_x, c_in, c_out, bias=use_bias)
+        with torch.no_grad():
+            if layer.P_weight.active:
+                layer.weight.copy_(torch.from_numpy(w_shards[int(P_x.index[-1])]).view(layer.weight.shape))
+            if use_bias and layer.P_store_bias.active:
+                layer.bias.copy_(b.view(layer.bias.shape))
+        xin = torch.from_numpy(xs[P_x.rank]).cuda().requires_grad_(True)
+        y = layer(xin)
+        y.backward(torch.from_numpy(dys[P_x.rank]).cuda())
+        torch.cuda.synchronize()
+        dw = layer.weight.grad.cpu() if layer.P_weight.active else None
+        db = layer.bias.grad.cpu() if use_bias and layer.P_store_bias.active else None
+        return y.detach().cpu(), xin.grad.cpu(), dw, db, int(P_x.index[-1])
+
+    outs = SimWorld(n).run(body)
+    xr = x.clone().requires_grad_(True)
+    wr = w.clone().requires_grad_(True)
+    br = b.clone().requires_grad_(True) if use_bias else None
+    yr = F.linear(xr, wr, br)
+    yr.backward(dy)
+    want_y = o_rep.scatter(yr.detach().numpy(), P)
+    want_dx = o_rep.scatter(xr.grad.numpy(), P)
+    want_dw = o_rep.scatter(wr.grad.numpy().reshape(1, c_out, c_in), [1, 1, M])
+    seen_w = 0
+    for r, (y, dx, dw, db, col) in enumerate(outs):
+        assert np.allclose(y.numpy(), want_y[r], rtol=1e-5, atol=1e-5)
+        assert np.allclose(dx.numpy(), want_dx[r], rtol=1e-5, atol=1e-5)
+        if dw is not None:
+            seen_w += 1
+            assert np.allclose(dw.numpy().reshape(c_out, -1), want_dw[col].reshape(c_out, -1), rtol=1e-5, atol=1e-4)
+        if db is not None:
+            assert r == 0 and np.allclose(db.numpy().reshape(-1), br.grad.numpy(), rtol=1e-5, atol=1e-4)
+    assert seen_w == M
