@@ -94,6 +94,7 @@ class Timed:
         self.step_fns = launches_per_step      # list over buffer sets of [closures of one step]
         self.use_graph = use_graph
         self.graph = None
+        self.rest_graphs = {}
         self.mode = "stream"
 
     def _run_sets(self):
@@ -121,13 +122,39 @@ class Timed:
             self.graph = None
             torch.cuda.synchronize()
 
+    def _rest_graph(self, rest):
+        """A graph of the first `rest` buffer sets, for step counts that are no
+        multiple of the number of sets; captured (and replayed once) outside the
+        timed region.  None when capture is refused."""
+        torch = self.torch
+        if rest in self.rest_graphs:
+            return self.rest_graphs[rest]
+        graph = None
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                bind_stream(torch)
+                for fns in self.step_fns[:rest]:
+                    for fn in fns:
+                        fn()
+            graph.replay()
+            torch.cuda.synchronize()
+        except Exception as exc:
+            sys.stderr.write(f"[bench] capture of the {rest}-step remainder refused ({exc}); launching it on the stream\n")
+            graph = None
+            torch.cuda.synchronize()
+        self.rest_graphs[rest] = graph
+        return graph
+
     def run(self, steps):
         """Runs exactly `steps` steps: whole passes over the buffer sets (graph
-        replays when a graph was captured) and the remaining steps launched on
-        the stream.  Returns (steps, wall seconds, event seconds)."""
+        replays when a graph was captured) and the remaining steps from a
+        second, shorter graph (or launched on the stream when nothing could be
+        captured).  Returns (steps, wall seconds, event seconds)."""
         torch = self.torch
         nsets = len(self.step_fns)
         passes, rest = divmod(steps, nsets)
+        rest_graph = self._rest_graph(rest) if self.graph is not None and rest else None
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         bind_stream(torch)
@@ -138,9 +165,12 @@ class Timed:
                 self.graph.replay()
             else:
                 self._run_sets()
-        for fns in self.step_fns[:rest]:
-            for fn in fns:
-                fn()
+        if rest_graph is not None:
+            rest_graph.replay()
+        else:
+            for fns in self.step_fns[:rest]:
+                for fn in fns:
+                    fn()
         e1.record()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
