@@ -51,12 +51,6 @@ __device__ inline float4 affine4(float4 g, float4 o, float4 b) {
     return make_float4(g.x * o.x + b.x, g.y * o.y + b.y, g.z * o.z + b.z, g.w * o.w + b.w);
 }
 
-__device__ inline float wave_sum(float v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
-}
-
 // Sum over the workgroup, the same value in every thread.  `scratch` holds one
 // float per wavefront; the leading barrier lets it be reused call after call.
 __device__ inline float block_sum(float v, float* scratch) {

@@ -33,12 +33,6 @@ constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr int kStrip = 64;     // columns per workgroup of the parameter kernel
 
-__device__ inline float wave_sum(float v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
-}
-
 template <typename T, bool VEC>
 __global__ __launch_bounds__(kBlock) void ln_bwd_partial(const T* __restrict__ dy, const T* __restrict__ x, int64_t rows,
                                                          int64_t cols, int64_t ld_dy, int64_t ld_x,

@@ -19,6 +19,27 @@ __device__ inline uint32_t f32_to_bf16(float f) {
     return u >> 16;
 }
 
+// Sum over the 64 lanes of a wavefront, the same value in every lane.  Data
+// moves between lanes inside the vector ALU (DPP: pairs, quads, half rows and
+// rows of 16 lanes by mirroring, then lane 15 / 31 of the rows below broadcast
+// into the rows above), six dependent additions of a few cycles each; the
+// total ends in lane 63 and is read from there.  (A butterfly of __shfl_xor goes
+// through the LDS crossbar six times, about a hundred cycles each, which at
+// 8 MiB inputs was a tenth of a kernel's duration per reduction.)
+template <int CTRL, int ROW_MASK>
+__device__ inline float dpp_moved(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xF, false));
+}
+__device__ inline float wave_sum(float v) {
+    v += dpp_moved<0xB1, 0xF>(v);    // quad_perm [1,0,3,2]
+    v += dpp_moved<0x4E, 0xF>(v);    // quad_perm [2,3,0,1]
+    v += dpp_moved<0x141, 0xF>(v);   // row_half_mirror
+    v += dpp_moved<0x140, 0xF>(v);   // row_mirror: every lane holds the sum of its row of 16
+    v += dpp_moved<0x142, 0xA>(v);   // row_bcast15 into rows 1 and 3
+    v += dpp_moved<0x143, 0xC>(v);   // row_bcast31 into rows 2 and 3
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
 // Four consecutive elements as floats; what these kernels store is never read
 // again by them, so it leaves with streaming stores.
 __device__ inline float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
