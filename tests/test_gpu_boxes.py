@@ -294,6 +294,47 @@ def test_repartition_reference_adjoint_layouts(layout, balanced):
     assert np.isclose(ipx / d, ipy / d)
 
 
+@pytest.mark.parametrize("dtype,test_backward", [(torch.float32, True), (torch.int32, False), (torch.float64, True)])
+def test_repartition_reference_dtype_cases(dtype, test_backward):
+    """The reference's test_repartition_dtype (tests/primitives/test_repartition.py:428-546):
+    [77, 55] from a 4 x 1 to a 2 x 2 partition of the same four workers in
+    float32, int32 (no gradient) and float64; the output, and the gradient where
+    there is one, keep the dtype -- and here also the values."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import Repartition
+    shape, P_x_shape, P_y_shape = [77, 55], [4, 1], [2, 2]
+    gen = torch.Generator().manual_seed(17)
+    gx = (10 * torch.randn(*shape, generator=gen)).to(dtype)
+    gdy = (10 * torch.randn(*shape, generator=gen)).to(dtype)
+    xb = [_shard_bounds(shape[d], P_x_shape[d], True) for d in range(2)]
+    yb = [_shard_bounds(shape[d], P_y_shape[d], True) for d in range(2)]
+
+    def split(t, bounds, pshape):
+        return [t[bounds[0][i][0]:bounds[0][i][1], bounds[1][j][0]:bounds[1][j][1]].contiguous()
+                for i in range(pshape[0]) for j in range(pshape[1])]
+    xs, dys = split(gx, xb, P_x_shape), split(gdy, yb, P_y_shape)
+    want_y, want_dx = split(gx, yb, P_y_shape), split(gdy, xb, P_x_shape)
+
+    def body(P_world):
+        P_x = P_world.create_partition_inclusive([0, 1, 2, 3]).create_cartesian_topology_partition(P_x_shape)
+        P_y = P_world.create_partition_inclusive([0, 1, 2, 3]).create_cartesian_topology_partition(P_y_shape)
+        layer = Repartition(P_x, P_y, preserve_batch=False)
+        x = xs[P_x.rank].cuda()
+        x.requires_grad = test_backward
+        y = layer(x)
+        dx = None
+        if test_backward:
+            y.backward(dys[P_y.rank].cuda())
+            dx = x.grad.cpu()
+        torch.cuda.synchronize()
+        return P_x.rank, P_y.rank, y.detach().cpu(), dx
+
+    for xr, yr, y, dx in SimWorld(4).run(body):
+        assert y.dtype == dtype and torch.equal(y, want_y[yr])
+        if test_backward:
+            assert dx.dtype == dtype and torch.equal(dx, want_dx[xr])
+
+
 def test_repartition_layer_golden_example(golden):
     g = golden("repartition_7x5.json")
     xs = [torch.tensor(a) for a in g["input_by_x_rank"]]
