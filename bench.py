@@ -1087,6 +1087,9 @@ def main():
                          "traffic_source": f"profiles/{name}_hbm_traffic_pmc.txt (earlier rocprofv3 --pmc runs, not this run)"
                          if traffic is not None else None},
         }
+        if name == "layernorm_joined":
+            # the same step counted with config 1's algorithmic bytes (x read by both halves), for comparison with `layernorm`
+            results[name]["roofline"]["frac_of_config1_bytes"] = 25298944 / (m["launch_s"] * launches) / 1e9 / HBM_PEAK_GBS
         del step_fns, keep
         torch.cuda.empty_cache()
         if layer_fn is not None and not args.skip_layers:
