@@ -95,12 +95,42 @@ __device__ inline void ln_bwd_input_body(uint32_t block, const T* __restrict__ d
         p2 += s.y;
     }
     const float m = mean[r], rs = rstd[r];
-    const float S1 = wave_sum(p1) * weight, S2 = wave_sum(p2) * weight;   // already times a_p
     const T* dyr = dy + r * ld_dy;
     const T* xr = x + r * ld_x;
     T* dxr = dx + r * ld_dx;
+    // The first kAhead pieces of the row are requested before the sums are
+    // reduced: the reduction waits for the gathered pairs, and the row should
+    // not wait behind it (one memory round trip instead of two for rows of up
+    // to 1024 columns).
+    constexpr int kAhead = 4;
+    float4 d0[kAhead], v0[kAhead], g0[kAhead];
     if (VEC) {
-        for (int64_t c = lane * 4; c < cols; c += kWave * 4) {
+#pragma unroll
+        for (int k = 0; k < kAhead; ++k) {
+            const int64_t c = lane * 4 + static_cast<int64_t>(k) * (kWave * 4);
+            g0[k] = make_float4(1.f, 1.f, 1.f, 1.f);
+            if (c < cols) {
+                d0[k] = load4(dyr + c);
+                v0[k] = load4(xr + c);
+                if (gamma) g0[k] = load4(gamma + c);
+            }
+        }
+    }
+    const float S1 = wave_sum(p1) * weight, S2 = wave_sum(p2) * weight;   // already times a_p
+    if (VEC) {
+#pragma unroll
+        for (int k = 0; k < kAhead; ++k) {
+            const int64_t c = lane * 4 + static_cast<int64_t>(k) * (kWave * 4);
+            if (c < cols) {
+                float4 o;
+                o.x = dx_value(d0[k].x, g0[k].x, v0[k].x, m, rs, S1, S2);
+                o.y = dx_value(d0[k].y, g0[k].y, v0[k].y, m, rs, S1, S2);
+                o.z = dx_value(d0[k].z, g0[k].z, v0[k].z, m, rs, S1, S2);
+                o.w = dx_value(d0[k].w, g0[k].w, v0[k].w, m, rs, S1, S2);
+                store4(dxr + c, o);
+            }
+        }
+        for (int64_t c = lane * 4 + static_cast<int64_t>(kAhead) * (kWave * 4); c < cols; c += kWave * 4) {
             const float4 d = load4(dyr + c);
             const float4 v = load4(xr + c);
             float4 g = make_float4(1.f, 1.f, 1.f, 1.f);
@@ -276,12 +306,16 @@ __global__ __launch_bounds__(kFusedBlock) void ln_bwd_partial_cols(const T* __re
     for (int64_t r0 = r_begin + wave; r0 < r_end; r0 += kFusedWaves * RU) {
         float m[RU], rs[RU];
         float4 d[RU][NV], v[RU][NV];
+        float2 peer[RU];   // WITH_DX: the pair of worker `lane` for this row, requested together with the row
 #pragma unroll
         for (int u = 0; u < RU; ++u) {
             const int64_t r = r0 + u * kFusedWaves;
             const bool on = r < r_end;
             m[u] = on ? mean[r] : 0.f;
             rs[u] = on ? rstd[r] : 0.f;
+            peer[u] = make_float2(0.f, 0.f);
+            if (WITH_DX && on && lane < dxa.nparts && lane != dxa.my_part)
+                peer[u] = reinterpret_cast<const float2*>(dxa.part_sums)[static_cast<int64_t>(lane) * rows + r];
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
                 const int c = lane + k * kWave;
@@ -313,13 +347,8 @@ __global__ __launch_bounds__(kFusedBlock) void ln_bwd_partial_cols(const T* __re
             if (lane == 0 && sums) reinterpret_cast<float2*>(sums)[r] = make_float2(s1, s2);
             if (WITH_DX) {
                 // the pairs of all workers of this row, one worker per lane (at most 64 workers)
-                float p1 = 0.f, p2 = 0.f;
-                if (lane == dxa.my_part) {
-                    p1 = s1, p2 = s2;
-                } else if (lane < dxa.nparts) {
-                    const float2 o = reinterpret_cast<const float2*>(dxa.part_sums)[static_cast<int64_t>(lane) * rows + r];
-                    p1 = o.x, p2 = o.y;
-                }
+                float p1 = peer[u].x, p2 = peer[u].y;
+                if (lane == dxa.my_part) p1 = s1, p2 = s2;
                 const float S1 = wave_sum(p1) * dxa.weight, S2 = wave_sum(p2) * dxa.weight;
                 T* dxr = static_cast<T*>(dxa.dx) + r * dxa.ld_dx;
 #pragma unroll
