@@ -29,6 +29,8 @@ DDL_DT_F32 = 1
 DDL_DT_F64 = 2
 DDL_DT_BF16 = 3
 DDL_DT_F16 = 4
+DDL_DT_I32 = 5
+DDL_DT_I64 = 6
 
 DDL_HALO_AUTO = 0
 DDL_HALO_ROWS = 1

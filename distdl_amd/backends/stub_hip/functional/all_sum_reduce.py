@@ -11,6 +11,7 @@ class AllSumReduceFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, P_reduce, tag=None):
+        ctx.P_reduce, ctx.tag = P_reduce, tag
         if not P_reduce.active or P_reduce.size == 1:
             return input
         parts = P_reduce._world.transport.allgather(P_reduce, input.detach(), tag=tag)
@@ -18,4 +19,9 @@ class AllSumReduceFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        raise NotImplementedError("the adjoint of AllSumReduce is a collective, not part of this build")
+        # The all-sum-reduce is its own adjoint (reference :95-161).
+        P_reduce = ctx.P_reduce
+        if not P_reduce.active or P_reduce.size == 1:
+            return grad_output, None, None
+        parts = P_reduce._world.transport.allgather(P_reduce, grad_output.detach().contiguous(), tag=("adjoint", ctx.tag))
+        return parts.sum(dim=0), None, None

@@ -9,24 +9,35 @@ __all__ = ["BroadcastFunction"]
 
 import torch
 
+from ....utilities.torch import zero_volume_tensor
+
 
 class BroadcastFunction(torch.autograd.Function):
 
     @staticmethod
-    def forward(ctx, input, P_send, P_recv, preserve_batch=False, tag=None):
+    def forward(ctx, input, P_send, P_recv, preserve_batch=False, tag=None, transpose_src=False, transpose_dest=False):
         if not (P_send.active or P_recv.active):
             return input
         ctx.P_send, ctx.P_recv, ctx.tag = P_send, P_recv, tag
+        ctx.transposes = (transpose_src, transpose_dest)
         ctx.input_like = (tuple(input.shape), input.dtype, input.device)
         world = P_send._world if P_send._world is not None else P_recv._world
-        return world.transport.broadcast(P_send, P_recv, input.detach(), tag=tag)
+        out = world.transport.broadcast(P_send, P_recv, input.detach(), transpose_src=transpose_src,
+                                        transpose_dst=transpose_dest, tag=tag)
+        if not P_recv.active:
+            # A worker that only sends holds nothing afterwards (reference :50-54, :116-128).
+            batch = int(input.shape[0]) if (preserve_batch and input.dim() > 0) else None
+            out = zero_volume_tensor(batch, dtype=input.dtype, device=input.device)
+        return out
 
     @staticmethod
     def backward(ctx, grad_output):
         P_send, P_recv = ctx.P_send, ctx.P_recv
         world = P_send._world if P_send._world is not None else P_recv._world
-        grad = world.transport.broadcast_adjoint(P_send, P_recv, grad_output.detach(), tag=ctx.tag)
+        transpose_src, transpose_dest = ctx.transposes
+        grad = world.transport.broadcast_adjoint(P_send, P_recv, grad_output.detach(), transpose_src=transpose_src,
+                                                 transpose_dst=transpose_dest, tag=ctx.tag)
         if grad is None:
             shape, dtype, device = ctx.input_like
             grad = torch.zeros(shape, dtype=dtype, device=device)
-        return grad, None, None, None, None
+        return grad, None, None, None, None, None, None

@@ -1,20 +1,49 @@
-"""Sum-reduce stand-in (reference: backends/mpi_numpy/functional/sum_reduce.py:115-122).
-A collective, hence outside this build; only the trivial one-source case is
-answered, everything else raises."""
+"""Sum-reduce stand-in (reference: backends/mpi_numpy/functional/sum_reduce.py:13-122,
+:125-206).  The reduction is the adjoint of the broadcast and is delegated to
+the transport the same way: the partial tensors of the workers of ``P_send``
+are added, in rank order, onto the worker of ``P_recv`` they would receive a
+broadcast from; the adjoint hands that worker's gradient back to every one of
+them.  Workers outside the receiving partition get the reference's zero-volume
+tensor."""
 
 __all__ = ["SumReduceFunction"]
 
 import torch
 
+from ....utilities.torch import zero_volume_tensor
+
+
+def _world_of(P_send, P_recv):
+    return P_send._world if P_send._world is not None else P_recv._world
+
 
 class SumReduceFunction(torch.autograd.Function):
 
     @staticmethod
-    def forward(ctx, input, P_send, P_recv, preserve_batch=True, tag=None):
-        if P_send.active and P_send.size == 1 and P_recv.active:
+    def forward(ctx, input, P_send, P_recv, preserve_batch=True, tag=None, transpose_src=False, transpose_dest=False):
+        if not (P_send.active or P_recv.active):
             return input
-        raise NotImplementedError("SumReduce over more than one source is a collective, not part of this build")
+        ctx.P_send, ctx.P_recv, ctx.tag = P_send, P_recv, tag
+        ctx.transposes = (transpose_src, transpose_dest)
+        ctx.input_like = (tuple(input.shape), input.dtype, input.device)
+        # The receiving partition is the smaller one, the "source" of the
+        # broadcast this reduction is the adjoint of.
+        out = _world_of(P_send, P_recv).transport.broadcast_adjoint(
+            P_recv, P_send, input.detach(), transpose_src=transpose_dest, transpose_dst=transpose_src,
+            tag=("sum-reduce", tag))
+        if out is None:
+            batch = int(input.shape[0]) if (preserve_batch and input.dim() > 0) else None
+            out = zero_volume_tensor(batch, dtype=input.dtype, device=input.device)
+        return out
 
     @staticmethod
     def backward(ctx, grad_output):
-        raise NotImplementedError("the adjoint of SumReduce is a collective, not part of this build")
+        P_send, P_recv = ctx.P_send, ctx.P_recv
+        transpose_src, transpose_dest = ctx.transposes
+        shape, dtype, device = ctx.input_like
+        grad = _world_of(P_send, P_recv).transport.broadcast(
+            P_recv, P_send, grad_output.detach(), transpose_src=transpose_dest, transpose_dst=transpose_src,
+            tag=("sum-reduce-adjoint", ctx.tag))
+        if not P_send.active:
+            grad = torch.zeros(shape, dtype=dtype, device=device)
+        return grad, None, None, None, None, None, None

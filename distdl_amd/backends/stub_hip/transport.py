@@ -26,6 +26,35 @@ class TransportError(RuntimeError):
     pass
 
 
+def broadcast_partner(small_shape, small_index, big_shape, big_index, transpose_small=False, transpose_big=False):
+    """Whether the worker at ``small_index`` of the smaller partition is the one
+    the worker at ``big_index`` of the larger partition receives a broadcast
+    from (sends its part of a sum to).  The rule of the reference
+    (backends/common/partition.py:552-604, :745-794): either shape may be
+    reversed first, the smaller one is then padded with ones on the left, a
+    dimension takes part where the two extents agree, and must have extent 1 in
+    the smaller partition where they do not."""
+    small_shape = [int(n) for n in small_shape]
+    small_index = [int(i) for i in small_index]
+    big_shape = [int(n) for n in big_shape]
+    big_index = [int(i) for i in big_index]
+    if transpose_small:
+        small_shape, small_index = small_shape[::-1], small_index[::-1]
+    if transpose_big:
+        big_shape, big_index = big_shape[::-1], big_index[::-1]
+    pad = len(big_shape) - len(small_shape)
+    if pad < 0:
+        raise TransportError("broadcast: the source partition has more dimensions than the destination")
+    small_shape, small_index = [1] * pad + small_shape, [0] * pad + small_index
+    for d, (a, b) in enumerate(zip(small_shape, big_shape)):
+        if a == b:
+            if small_index[d] != big_index[d]:
+                return False
+        elif a != 1:
+            raise TransportError(f"broadcast: extents {a} and {b} of dimension {d} neither agree nor is the smaller one 1")
+    return True
+
+
 # ---------------------------------------------------------------------------
 # Solo
 # ---------------------------------------------------------------------------
@@ -127,14 +156,14 @@ class SoloTransport:
         fn = self._gather_providers.get(tag)
         return fn is None or self._seeded.get(tag) == (buffer.data_ptr(), tuple(buffer.shape))
 
-    def broadcast(self, P_src, P_dst, tensor, tag=None):
+    def broadcast(self, P_src, P_dst, tensor, transpose_src=False, transpose_dst=False, tag=None):
         if P_src.active:
             return tensor
         raise TransportError("solo transport: the live rank is not a source of this broadcast")
 
-    def broadcast_adjoint(self, P_src, P_dst, grad, tag=None):
-        """The live rank owns the data; the gradients of the absent workers are
-        absent too."""
+    def broadcast_adjoint(self, P_src, P_dst, grad, transpose_src=False, transpose_dst=False, tag=None):
+        """Sum-reduce from ``P_dst`` onto ``P_src``.  The live rank owns the
+        data; the contributions of the absent workers are absent too."""
         return grad if P_src.active else None
 
     def gather_list(self, P, tensor, tag=None):
@@ -335,29 +364,40 @@ class LoopbackTransport:
         self._allgather_obj(P, None, ("tgather-into-done", tag))
         return buffer
 
-    def broadcast(self, P_src, P_dst, tensor, tag=None):
+    def _shapes_of(self, union, P_src, P_dst, kind, tag):
+        """The shapes of both partitions, known to every worker of the union
+        (a worker outside a partition does not know that partition's shape)."""
+        mine = (tuple(int(n) for n in P_src.shape) if P_src.active else None,
+                tuple(int(n) for n in P_dst.shape) if P_dst.active else None)
+        everyone = self._allgather_obj(union, mine, (kind, tag))
+        src_shape = next(a for a, _ in everyone if a is not None)
+        dst_shape = next(b for _, b in everyone if b is not None)
+        return src_shape, dst_shape
+
+    def broadcast(self, P_src, P_dst, tensor, transpose_src=False, transpose_dst=False, tag=None):
         """Every worker of ``P_dst`` receives the tensor held by the worker of
         ``P_src`` that shares its index in the dimensions ``P_src`` spans
-        (weights stored on a sub-grid, used on the full grid)."""
+        (weights stored on a sub-grid, used on the full grid); see
+        :func:`broadcast_partner`."""
         union = P_src.create_partition_union(P_dst)
         key = ("tbcast", tag)
+        src_shape, dst_shape = self._shapes_of(union, P_src, P_dst, "tbcast-shapes", tag)
         payload = (tuple(int(i) for i in P_src.index), tensor) if P_src.active else None
         everyone = self._allgather_obj(union, payload, key)
         out = tensor
-        if P_dst.active and not P_src.active:
+        if P_dst.active:
             mine = [int(i) for i in P_dst.index]
             match = None
             for item in everyone:
                 if item is None:
                     continue
                 index, t = item
-                src_shape = [int(s) for s in P_src.shape]
-                if all(src_shape[d] == 1 or index[d] == mine[d] for d in range(len(src_shape))):
+                if broadcast_partner(src_shape, index, dst_shape, mine, transpose_src, transpose_dst):
                     match = t
                     break
             if match is None:
                 raise TransportError("broadcast: no source worker matches this destination index")
-            out = match.clone()
+            out = tensor if match is tensor else match.clone()
         self._allgather_obj(union, None, ("tbcast-done", tag))
         return out
 
@@ -372,23 +412,24 @@ class LoopbackTransport:
         owners may reuse them from here on."""
         self._allgather_obj(P, None, ("tlist-done", tag))
 
-    def broadcast_adjoint(self, P_src, P_dst, grad, tag=None):
+    def broadcast_adjoint(self, P_src, P_dst, grad, transpose_src=False, transpose_dst=False, tag=None):
         """Sum-reduce: every worker of ``P_src`` receives the sum of the
-        gradients held by the workers of ``P_dst`` it was broadcast to; the
-        other workers receive None."""
+        tensors held by the workers of ``P_dst`` it would broadcast to, added in
+        rank order; the other workers receive None."""
         from ... import hip_ops
         union = P_src.create_partition_union(P_dst)
+        src_shape, dst_shape = self._shapes_of(union, P_src, P_dst, "tbcast-adj-shapes", tag)
         payload = (tuple(int(i) for i in P_dst.index), grad) if P_dst.active else None
         everyone = self._allgather_obj(union, payload, ("tbcast-adj", tag))
         out = None
         if P_src.active:
             mine = [int(i) for i in P_src.index]
-            src_shape = [int(s) for s in P_src.shape]
-            for item in everyone:
+            # In the order of the workers' ranks in the world, whatever the order of the union.
+            for _, item in sorted(zip(union._ranks, everyone), key=lambda pair: pair[0]):
                 if item is None:
                     continue
                 index, g = item
-                if not all(src_shape[d] == 1 or index[d] == mine[d] for d in range(len(src_shape))):
+                if not broadcast_partner(src_shape, mine, dst_shape, index, transpose_src, transpose_dst):
                     continue
                 if out is None:
                     out = g.clone()

@@ -97,6 +97,19 @@ struct f16_bits {
     uint16_t u;
 };
 
+// Integers wrap around, as two's-complement sums do in NumPy and ATen.
+template <>
+struct AddOp<int32_t> {
+    static __device__ int32_t apply(int32_t a, int32_t b) {
+        return static_cast<int32_t>(static_cast<uint32_t>(a) + static_cast<uint32_t>(b));
+    }
+};
+template <>
+struct AddOp<int64_t> {
+    static __device__ int64_t apply(int64_t a, int64_t b) {
+        return static_cast<int64_t>(static_cast<uint64_t>(a) + static_cast<uint64_t>(b));
+    }
+};
 template <>
 struct AddOp<bf16_bits> {
     // fp32 add, round to nearest even, quiet NaN: the arithmetic ATen uses for
@@ -495,9 +508,9 @@ int launch_batches(const std::vector<DevBox>& boxes, hipStream_t stream) {
 int run_boxes(const ddl_box_t* boxes, int nbox, int elem_size, int op, int dtype, bool has_src, hipStream_t stream) {
     if (nbox < 0 || (nbox > 0 && boxes == nullptr)) return fail(DDL_E_ARG, "bad box list (nbox=%d)", nbox);
     if (elem_size < 1 || elem_size > 4096) return fail(DDL_E_ARG, "element size %d outside [1,4096]", elem_size);
-    static const int dt_size[] = {0, 4, 8, 2, 2};
+    static const int dt_size[] = {0, 4, 8, 2, 2, 4, 8};
     if (op == DDL_OP_ADD) {
-        if (dtype < DDL_DT_F32 || dtype > DDL_DT_F16) return fail(DDL_E_ARG, "DDL_OP_ADD needs a floating dtype, got %d", dtype);
+        if (dtype < DDL_DT_F32 || dtype > DDL_DT_I64) return fail(DDL_E_ARG, "DDL_OP_ADD needs an arithmetic dtype, got %d", dtype);
         if (dt_size[dtype] != elem_size) return fail(DDL_E_ARG, "dtype %d does not have element size %d", dtype, elem_size);
     } else if (op != DDL_OP_COPY && op != OP_ZERO) {
         return fail(DDL_E_ARG, "unknown box operation %d", op);
@@ -513,6 +526,8 @@ int run_boxes(const ddl_box_t* boxes, int nbox, int elem_size, int op, int dtype
         case DDL_DT_F32: return launch_batches<OP_ADD, float>(dev, stream);
         case DDL_DT_F64: return launch_batches<OP_ADD, double>(dev, stream);
         case DDL_DT_BF16: return launch_batches<OP_ADD, bf16_bits>(dev, stream);
+        case DDL_DT_I32: return launch_batches<OP_ADD, int32_t>(dev, stream);
+        case DDL_DT_I64: return launch_batches<OP_ADD, int64_t>(dev, stream);
         default: return launch_batches<OP_ADD, f16_bits>(dev, stream);
     }
 }

@@ -14,6 +14,8 @@ _ADD_DTYPES = {
     torch.float64: _lib.DDL_DT_F64,
     torch.bfloat16: _lib.DDL_DT_BF16,
     torch.float16: _lib.DDL_DT_F16,
+    torch.int32: _lib.DDL_DT_I32,
+    torch.int64: _lib.DDL_DT_I64,
 }
 
 
@@ -171,6 +173,8 @@ def copy_box(src, src_slices, dst, dst_slices, accumulate=False):
     box.dst = dst.data_ptr() + doff * es
     op, dt = _lib.DDL_OP_COPY, _lib.DDL_DT_BITS
     if accumulate:
+        if src.dtype not in _ADD_DTYPES:
+            raise ValueError(f"accumulating copy is not available for {src.dtype}")
         op, dt = _lib.DDL_OP_ADD, _ADD_DTYPES[src.dtype]
     rc = _lib.load().ddl_copy_boxes(ctypes.byref(box), 1, es, op, dt, _stream())
     _lib.check(rc, "ddl_copy_boxes")

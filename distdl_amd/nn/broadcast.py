@@ -11,6 +11,8 @@ class Broadcast(Module):
         super().__init__()
         self.P_x = P_x
         self.P_y = P_y
+        self.transpose_src = transpose_src
+        self.transpose_dest = transpose_dest
         self.preserve_batch = preserve_batch
         # Source and destination are the same team: nothing moves.
         self.identity = (P_x == P_y)
@@ -19,4 +21,5 @@ class Broadcast(Module):
         if self.identity or not (self.P_x.active or self.P_y.active):
             return input
         Function = self._distdl_backend.functional.broadcast.BroadcastFunction
-        return Function.apply(input, self.P_x, self.P_y, self.preserve_batch, None)
+        return Function.apply(input, self.P_x, self.P_y, self.preserve_batch, None,
+                              self.transpose_src, self.transpose_dest)

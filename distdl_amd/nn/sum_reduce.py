@@ -1,6 +1,7 @@
-"""SumReduce layer stand-in (reference: nn/sum_reduce.py).  Only the case in
-which every destination worker has a single source is answered (no arithmetic
-is needed then); a true reduction is a collective outside this build."""
+"""SumReduce layer stand-in (reference: nn/sum_reduce.py): the partial tensors
+held on ``P_x`` are summed onto ``P_y`` along the dimensions in which ``P_y`` has
+one worker, by the reference's broadcast rules read backwards.  The collective
+itself is outside this build; see backends/stub_hip/functional/sum_reduce.py."""
 
 from .module import Module
 
@@ -11,13 +12,15 @@ class SumReduce(Module):
         super().__init__()
         self.P_x = P_x
         self.P_y = P_y
+        self.transpose_src = transpose_src
+        self.transpose_dest = transpose_dest
         self.preserve_batch = preserve_batch
+        # Source and destination are the same team: nothing is added.
+        self.identity = (P_x == P_y)
 
     def forward(self, input):
-        if not (self.P_x.active or self.P_y.active):
+        if self.identity or not (self.P_x.active or self.P_y.active):
             return input
-        sources = max(int(self.P_x.size), 1) // max(int(self.P_y.size), 1)
-        if self.P_x.active and self.P_y.active and sources == 1:
-            return input
-        raise NotImplementedError("SumReduce with more than one source per destination is a collective, "
-                                  "not part of this build")
+        Function = self._distdl_backend.functional.sum_reduce.SumReduceFunction
+        return Function.apply(input, self.P_x, self.P_y, self.preserve_batch, None,
+                              self.transpose_src, self.transpose_dest)

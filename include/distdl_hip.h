@@ -84,6 +84,8 @@ typedef struct ddl_box {
 #define DDL_DT_F64  2
 #define DDL_DT_BF16 3
 #define DDL_DT_F16  4
+#define DDL_DT_I32  5   /* box accumulation only; sums wrap around             */
+#define DDL_DT_I64  6   /* box accumulation only; sums wrap around             */
 
 /* Copies (or accumulates) `nbox` boxes in as few launches as possible (16
  * boxes per launch).  Boxes of one call must not overlap each other on the

@@ -467,3 +467,24 @@ def test_all_gather_and_reduce_scatter_layers(P, shape, axis, dtype):
         assert np.array_equal(dx, want_dx[r])
         assert np.array_equal(z, want_z[r])
         assert np.array_equal(dfull, dz_full)
+
+
+@pytest.mark.parametrize("dtype", [torch.int32, torch.int64])
+def test_box_accumulate_integers_wrap_around(dtype):
+    """dst += src on integer boxes (the forward-only integer cases of the
+    reference's reduction tests): exact, and two's-complement wrap-around at
+    the ends of the range, as NumPy and ATen add."""
+    from distdl_amd import hip_ops
+    info = torch.iinfo(dtype)
+    gen = torch.Generator().manual_seed(3)
+    src = torch.randint(-1000, 1000, (5, 37, 19), generator=gen).to(dtype)
+    dst = torch.randint(-1000, 1000, (7, 40, 23), generator=gen).to(dtype)
+    src[0, 0, 0], dst[1, 2, 3] = info.max, 5            # wraps to min + 4
+    src[4, 36, 18], dst[5, 38, 21] = info.min, -1       # wraps to max
+    want = dst.clone()
+    want[1:6, 2:39, 3:22] += src
+    assert int(want[1, 2, 3]) == info.min + 4 and int(want[5, 38, 21]) == info.max
+    d = dst.cuda()
+    hip_ops.copy_box(src.cuda(), [slice(0, 5), slice(0, 37), slice(0, 19)], d, [slice(1, 6), slice(2, 39), slice(3, 22)],
+                     accumulate=True)
+    assert torch.equal(d.cpu(), want)

@@ -523,3 +523,34 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     rc = lib.ddl_embedding_gather(16, 8, 8, 3, 16, 1, 4, 0, 4, 16, None)
     assert rc == -1
     assert lib.ddl_pack_boxes(1, shape, shape, 2, 4, 0, shape, shape, _lib.ptr_array([]), None) == 0
+
+
+def test_broadcast_partner_follows_the_reference_rule():
+    """backends/common/partition.py:552-604, :745-794: shapes compared after an
+    optional reversal and left-padding of the smaller one with ones; a worker of
+    the larger team belongs to the smaller team's worker with the same index in
+    the dimensions whose extents agree."""
+    import itertools
+
+    from distdl_amd.backends.stub_hip.transport import TransportError, broadcast_partner
+
+    def owners(small_shape, big_shape, big_index, transpose_small=False, transpose_big=False):
+        return [s for s in itertools.product(*[range(n) for n in small_shape])
+                if broadcast_partner(small_shape, s, big_shape, big_index, transpose_small, transpose_big)]
+
+    for i in itertools.product(range(2), range(2), range(3)):
+        assert owners([2, 2, 1], [2, 2, 3], i) == [(i[0], i[1], 0)]
+    for i in itertools.product(range(3), range(2), range(2)):
+        assert owners([2, 2, 1], [3, 2, 2], i, transpose_big=True) == [(i[2], i[1], 0)]     # [2, 2, 3] against [2, 2, 1]
+        assert owners([2, 2, 1], [3, 2, 2], i, transpose_small=True) == [(i[2], i[1], 0)]   # [3, 2, 2] against [1, 2, 2]
+    for c in range(3):
+        assert owners([1], [1, 1, 3], (0, 0, c)) == [(0,)]
+    # The affine layer: x on 1 x P_fi goes down the columns of P_fo x P_fi,
+    # partial outputs are summed along its rows onto 1 x P_fo.
+    for o, i in itertools.product(range(3), range(4)):
+        assert owners([1, 4], [3, 4], (o, i)) == [(0, i)]
+        assert owners([1, 3], [3, 4], (o, i), transpose_big=True) == [(0, o)]
+    with pytest.raises(TransportError):
+        broadcast_partner([2, 3], [0, 0], [2, 2], [0, 0])
+    with pytest.raises(TransportError):
+        broadcast_partner([1, 1, 2], [0, 0, 0], [2, 2], [0, 0])
