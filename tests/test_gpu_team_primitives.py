@@ -1,6 +1,6 @@
-"""Broadcast, SumReduce and AllSumReduce between simulated workers, on the
-parametrizations of the reference's own tests, and DistributedLinear with a
-partitioned input dimension on top of them.  The collectives themselves are
+"""Broadcast, SumReduce, AllSumReduce, AllGather and ReduceScatter between
+simulated workers, on the parametrizations of the reference's own tests, and
+DistributedLinear with a partitioned input dimension on top of them.  The collectives themselves are
 stand-ins (rank threads of one process); the sums run on the box kernel and the
 shard products on the GEMM kernels.  Expected values come from a rule written
 out per case below, not from the transport's own partner search."""
@@ -265,3 +265,119 @@ def test_linear_layer_reference_cases(x_ranks, P_x_shape, y_ranks, P_y_shape, P_
                 seen[3] += 1
                 assert rw % P_fi == 0 and np.allclose(db.numpy(), want_db[rw // P_fi], rtol=1e-5, atol=1e-5)
     assert seen == [len(y_ranks), len(x_ranks), P_fo * P_fi, P_fo if use_bias else 0]
+
+
+def _integers(n, shape, seed):
+    rng = np.random.default_rng(seed)
+    return [rng.integers(-4, 5, size=shape).astype(np.float32) for _ in range(n)]
+
+
+# (P_x shape, shape of the scattered tensor, shape of the gathered tensor, axis).
+# The shapes are "global" in the reference's sense: every worker holds the
+# balanced piece of each at its own index.
+GATHER_LAYOUTS = [
+    pytest.param([2, 3], [2, 3], [4, 3], 0, id="2x3-axis0"),
+    pytest.param([2, 3], [2, 3], [2, 9], 1, id="2x3-axis1"),
+    pytest.param([4], [4], [16], 0, id="4-axis0"),
+    pytest.param([2, 3], [3, 3], [6, 3], 0, id="2x3-axis0-uneven"),
+    pytest.param([2, 3], [2, 4], [2, 12], 1, id="2x3-axis1-uneven"),
+    pytest.param([4], [6], [24], 0, id="4-axis0-uneven"),
+]
+
+
+def _piece_shapes(P_shape, global_shape):
+    from oracle import partition_math as pm
+    boxes = pm.boxes_balanced(P_shape, global_shape)
+    return [tuple(int(b) - int(a) for a, b in zip(*boxes[idx])) for idx in pm.indices(P_shape)]
+
+
+def _line_of(rank, P_shape, axis):
+    """World ranks of the workers that differ from `rank` along `axis` only, in order."""
+    index = list(_index_of(rank, P_shape))
+    line = []
+    for k in range(P_shape[axis]):
+        index[axis] = k
+        line.append(int(np.ravel_multi_index(index, P_shape)))
+    return line
+
+
+@pytest.mark.parametrize("P_shape,small_global,big_global,axis", GATHER_LAYOUTS)
+def test_all_gather_and_reduce_scatter_reference_layouts(P_shape, small_global, big_global, axis):
+    """tests/primitives/test_all_gather.py:10-81 and test_reduce_scatter.py:10-81:
+    partitions with a second, untouched dimension and one-dimensional ones, even
+    and uneven pieces.  AllGather: every worker ends with the pieces of its line
+    along the axis, concatenated in order; ReduceScatter: with its piece of the
+    line's sum; each is the other's adjoint.  Small integers, so sums are exact."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import AllGather, ReduceScatter
+    n = int(np.prod(P_shape))
+    small_shapes = _piece_shapes(P_shape, small_global)
+    xs = [_integers(1, small_shapes[r], 10 + r)[0] for r in range(n)]
+    lines = [_line_of(r, P_shape, axis) for r in range(n)]
+    gathered_shapes = []
+    for r in range(n):
+        shape = list(small_shapes[r])
+        shape[axis] = sum(small_shapes[s][axis] for s in lines[r])
+        gathered_shapes.append(tuple(shape))
+    dys = [_integers(1, gathered_shapes[r], 40 + r)[0] for r in range(n)]
+    fulls = [_integers(1, gathered_shapes[r], 70 + r)[0] for r in range(n)]
+    dzs = [_integers(1, small_shapes[r], 100 + r)[0] for r in range(n)]
+
+    def body(P_world):
+        P_x = P_world.create_partition_inclusive(list(range(n))).create_cartesian_topology_partition(P_shape)
+        r = P_x.rank
+        xin = torch.from_numpy(xs[r]).cuda().requires_grad_(True)
+        y = AllGather(P_x, axes_all_gather=(axis,))(xin)
+        y.backward(torch.from_numpy(dys[r]).cuda())
+        fin = torch.from_numpy(fulls[r]).cuda().requires_grad_(True)
+        z = ReduceScatter(P_x, axes_reduce_scatter=(axis,))(fin)
+        z.backward(torch.from_numpy(dzs[r]).cuda())
+        torch.cuda.synchronize()
+        return y.detach().cpu().numpy(), xin.grad.cpu().numpy(), z.detach().cpu().numpy(), fin.grad.cpu().numpy()
+
+    outs = SimWorld(n).run(body)
+    for r, (y, dx, z, dfull) in enumerate(outs):
+        line = lines[r]
+        me = line.index(r)
+        starts = np.cumsum([0] + [small_shapes[s][axis] for s in line])
+        mine = [slice(None)] * len(P_shape)
+        mine[axis] = slice(int(starts[me]), int(starts[me + 1]))
+        assert np.array_equal(y, np.concatenate([xs[s] for s in line], axis=axis)), f"worker {r}"
+        assert np.array_equal(dx, sum(dys[s] for s in line)[tuple(mine)]), f"worker {r}"
+        assert np.array_equal(z, sum(fulls[s] for s in line)[tuple(mine)]), f"worker {r}"
+        assert np.array_equal(dfull, np.concatenate([dzs[s] for s in line], axis=axis)), f"worker {r}"
+
+
+@pytest.mark.parametrize("P_shape,shape,axes", [
+    ([2, 2, 3], [3, 4], ()), ([2, 2, 3], [3, 4], (0,)), ([2, 2, 3], [3, 4], (1,)), ([2, 2, 3], [3, 4], (2,)),
+    ([2, 2, 3], [3, 4], (0, 1)), ([2, 2, 3], [3, 4], (0, 2)), ([2, 2, 3], [3, 4], (1, 2)), ([2, 2, 3], [3, 4], (0, 1, 2)),
+    ([12], [30, 344], (0,)),
+])
+def test_all_sum_reduce_reference_layouts(P_shape, shape, axes):
+    """tests/primitives/test_all_sum_reduce.py:10-107: twelve workers as
+    2 x 2 x 3, reduced along every subset of the axes, and the twelve-way sum
+    of a [30, 344] weight; output and gradient are the sums over the workers
+    that share the index outside the reduced axes."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import AllSumReduce
+    n = int(np.prod(P_shape))
+    xs = _integers(n, shape, 5)
+    dys = _integers(n, shape, 6)
+
+    def body(P_world):
+        P_x = P_world.create_partition_inclusive(list(range(n))).create_cartesian_topology_partition(P_shape)
+        layer = AllSumReduce(P_x, axes_reduce=axes)
+        x = torch.from_numpy(xs[P_x.rank]).cuda().requires_grad_(True)
+        y = layer(x)
+        y.backward(torch.from_numpy(dys[P_x.rank]).cuda())
+        torch.cuda.synchronize()
+        return y.detach().cpu().numpy(), x.grad.cpu().numpy()
+
+    outs = SimWorld(n).run(body)
+    for r in range(n):
+        mine = _index_of(r, P_shape)
+        group = [s for s in range(n)
+                 if all(a == b for d, (a, b) in enumerate(zip(_index_of(s, P_shape), mine)) if d not in axes)]
+        assert len(group) == int(np.prod([P_shape[d] for d in axes])) if axes else group == [r]
+        assert np.array_equal(outs[r][0], sum(xs[s] for s in group)), f"worker {r}"
+        assert np.array_equal(outs[r][1], sum(dys[s] for s in group)), f"worker {r}"
