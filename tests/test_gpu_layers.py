@@ -634,6 +634,78 @@ def test_layernorm_layer_backward_matches_torch():
         assert np.allclose(sum(g.reshape(-1) for g in got_b), br.grad.numpy()[lo:hi], rtol=1e-4, atol=1e-4)
 
 
+def test_layernorm_training_step_reference_cases(golden):
+    """The reference's test_batch_norm_with_training (tests/layers/test_layernorm.py:143-277)
+    on its ten geometries: scatter from one worker, DistributedLayerNorm, gather,
+    squared-error loss, backward, a parameter step, a second forward -- against
+    torch.nn.LayerNorm on the whole tensor with the reference's tolerances
+    (rtol 1e-4, atol sqrt(1e-7)); the parameter gradients, which the reference
+    collects but never compares, are compared here as well."""
+    import math
+
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedLayerNorm, Repartition
+    from distdl_amd.utilities.torch import zero_volume_tensor
+    rtol, atol = 1e-4, math.sqrt(1e-7)
+    for geom in golden("layer_geometries.json")["layernorm"]:
+        P, shape, norm = geom["P_x_shape"], geom["input_shape"], geom["normalized_shape"]
+        n, nn_ = int(np.prod(P)), len(norm)
+        torch.manual_seed(0)
+        x_train, x_eval, target = torch.rand(shape), torch.rand(shape), torch.rand(shape)
+        seq = torch.nn.LayerNorm(norm)
+        seq_out1 = seq(x_train)
+        seq_loss = ((seq_out1 - target) ** 2).sum()
+        seq_loss.backward()
+        seq_grads = [p.grad.detach().clone() for p in seq.parameters()]
+        with torch.no_grad():
+            for p in seq.parameters():
+                p.copy_(p + 0.1 * p.grad)
+            seq_out2 = seq(x_eval)
+        Pn = [1] * (len(shape) - nn_) + list(P[-nn_:])
+        full = [1] * (len(shape) - nn_) + list(norm)
+        want_grads = [o_rep.scatter(g.numpy().reshape(full), Pn) for g in seq_grads]
+
+        def body(P_world):
+            P_root = P_world.create_partition_inclusive([0]).create_cartesian_topology_partition([1] * len(shape))
+            P_x = P_world.create_partition_inclusive(list(range(n))).create_cartesian_topology_partition(P)
+            scatter, gather = Repartition(P_root, P_x), Repartition(P_x, P_root)
+            layer = DistributedLayerNorm(P_x, norm)
+
+            def held(t):
+                return t.cuda() if P_root.active else zero_volume_tensor(device="cuda")
+            layer.train()
+            out1 = gather(layer(scatter(held(x_train))))
+            loss = ((out1 - held(target)) ** 2).sum()
+            assert loss.requires_grad
+            loss.backward()
+            grads = None
+            if layer.P_w.active:
+                grads = [p.grad.detach().cpu().numpy().copy() for p in layer.parameters()]
+                with torch.no_grad():
+                    for p in layer.parameters():
+                        p.copy_(p + 0.1 * p.grad)
+            layer.eval()
+            out2 = gather(layer(scatter(held(x_eval)))).detach()
+            torch.cuda.synchronize()
+            red = int(np.ravel_multi_index(tuple(int(i) for i in P_x.index[-nn_:]), tuple(P[-nn_:])))
+            return out1.detach().cpu(), loss.detach().cpu(), grads, red, out2.cpu()
+
+        outs = SimWorld(n).run(body)
+        out1, loss, _, _, out2 = outs[0]
+        assert out1.shape == seq_out1.shape and torch.allclose(out1, seq_out1.detach(), rtol=rtol, atol=atol), geom
+        assert torch.allclose(loss, seq_loss.detach(), rtol=rtol, atol=atol), geom
+        assert out2.shape == seq_out2.shape and torch.allclose(out2, seq_out2, rtol=rtol, atol=atol), geom
+        holders = 0
+        for _, _, grads, red, _ in outs:
+            if grads is None:
+                continue
+            holders += 1
+            assert len(grads) == 2
+            for got, want in zip(grads, want_grads):
+                assert got.shape == want[red].shape and np.allclose(got, want[red], rtol=rtol, atol=atol), geom
+        assert holders == int(np.prod(P[-nn_:])), geom
+
+
 # ---------------------------------------------------------------- Embedding --
 
 def test_embedding_config3_rank0_bit_exact(ops):
@@ -694,6 +766,68 @@ def test_embedding_layer_full_window_matches_torch():
 
     outs = SimWorld(4).run(body)
     assert torch.equal(torch.cat(outs, dim=-1), want)
+
+
+@pytest.mark.parametrize("P,table_shape", [([1, 1], (4, 12)), ([1, 4], (4, 12)), ([1, 3], (9, 16))])
+def test_embedding_training_step_reference_cases(P, table_shape):
+    """The reference's test_batch_norm_with_training for the embedding
+    (tests/layers/test_embedding.py:10-156; serial and 1 x 4 workers on a
+    [4, 12] table, and a table whose width does not divide evenly): the table is
+    scattered from one worker and handed to the layer as ``_weight``; lookup of
+    every row, gather, squared-error loss, backward, a parameter step, a second
+    lookup -- against torch.nn.Embedding with the reference's tolerances."""
+    import math
+
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedEmbedding, Repartition
+    from distdl_amd.utilities.torch import zero_volume_tensor
+    rtol, atol = 1e-4, math.sqrt(1e-7)
+    n = int(np.prod(P))
+    torch.manual_seed(0)
+    table, target = torch.rand(table_shape), torch.rand(table_shape)
+    ids = torch.arange(table_shape[0])
+    seq = torch.nn.Embedding(*table_shape, _weight=table.clone())
+    seq_out1 = seq(ids)
+    seq_loss = ((seq_out1 - target) ** 2).sum()
+    seq_loss.backward()
+    seq_grad = seq.weight.grad.detach().clone()
+    with torch.no_grad():
+        seq.weight.copy_(seq.weight + 0.1 * seq.weight.grad)
+        seq_out2 = seq(ids)
+    want_grad = o_rep.scatter(seq_grad.numpy(), P)
+
+    def body(P_world):
+        P_root = P_world.create_partition_inclusive([0]).create_cartesian_topology_partition([1, 1])
+        P_x = P_world.create_partition_inclusive(list(range(n))).create_cartesian_topology_partition(P)
+        scatter, gather = Repartition(P_root, P_x), Repartition(P_x, P_root)
+
+        def held(t):
+            return t.cuda() if P_root.active else zero_volume_tensor(device="cuda")
+        layer = DistributedEmbedding(P_x, *table_shape, _weight=scatter(held(table)))
+        assert list(layer.P_weight.shape) == list(P)
+        layer.train()
+        out1 = gather(layer(ids.cuda()))
+        loss = ((out1 - held(target)) ** 2).sum()
+        assert loss.requires_grad
+        loss.backward()
+        grad = None
+        if layer.P_weight.active:
+            grad = layer.weight.grad.detach().cpu().numpy().copy()
+            with torch.no_grad():
+                layer.weight.copy_(layer.weight + 0.1 * layer.weight.grad)
+        layer.eval()
+        out2 = gather(layer(ids.cuda())).detach()
+        torch.cuda.synchronize()
+        return out1.detach().cpu(), loss.detach().cpu(), grad, out2.cpu()
+
+    outs = SimWorld(n).run(body)
+    out1, loss, _, out2 = outs[0]
+    assert out1.shape == seq_out1.shape and torch.allclose(out1, seq_out1.detach(), rtol=rtol, atol=atol)
+    assert torch.allclose(loss, seq_loss.detach(), rtol=rtol, atol=atol)
+    assert out2.shape == seq_out2.shape and torch.allclose(out2, seq_out2, rtol=rtol, atol=atol)
+    for r, (_, _, grad, _) in enumerate(outs):
+        assert grad is not None and grad.shape == want_grad[r].shape
+        assert np.allclose(grad, want_grad[r], rtol=rtol, atol=atol)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
@@ -1290,27 +1424,103 @@ def test_linear_layers_forward(ops):
     _lin_check(bits16(y3), x3, ag.weight.detach().cpu().view(128, 256), ag.bias.detach().cpu().view(128))
 
 
-@pytest.mark.parametrize("P,use_bias", [([1, 1, 4], True), ([2, 1, 2], True), ([1, 1, 3], False)])
-def test_linear_reduce_scatter_layer_matches_torch(ops, P, use_bias):
-    """DistributedLinearReduceScatter over all workers (loopback): every worker
-    multiplies its slice of the input features by its weight shard, the partial
-    products are summed and scattered along the output features.  Forward and
-    backward against torch.nn.functional.linear on the whole tensors (float32,
-    the reference's default; reference: nn/linear_rs.py:361-364)."""
+@pytest.mark.parametrize("P,x_shape,c_out", [
+    ([1, 1], [2, 2], 4), ([1, 4], [1, 12], 16), ([1, 1, 4], [1, 8, 12], 16), ([2, 1, 4], [2, 4, 12], 16),
+    ([1, 1, 1, 4], [1, 2, 4, 12], 16), ([1, 2, 1, 2], [2, 2, 4, 12], 16), ([2, 1, 1, 2], [2, 2, 4, 12], 16),
+    ([2, 2, 1, 2], [2, 2, 4, 12], 16), ([2, 1, 3], [4, 5, 26], 20),
+])
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_linear_all_gather_layer_reference_layouts(ops, P, x_shape, c_out, use_bias):
+    """DistributedLinearAllGather over all workers (loopback) on the partitions
+    and shapes of the reference's adjoint tests (tests/layers/test_linear_ag.py:13-108:
+    two to four dimensions, data-parallel axes beside the feature axis) and on
+    an uneven one: the input is gathered along the features, every worker
+    applies its rows of the weight (stored on the first line of workers,
+    broadcast to the others), the output stays partitioned along the features.
+    Forward and all three gradients against torch.nn.functional.linear on the
+    whole tensors (float32, the reference's default)."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedLinearAllGather
+    from oracle import repartition as o_rep
+    n, M, c_in = int(np.prod(P)), P[-1], x_shape[-1]
+    gen = torch.Generator().manual_seed(sum(P) * 10 + len(P) + use_bias)
+    x = torch.randn(*x_shape, generator=gen)
+    w = 0.2 * torch.randn(c_out, c_in, generator=gen)
+    b = 0.2 * torch.randn(c_out, generator=gen) if use_bias else None
+    dy = torch.randn(*x_shape[:-1], c_out, generator=gen)
+    xs = o_rep.scatter(x.numpy(), P)
+    dys = o_rep.scatter(dy.numpy(), P)
+    w_rows = o_rep.scatter(w.numpy(), [M, 1])
+    b_rows = o_rep.scatter(b.numpy(), [M]) if use_bias else None
+
+    def body(P_world):
+        P_y = P_world.create_partition_inclusive(list(range(n))).create_cartesian_topology_partition(P)
+        layer = DistributedLinearAllGather(P_y, c_in, c_out, bias=use_bias)
+        stores = layer.P_store_weight.active
+        if stores:
+            m = int(layer.P_store_weight.index[-2])
+            assert m == int(P_y.index[-1]) and all(int(i) == 0 for i in P_y.index[:-1])
+            with torch.no_grad():
+                layer.weight.copy_(torch.from_numpy(w_rows[m]).view(layer.weight.shape))
+                if use_bias:
+                    layer.bias.copy_(torch.from_numpy(b_rows[m]).view(layer.bias.shape))
+        xin = torch.from_numpy(xs[P_y.rank]).cuda().requires_grad_(True)
+        y = layer(xin)
+        y.backward(torch.from_numpy(dys[P_y.rank]).cuda())
+        torch.cuda.synchronize()
+        dw = layer.weight.grad.cpu() if stores else None
+        db = layer.bias.grad.cpu() if stores and use_bias else None
+        return y.detach().cpu(), xin.grad.cpu(), dw, db, int(P_y.index[-1])
+
+    outs = SimWorld(n).run(body)
+    xr = x.clone().requires_grad_(True)
+    wr = w.clone().requires_grad_(True)
+    br = b.clone().requires_grad_(True) if use_bias else None
+    yr = F.linear(xr, wr, br)
+    yr.backward(dy)
+    want_y = o_rep.scatter(yr.detach().numpy(), P)
+    want_dx = o_rep.scatter(xr.grad.numpy(), P)
+    want_dw = o_rep.scatter(wr.grad.numpy(), [M, 1])
+    want_db = o_rep.scatter(br.grad.numpy(), [M]) if use_bias else None
+    seen = 0
+    for r, (y, dx, dw, db, m) in enumerate(outs):
+        assert np.allclose(y.numpy(), want_y[r], rtol=1e-5, atol=1e-5)
+        assert np.allclose(dx.numpy(), want_dx[r], rtol=1e-5, atol=1e-5)
+        if dw is not None:
+            seen += 1
+            assert np.allclose(dw.numpy().reshape(-1, c_in), want_dw[m], rtol=1e-5, atol=1e-4)
+            if use_bias:
+                assert np.allclose(db.numpy().reshape(-1), want_db[m], rtol=1e-5, atol=1e-4)
+    assert seen == M
+
+
+@pytest.mark.parametrize("P,x_shape,c_out", [
+    ([1, 1], [2, 12], 16), ([1, 4], [1, 12], 16), ([1, 1, 4], [1, 8, 12], 16), ([2, 1, 4], [2, 4, 12], 16),
+    ([1, 1, 1, 4], [1, 2, 4, 12], 16), ([1, 2, 1, 2], [2, 2, 4, 12], 16), ([2, 1, 1, 2], [2, 2, 4, 12], 16),
+    ([2, 2, 1, 2], [2, 2, 4, 12], 16), ([2, 1, 2], [4, 5, 26], 21), ([1, 1, 3], [2, 5, 26], 21),
+])
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_linear_reduce_scatter_layer_matches_torch(ops, P, x_shape, c_out, use_bias):
+    """DistributedLinearReduceScatter over all workers (loopback) on the
+    partitions and shapes of the reference's adjoint tests
+    (tests/layers/test_linear_rs.py:10-105) and on two whose feature counts do
+    not divide evenly: every worker multiplies its slice of the input features
+    by its weight shard, the partial products are summed and scattered along the
+    output features.  Forward and backward against torch.nn.functional.linear on
+    the whole tensors (float32, the reference's default; reference:
+    nn/linear_rs.py:361-364)."""
     from distdl_amd.backends.stub_hip import SimWorld
     from distdl_amd.nn import DistributedLinearReduceScatter
     from oracle import repartition as o_rep
-    D, M = P[0], P[2]
-    n = D * M
-    batch, tokens, c_in, c_out = 2 * D, 5, 26, 21          # neither feature count divides evenly among 3 or 4 workers
-    gen = torch.Generator().manual_seed(sum(P) * 10 + use_bias)
-    x = torch.randn(batch, tokens, c_in, generator=gen)
+    n, M, c_in = int(np.prod(P)), P[-1], x_shape[-1]
+    gen = torch.Generator().manual_seed(sum(P) * 10 + len(P) + use_bias)
+    x = torch.randn(*x_shape, generator=gen)
     w = 0.2 * torch.randn(c_out, c_in, generator=gen)
     b = 0.2 * torch.randn(c_out, generator=gen) if use_bias else None
-    dy = torch.randn(batch, tokens, c_out, generator=gen)
+    dy = torch.randn(*x_shape[:-1], c_out, generator=gen)
     xs = o_rep.scatter(x.numpy(), P)
     dys = o_rep.scatter(dy.numpy(), P)
-    w_shards = o_rep.scatter(w.numpy().reshape(1, c_out, c_in), [1, 1, M])
+    w_shards = o_rep.scatter(w.numpy(), [1, M])
 
     def body(P_world):
         P_x = P_world.create_partition_inclusive(list(range(n))).create_cartesian_topology_partition(P)
@@ -1336,14 +1546,14 @@ def test_linear_reduce_scatter_layer_matches_torch(ops, P, use_bias):
     yr.backward(dy)
     want_y = o_rep.scatter(yr.detach().numpy(), P)
     want_dx = o_rep.scatter(xr.grad.numpy(), P)
-    want_dw = o_rep.scatter(wr.grad.numpy().reshape(1, c_out, c_in), [1, 1, M])
+    want_dw = o_rep.scatter(wr.grad.numpy(), [1, M])
     seen_w = 0
     for r, (y, dx, dw, db, col) in enumerate(outs):
         assert np.allclose(y.numpy(), want_y[r], rtol=1e-5, atol=1e-5)
         assert np.allclose(dx.numpy(), want_dx[r], rtol=1e-5, atol=1e-5)
         if dw is not None:
             seen_w += 1
-            assert np.allclose(dw.numpy().reshape(c_out, -1), want_dw[col].reshape(c_out, -1), rtol=1e-5, atol=1e-4)
+            assert np.allclose(dw.numpy().reshape(c_out, -1), want_dw[col], rtol=1e-5, atol=1e-4)
         if db is not None:
             assert r == 0 and np.allclose(db.numpy().reshape(-1), br.grad.numpy(), rtol=1e-5, atol=1e-4)
     assert seen_w == M
