@@ -375,26 +375,41 @@ def test_feature_conv_matches_sequential_conv(golden):
             assert np.allclose(got, part, atol=1e-4, rtol=1e-4), geom["id"]
 
 
-def test_feature_conv_backward_matches_sequential_conv():
+@pytest.mark.parametrize("P,gshape,out_channels,padding,y_local", [
+    pytest.param([1, 1, 2, 2], [2, 3, 11, 13], 4, 1, None, id="2d-uneven-padded"),
+    # tests/layers/test_conv_1d.py:10-19, test_conv_2d.py:10-19, test_conv_3d.py:10-19 (kernel 3, ten output channels)
+    pytest.param([1, 1, 3], [1, 5, 10], 10, 0, None, id="reference-1d"),
+    pytest.param([1, 1, 2, 2], [1, 5, 10, 10], 10, 0, [1, 10, 4, 4], id="reference-2d"),
+    pytest.param([1, 1, 3, 2, 2], [1, 5, 10, 10, 10], 10, 0, None, id="reference-3d"),
+    # tests/layers/test_conv_2d.py:233-256: the local output shapes it states
+    pytest.param([1, 1, 2, 2], [1, 5, 10, 10], 10, 1, [1, 10, 5, 5], id="reference-2d-padded"),
+])
+def test_feature_conv_backward_matches_sequential_conv(P, gshape, out_channels, padding, y_local):
     """Input and parameter gradients of the distributed convolution (staging
     crop, halo-exchange adjoint, broadcast adjoint) against torch autograd on
-    the whole tensor: the reference's adjoint-style check, with values."""
+    the whole tensor: the reference's adjoint tests of the input, the weight and
+    the bias on its own partitions and sizes, with values instead of the inner
+    products, and the local output shapes its shape test states."""
     from distdl_amd.backends.stub_hip import SimWorld
-    from distdl_amd.nn import DistributedConv2d
-    rng = np.random.default_rng(62)
-    P, gshape, k = [1, 1, 2, 2], [2, 3, 11, 13], [3, 3]
+    from distdl_amd import nn as dnn
+    nd = len(gshape) - 2
+    n = int(np.prod(P))
+    Conv = {1: dnn.DistributedConv1d, 2: dnn.DistributedConv2d, 3: dnn.DistributedConv3d}[nd]
+    conv = {1: F.conv1d, 2: F.conv2d, 3: F.conv3d}[nd]
+    rng = np.random.default_rng(62 + nd)
+    k = [3] * nd
     x = rng.standard_normal(gshape).astype(np.float32)
-    w = torch.from_numpy(rng.standard_normal([4, 3] + k).astype(np.float32))
-    b = torch.from_numpy(rng.standard_normal(4).astype(np.float32))
+    w = torch.from_numpy(rng.standard_normal([out_channels, gshape[1]] + k).astype(np.float32))
+    b = torch.from_numpy(rng.standard_normal(out_channels).astype(np.float32))
     xr, wr, br = torch.from_numpy(x).requires_grad_(True), w.clone().requires_grad_(True), b.clone().requires_grad_(True)
-    yr = F.conv2d(xr, wr, br, padding=1)
+    yr = conv(xr, wr, br, padding=padding)
     dy = rng.standard_normal(tuple(yr.shape)).astype(np.float32)
     yr.backward(torch.from_numpy(dy))
     shards, dys = o_rep.scatter(x, P), o_rep.scatter(dy, P)
 
     def body(P_world):
-        P_x = P_world.create_partition_inclusive(list(range(4))).create_cartesian_topology_partition(P)
-        layer = DistributedConv2d(P_x, in_channels=3, out_channels=4, kernel_size=k, padding=1, bias=True)
+        P_x = P_world.create_partition_inclusive(list(range(n))).create_cartesian_topology_partition(P)
+        layer = Conv(P_x, in_channels=gshape[1], out_channels=out_channels, kernel_size=k, padding=padding, bias=True)
         if P_x.rank == 0:
             with torch.no_grad():
                 layer.weight.copy_(w.cuda())
@@ -402,17 +417,21 @@ def test_feature_conv_backward_matches_sequential_conv():
         xin = torch.from_numpy(shards[P_x.rank]).cuda().requires_grad_(True)
         y = layer(xin)
         assert tuple(y.shape) == dys[P_x.rank].shape
+        if y_local is not None:
+            assert list(y.shape) == y_local
         y.backward(torch.from_numpy(dys[P_x.rank]).cuda())
         torch.cuda.synchronize()
         wg = layer.weight.grad.cpu().numpy() if P_x.rank == 0 else None
         bg = layer.bias.grad.cpu().numpy() if P_x.rank == 0 else None
-        return xin.grad.cpu().numpy(), wg, bg
+        return y.detach().cpu().numpy(), xin.grad.cpu().numpy(), wg, bg
 
-    outs = SimWorld(4).run(body)
-    for (dx, _, _), part in zip(outs, o_rep.scatter(xr.grad.numpy(), P)):
+    outs = SimWorld(n).run(body)
+    for (y, _, _, _), part in zip(outs, o_rep.scatter(yr.detach().numpy(), P)):
+        assert np.allclose(y, part, atol=1e-4, rtol=1e-4)
+    for (_, dx, _, _), part in zip(outs, o_rep.scatter(xr.grad.numpy(), P)):
         assert np.allclose(dx, part, atol=1e-4, rtol=1e-4)
-    assert np.allclose(outs[0][1], wr.grad.numpy(), atol=1e-3, rtol=1e-4)
-    assert np.allclose(outs[0][2], br.grad.numpy(), atol=1e-3, rtol=1e-4)
+    assert np.allclose(outs[0][2], wr.grad.numpy(), atol=1e-3, rtol=1e-4)
+    assert np.allclose(outs[0][3], br.grad.numpy(), atol=1e-3, rtol=1e-4)
 
 
 def test_solo_conv_staging_uses_fused_kernel_and_matches_oracle(ops):
