@@ -554,3 +554,32 @@ def test_broadcast_partner_follows_the_reference_rule():
         broadcast_partner([2, 3], [0, 0], [2, 2], [0, 0])
     with pytest.raises(TransportError):
         broadcast_partner([1, 1, 2], [0, 0, 0], [2, 2], [0, 0])
+
+
+def test_conv_selector_picks_the_feature_class_and_rejects_what_the_reference_rejects():
+    """tests/layers/test_conv.py:10-60, :88-100 (a selector given P_x alone
+    builds the feature-partitioned layer) and :200-236 (only one of P_y, P_w:
+    ValueError).  The channel-partitioned and general layers the reference
+    builds when both are given do not exist here: that request says so."""
+    from distdl_amd import nn as dnn
+    from distdl_amd.backends.stub_hip import SimWorld
+    world = SimWorld(8, device="cpu")
+    P_world = world.partition(0)
+    cases = [(dnn.DistributedConv1d, dnn.DistributedFeatureConv1d, [1, 1, 4], [3]),
+             (dnn.DistributedConv2d, dnn.DistributedFeatureConv2d, [1, 1, 2, 2], [3, 3]),
+             (dnn.DistributedConv3d, dnn.DistributedFeatureConv3d, [1, 1, 2, 2, 1], [3, 3, 3])]
+    for Selector, Feature, shape, ks in cases:
+        P_x = P_world.create_partition_inclusive(list(range(4))).create_cartesian_topology_partition(shape)
+        layer = Selector(P_x, in_channels=3, out_channels=3, kernel_size=ks)
+        assert isinstance(layer, Feature)
+    P2 = P_world.create_partition_inclusive([0, 1])
+    P4 = P_world.create_partition_inclusive([0, 1, 2, 3])
+    P_x = P2.create_cartesian_topology_partition([1, 2, 1, 1])
+    P_y = P2.create_cartesian_topology_partition([1, 2, 1, 1])
+    P_w = P4.create_cartesian_topology_partition([2, 2, 1, 1])
+    with pytest.raises(ValueError):
+        dnn.DistributedConv2d(P_x, P_y=P_y, in_channels=3, out_channels=3, kernel_size=[3, 3])
+    with pytest.raises(ValueError):
+        dnn.DistributedConv2d(P_x, P_w=P_w, in_channels=3, out_channels=3, kernel_size=[3, 3])
+    with pytest.raises(NotImplementedError):
+        dnn.DistributedConv2d(P_x, P_y=P_y, P_w=P_w, in_channels=3, out_channels=3, kernel_size=[3, 3])
