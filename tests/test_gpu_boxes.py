@@ -6,7 +6,6 @@ import numpy as np
 import pytest
 import torch
 
-from oracle import partition_math as pm
 from oracle import repartition as o_rep
 
 pytestmark = pytest.mark.gpu

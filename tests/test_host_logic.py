@@ -10,7 +10,6 @@ import numpy as np
 import pytest
 import torch
 
-import distdl_amd
 from distdl_amd import _lib
 from distdl_amd.backends.stub_hip import BufferManager
 from distdl_amd.backends.stub_hip import ExpandableBuffer
