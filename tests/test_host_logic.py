@@ -582,3 +582,33 @@ def test_conv_selector_picks_the_feature_class_and_rejects_what_the_reference_re
         dnn.DistributedConv2d(P_x, P_w=P_w, in_channels=3, out_channels=3, kernel_size=[3, 3])
     with pytest.raises(NotImplementedError):
         dnn.DistributedConv2d(P_x, P_y=P_y, P_w=P_w, in_channels=3, out_channels=3, kernel_size=[3, 3])
+
+
+def test_sum_reduce_and_broadcast_layers_with_one_live_worker():
+    """Solo transport: the peers are absent, so a reduction hands the live
+    worker its own contribution if it receives (and the reference's zero-volume
+    tensor if it only sends), and a broadcast is the identity on the owner."""
+    from distdl_amd.nn import Broadcast, SumReduce
+    for rank, receives in ((0, True), (3, False)):
+        world = SimWorld(4, device=torch.device("cpu"))
+        P_world = world.partition(rank)
+        P_w = P_world.create_partition_inclusive([0, 1, 2, 3]).create_cartesian_topology_partition([2, 2])
+        P_y = P_world.create_partition_inclusive([0, 1]).create_cartesian_topology_partition([1, 2])
+        layer = SumReduce(P_w, P_y, transpose_src=True, preserve_batch=True)
+        x = torch.arange(12.0).reshape(3, 4).requires_grad_(True)
+        y = layer(x)
+        if receives:
+            assert torch.equal(y.detach(), x.detach())
+            y.backward(torch.ones_like(y))
+            assert torch.equal(x.grad, torch.ones(3, 4))
+        else:
+            assert tuple(y.shape) == (3, 0)
+    world = SimWorld(4, device=torch.device("cpu"))
+    P_world = world.partition(0)
+    P_x = P_world.create_partition_inclusive([0, 1]).create_cartesian_topology_partition([1, 2])
+    P_w = P_world.create_partition_inclusive([0, 1, 2, 3]).create_cartesian_topology_partition([2, 2])
+    x = torch.arange(6.0).reshape(2, 3).requires_grad_(True)
+    y = Broadcast(P_x, P_w, preserve_batch=True)(x)
+    assert torch.equal(y.detach(), x.detach())
+    y.backward(2 * torch.ones_like(y))
+    assert torch.equal(x.grad, 2 * torch.ones(2, 3))
