@@ -105,6 +105,8 @@ SIGNATURES = {
                                             c_void_p, c_void_p, c_void_p]),
     "ddl_embedding_gather": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_int, c_int64, c_int64, c_int64,
                                      c_void_p, c_void_p]),
+    "ddl_embedding_renorm": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64, c_float,
+                                     c_float, c_void_p, c_void_p]),
     "ddl_embedding_backward": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64,
                                        c_int, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "ddl_embedding_backward_static": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64,

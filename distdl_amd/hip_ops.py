@@ -524,6 +524,32 @@ def embedding_gather(weight, ids, lo, hi, out=None):
     return out
 
 
+def embedding_renorm(weight, ids, lo, hi, max_norm, norm_type=2.0):
+    """The ``max_norm`` step of ``F.embedding``: the rows of ``weight`` that
+    ``ids`` name inside [lo, hi) and whose ``norm_type``-norm exceeds
+    ``max_norm`` are scaled down to it, in place."""
+    _require_gpu(weight, ids)
+    if weight.dim() != 2 or (weight.shape[1] > 1 and weight.stride(1) != 1):
+        raise ValueError("embedding_renorm: weight must be 2-D with unit column stride")
+    if weight.dtype not in _LN_DTYPES:
+        raise ValueError(f"embedding_renorm: tables are float32, bfloat16 or float16, got {weight.dtype}")
+    if ids.dtype not in (torch.int64, torch.int32):
+        raise ValueError("embedding_renorm: ids must be int32 or int64")
+    if weight.shape[0] != hi - lo:
+        raise ValueError(f"embedding_renorm: table has {weight.shape[0]} rows but the window is [{lo},{hi})")
+    if weight.shape[0] == 0 or ids.numel() == 0:
+        return weight
+    ids_c = ids.contiguous()
+    dim = weight.shape[1]
+    flags = torch.empty(weight.shape[0], dtype=torch.int32, device=weight.device)
+    rc = _lib.load().ddl_embedding_renorm(weight.data_ptr(), _LN_DTYPES[weight.dtype], dim,
+                                          weight.stride(0) if weight.shape[0] > 1 else dim, ids_c.data_ptr(),
+                                          1 if ids.dtype == torch.int64 else 0, ids_c.numel(), int(lo), int(hi),
+                                          float(max_norm), float(norm_type), flags.data_ptr(), _stream())
+    _lib.check(rc, "ddl_embedding_renorm")
+    return weight
+
+
 def embedding_backward(grad_output, ids, lo, hi, padding_idx=None, scale_grad_by_freq=False):
     """Gradient of :func:`embedding_gather` with respect to the ``[hi-lo, dim]``
     table; with ``scale_grad_by_freq`` every row's sum is divided by the number

@@ -43,8 +43,10 @@ class DistributedEmbedding(Module):
 
     Signature of the reference.  ``padding_idx`` and ``scale_grad_by_freq``
     act on the gradient as they do in ``torch.nn.functional.embedding``;
-    ``max_norm`` (in-place renormalisation of the table during the lookup) and
-    ``sparse=True`` (a sparse gradient tensor) are refused.
+    ``max_norm`` renormalises, in place and before the lookup, the rows that are
+    looked up -- every worker its own columns by their own norm, as happens when
+    the reference hands its local table to ``F.embedding``; ``sparse=True`` (a
+    sparse gradient tensor) is refused.
 
     Without ``vocab_shard`` every id must lie in ``[0, num_embeddings)``; the
     kernel does not look (an id outside yields a zero row and no gradient).
@@ -66,8 +68,6 @@ class DistributedEmbedding(Module):
             elif padding_idx < 0:
                 assert padding_idx >= -self.num_embeddings, 'Padding_idx must be within num_embeddings'
                 padding_idx = self.num_embeddings + padding_idx
-        if max_norm is not None:
-            raise NotImplementedError("max_norm renormalises the table in place; not part of this build")
         if collect_state:
             raise NotImplementedError("collect_state=True is not part of this build")
         if sparse:
@@ -151,5 +151,9 @@ class DistributedEmbedding(Module):
             lo, hi = (int(v) for v in torch.aminmax(input))
             if lo < 0 or hi >= self.num_embeddings:
                 raise IndexError(f"token ids span [{lo}, {hi}], outside the table's [0, {self.num_embeddings})")
+        if self.max_norm is not None:
+            # As F.embedding does: in place on the tensor that is looked up (every
+            # worker scales its own columns by their own norm), outside autograd.
+            hip_ops.embedding_renorm(weight.detach(), input, self.vocab_lo, self.vocab_hi, self.max_norm, self.norm_type)
         return _EmbeddingShard.apply(weight, input, self.vocab_lo, self.vocab_hi, self.padding_idx,
                                      bool(self.scale_grad_by_freq))

@@ -386,6 +386,19 @@ int ddl_embedding_gather(const void* weight, int64_t dim, int64_t ldw,
                          int64_t n_ids, int64_t lo, int64_t hi,
                          void* out, void* stream);
 
+/* The max_norm step of torch.nn.functional.embedding(input, weight, padding_idx,
+ * max_norm, norm_type, ...) (nn/embedding.py:244-246), which runs before the
+ * lookup and changes the table in place: every row that some id of the window
+ * [lo, hi) names and whose `norm_type`-norm (1, 2, +inf or any p > 0; formed in
+ * fp32) exceeds max_norm is multiplied by max_norm / (norm + 1e-7), once per
+ * row however often it is named.  `weight` is [hi-lo, dim] of `dtype`
+ * (DDL_DT_F32, DDL_DT_BF16 or DDL_DT_F16) with row stride `ldw`; `flags` is a
+ * workspace of hi-lo int32.  ids as in ddl_embedding_gather. */
+int ddl_embedding_renorm(void* weight, int dtype, int64_t dim, int64_t ldw,
+                         const void* ids, int ids_is_i64, int64_t n_ids,
+                         int64_t lo, int64_t hi, float max_norm,
+                         float norm_type, int32_t* flags, void* stream);
+
 /* Adjoint of ddl_embedding_gather with respect to the table:
  *   dweight[r, :] = sum over t with ids[t] - lo == r and ids[t] != padding_idx
  *                   of dy[t, :]                        for every r in [0, hi-lo)

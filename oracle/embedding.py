@@ -8,7 +8,8 @@ out[t] = table[ids[t]-lo] if lo <= ids[t] < hi else 0.  Rows are moved as bit
 patterns (bf16 tables are passed as uint16).
 
 Pinned by torch.nn.functional.embedding on CPU (full window) and by a
-per-token Python loop (windowed).
+per-token Python loop (windowed); ``renorm`` by torch.nn.functional.embedding
+with ``max_norm`` on CPU.
 """
 
 import numpy as np
@@ -22,6 +23,21 @@ def gather(table, ids, lo=0, hi=None):
     safe = np.where(hit, ids - lo, 0)
     out = table[safe.reshape(-1)].reshape(ids.shape + (table.shape[1],)).copy()
     out[~hit] = 0
+    return out
+
+
+def renorm(table, ids, lo, hi, max_norm, norm_type=2.0):
+    """The renormalisation torch.nn.functional.embedding performs before the
+    lookup when ``max_norm`` is given (the reference passes it through,
+    nn/embedding.py:244-246): every row that is looked up and whose p-norm
+    exceeds max_norm is multiplied by max_norm / (norm + 1e-7), once however
+    often it is looked up.  Returns the new table (float64)."""
+    out = np.asarray(table, dtype=np.float64).copy()
+    ids = np.asarray(ids).reshape(-1)
+    for row in np.unique(ids[(ids >= lo) & (ids < hi)]) - lo:
+        norm = np.linalg.norm(out[row], ord=norm_type)
+        if norm > max_norm:
+            out[row] *= max_norm / (norm + 1e-7)
     return out
 
 

@@ -768,6 +768,92 @@ def test_embedding_layer_full_window_matches_torch():
     assert torch.equal(torch.cat(outs, dim=-1), want)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("norm_type", [1.0, 2.0, 3.0, float("inf")])
+@pytest.mark.parametrize("dim,idt", [(1, torch.int64), (7, torch.int32), (64, torch.int64), (300, torch.int32), (4100, torch.int64)])
+def test_embedding_renorm_matches_oracle(ops, dtype, norm_type, dim, idt):
+    """ddl_embedding_renorm on a window of a larger vocabulary, a pitched table,
+    repeated ids and rows nobody looks up: looked-up rows above max_norm are
+    scaled once (fp32 arithmetic, one rounding to the table's type), the others
+    keep their bits."""
+    gen = torch.Generator().manual_seed(dim)
+    rows, lo = 40, 3
+    hi = lo + rows
+    store = torch.randn(rows, dim + 8, generator=gen).to(dtype)
+    table = store[:, :dim]
+    ids = torch.randint(0, hi + 6, (5, 13), generator=gen).to(idt)
+    ids[0, :4] = lo + 7                                   # one row many times
+    norms = torch.linalg.vector_norm(table.double(), ord=norm_type, dim=1)
+    ordered = norms.sort().values
+    max_norm = float((ordered[rows // 2 - 1] + ordered[rows // 2]) / 2)   # half of the rows are above, none is at it
+    want = o_emb.renorm(table.double().numpy(), ids.numpy(), lo, hi, max_norm, norm_type)
+    g_store = store.cuda()
+    ops.embedding_renorm(g_store[:, :dim], ids.cuda(), lo, hi, max_norm, norm_type)
+    got = g_store.cpu()
+    assert torch.equal(got[:, dim:], store[:, dim:])      # the pitch is not touched
+    got = got[:, :dim]
+    looked_up = sorted(set(int(i) - lo for i in ids.reshape(-1).tolist() if lo <= int(i) < hi))
+    scaled = [r for r in looked_up if float(norms[r]) > max_norm]
+    kept = [r for r in range(rows) if r not in scaled]
+    assert scaled and len(kept) > len(set(range(rows)) - set(looked_up))
+    assert torch.equal(got[kept], table[kept])
+    if dtype == torch.float32:
+        assert np.allclose(got[scaled].double().numpy(), want[scaled], rtol=2e-6, atol=0)
+    else:
+        # the fp32 scale differs from the float64 one in the last bits: at most the neighbouring value of the type
+        w = torch.from_numpy(want[scaled])
+        near = w.to(dtype).double()
+        step = (torch.nextafter(near.abs().to(dtype), torch.tensor(float("inf"), dtype=dtype)).double() - near.abs())
+        assert bool(((got[scaled].double() - w).abs() <= step * 1.001).all())
+    if dim > 1 or norm_type == 1.0:
+        after = torch.linalg.vector_norm(got[scaled].double(), ord=norm_type, dim=1)
+        assert bool((after <= max_norm * (1 + 2.0 ** -7)).all())
+
+
+def test_embedding_layer_with_max_norm_matches_torch():
+    """DistributedEmbedding(max_norm=...) on one worker against
+    torch.nn.Embedding(max_norm=...): lookup, the table afterwards (both change
+    it in place) and the gradient; on 1 x 4 workers every worker renormalises its
+    own columns by their own norm (what the reference's local F.embedding call
+    does), compared with the oracle per column block."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedEmbedding
+    torch.manual_seed(14)
+    table = torch.randn(50, 24)
+    ids = torch.randint(0, 50, (3, 11))
+    dy = torch.randn(3, 11, 24)
+    seq = torch.nn.Embedding(50, 24, max_norm=2.5, _weight=table.clone())
+    want = seq(ids)
+    want.backward(dy)
+
+    def solo(P_world):
+        P_x = P_world.create_partition_inclusive([0]).create_cartesian_topology_partition([1, 1, 1])
+        layer = DistributedEmbedding(P_x, 50, 24, max_norm=2.5, _weight=table.clone().cuda())
+        y = layer(ids.cuda())
+        y.backward(dy.cuda())
+        torch.cuda.synchronize()
+        return y.detach().cpu(), layer.weight.detach().cpu(), layer.weight.grad.cpu()
+
+    y, w_after, dw = SimWorld(1).run(solo)[0]
+    assert torch.allclose(y, want.detach(), rtol=1e-6, atol=1e-7)
+    assert torch.allclose(w_after, seq.weight.detach(), rtol=1e-6, atol=1e-7) and not torch.equal(w_after, table)
+    assert torch.allclose(dw, seq.weight.grad, rtol=1e-6, atol=1e-6)
+
+    def body(P_world):
+        P_x = P_world.create_partition_inclusive([0, 1, 2, 3]).create_cartesian_topology_partition([1, 1, 4])
+        cols = slice(6 * P_x.rank, 6 * (P_x.rank + 1))
+        layer = DistributedEmbedding(P_x, 50, 24, max_norm=1.2, norm_type=1.0, _weight=table[:, cols].clone().cuda())
+        with torch.no_grad():
+            y = layer(ids.cuda()).cpu()
+        torch.cuda.synchronize()
+        return y
+
+    outs = SimWorld(4).run(body)
+    for r, y in enumerate(outs):
+        block = o_emb.renorm(table[:, 6 * r:6 * (r + 1)].double().numpy(), ids.numpy(), 0, 50, 1.2, 1.0)
+        assert np.allclose(y.double().numpy(), o_emb.gather(block, ids.numpy(), 0, 50), rtol=2e-6, atol=1e-7)
+
+
 @pytest.mark.parametrize("P,table_shape", [([1, 1], (4, 12)), ([1, 4], (4, 12)), ([1, 3], (9, 16))])
 def test_embedding_training_step_reference_cases(P, table_shape):
     """The reference's test_batch_norm_with_training for the embedding

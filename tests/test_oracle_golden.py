@@ -434,3 +434,25 @@ def test_embedding_backward_oracle_matches_torch_autograd():
     got = o_emb.backward(dy.numpy(), ids.numpy(), 0, 20, padding_idx=3, scale_grad_by_freq=True)
     assert np.allclose(got, table2.grad.numpy(), rtol=1e-13, atol=1e-13)
     assert not np.allclose(got, table.grad.numpy())      # the option changes the answer on this input
+
+
+@pytest.mark.parametrize("norm_type", [1.0, 2.0, 3.5, float("inf")])
+def test_embedding_renorm_oracle_matches_torch(norm_type):
+    """max_norm: torch.nn.functional.embedding renormalises the looked-up rows
+    in place (repeated ids once), leaves the others alone, and the lookup then
+    returns the renormalised rows; a window renormalises its own rows only."""
+    torch.manual_seed(8)
+    table = 2 * torch.randn(30, 7, dtype=torch.float64)
+    ids = torch.tensor([[3, 3, 9, 27], [0, 9, 9, 15]])
+    want_table = table.clone()
+    want_out = F.embedding(ids, want_table, max_norm=1.5, norm_type=norm_type)
+    got = o_emb.renorm(table.numpy(), ids.numpy(), 0, 30, 1.5, norm_type)
+    assert np.allclose(got, want_table.numpy(), rtol=1e-12, atol=1e-12)
+    untouched = [r for r in range(30) if r not in (0, 3, 9, 15, 27)]
+    assert np.array_equal(got[untouched], table.numpy()[untouched])
+    assert not np.allclose(got[[3, 9]], table.numpy()[[3, 9]])            # something was scaled on this input
+    assert np.allclose(o_emb.gather(got, ids.numpy(), 0, 30), want_out.numpy(), rtol=1e-12, atol=1e-12)
+    part = o_emb.renorm(table.numpy()[5:20], ids.numpy(), 5, 20, 1.5, norm_type)
+    assert np.allclose(part[[4, 10]], want_table.numpy()[[9, 15]], rtol=1e-12, atol=1e-12)
+    rest = [r for r in range(15) if r not in (4, 10)]
+    assert np.array_equal(part[rest], table.numpy()[5:20][rest])
