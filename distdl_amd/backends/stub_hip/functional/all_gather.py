@@ -61,8 +61,9 @@ def reduce_scatter_slabs(P, full, axis, tag):
 class AllGatherFunction(torch.autograd.Function):
 
     @staticmethod
-    def forward(ctx, input, P_allgather, axis=None, tag=None):
-        if not P_allgather.active or P_allgather.size == 1:
+    def forward(ctx, input, P_allgather, axis=None, tag=None, scale_backward=None):
+        ctx.scale_backward = scale_backward
+        if P_allgather is None or not P_allgather.active or P_allgather.size == 1:
             ctx.identity = True
             return input
         ctx.identity = False
@@ -71,7 +72,10 @@ class AllGatherFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output):
+        grad_output = grad_output.detach()
+        if ctx.scale_backward is not None:
+            grad_output = grad_output / ctx.scale_backward      # before the sum (reference :188-190)
         if ctx.identity:
-            return grad_output, None, None, None
-        dx = reduce_scatter_slabs(ctx.P, grad_output.detach(), ctx.axis, ("all_gather_adjoint", ctx.tag))
-        return dx, None, None, None
+            return grad_output, None, None, None, None
+        dx = reduce_scatter_slabs(ctx.P, grad_output, ctx.axis, ("all_gather_adjoint", ctx.tag))
+        return dx, None, None, None, None

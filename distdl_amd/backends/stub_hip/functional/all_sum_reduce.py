@@ -10,8 +10,8 @@ import torch
 class AllSumReduceFunction(torch.autograd.Function):
 
     @staticmethod
-    def forward(ctx, input, P_reduce, tag=None):
-        ctx.P_reduce, ctx.tag = P_reduce, tag
+    def forward(ctx, input, P_reduce, tag=None, scale_backward=None):
+        ctx.P_reduce, ctx.tag, ctx.scale_backward = P_reduce, tag, scale_backward
         if not P_reduce.active or P_reduce.size == 1:
             return input
         parts = P_reduce._world.transport.allgather(P_reduce, input.detach(), tag=tag)
@@ -21,7 +21,10 @@ class AllSumReduceFunction(torch.autograd.Function):
     def backward(ctx, grad_output):
         # The all-sum-reduce is its own adjoint (reference :95-161).
         P_reduce = ctx.P_reduce
+        grad_output = grad_output.detach()
+        if ctx.scale_backward is not None:
+            grad_output = grad_output / ctx.scale_backward      # before the sum (reference :127-128)
         if not P_reduce.active or P_reduce.size == 1:
-            return grad_output, None, None
-        parts = P_reduce._world.transport.allgather(P_reduce, grad_output.detach().contiguous(), tag=("adjoint", ctx.tag))
-        return parts.sum(dim=0), None, None
+            return grad_output, None, None, None
+        parts = P_reduce._world.transport.allgather(P_reduce, grad_output.contiguous(), tag=("adjoint", ctx.tag))
+        return parts.sum(dim=0), None, None, None

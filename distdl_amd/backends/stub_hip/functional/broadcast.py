@@ -15,11 +15,13 @@ from ....utilities.torch import zero_volume_tensor
 class BroadcastFunction(torch.autograd.Function):
 
     @staticmethod
-    def forward(ctx, input, P_send, P_recv, preserve_batch=False, tag=None, transpose_src=False, transpose_dest=False):
+    def forward(ctx, input, P_send, P_recv, preserve_batch=False, tag=None, transpose_src=False, transpose_dest=False,
+                scale_backward=None):
         if not (P_send.active or P_recv.active):
             return input
         ctx.P_send, ctx.P_recv, ctx.tag = P_send, P_recv, tag
         ctx.transposes = (transpose_src, transpose_dest)
+        ctx.scale_backward = scale_backward
         ctx.input_like = (tuple(input.shape), input.dtype, input.device)
         world = P_send._world if P_send._world is not None else P_recv._world
         out = world.transport.broadcast(P_send, P_recv, input.detach(), transpose_src=transpose_src,
@@ -35,9 +37,13 @@ class BroadcastFunction(torch.autograd.Function):
         P_send, P_recv = ctx.P_send, ctx.P_recv
         world = P_send._world if P_send._world is not None else P_recv._world
         transpose_src, transpose_dest = ctx.transposes
-        grad = world.transport.broadcast_adjoint(P_send, P_recv, grad_output.detach(), transpose_src=transpose_src,
+        grad_output = grad_output.detach()
+        if ctx.scale_backward is not None and P_recv.active:
+            # Every receiver's gradient is divided before the sum (reference :208-209).
+            grad_output = grad_output / ctx.scale_backward
+        grad = world.transport.broadcast_adjoint(P_send, P_recv, grad_output, transpose_src=transpose_src,
                                                  transpose_dst=transpose_dest, tag=ctx.tag)
         if grad is None:
             shape, dtype, device = ctx.input_like
             grad = torch.zeros(shape, dtype=dtype, device=device)
-        return grad, None, None, None, None, None, None
+        return grad, None, None, None, None, None, None, None

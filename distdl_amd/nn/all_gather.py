@@ -16,8 +16,7 @@ class AllGather(Module):
         self.P_x = P_x
         if not P_x.active:
             return
-        if scale_backward is not None:
-            raise NotImplementedError("scale_backward is not part of this build")
+        self.scale_backward = scale_backward
         if axes_all_gather is None:
             axes_all_gather = [d for d in range(P_x.dim) if d not in [int(a) for a in axes_keep]]
         self.axes = tuple(int(a) for a in axes_all_gather)
@@ -29,9 +28,10 @@ class AllGather(Module):
         if not self.P_x.active or self.identity:
             return input
         transport = self.P_x._world.transport
+        Function = self._distdl_backend.functional.all_gather.AllGatherFunction
         if getattr(transport, "ghosts_preloaded", False):
-            return input  # solo: the input already is the gathered tensor
+            # solo: the input already is the gathered tensor; only the scaling of the gradient remains
+            return input if self.scale_backward is None else Function.apply(input, None, None, None, self.scale_backward)
         if len(self.axes) != 1:
             raise NotImplementedError("AllGather along several axes is not part of this build")
-        Function = self._distdl_backend.functional.all_gather.AllGatherFunction
-        return Function.apply(input, self.P_allgather, self.axes[0], None)
+        return Function.apply(input, self.P_allgather, self.axes[0], None, self.scale_backward)

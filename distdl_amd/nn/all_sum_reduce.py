@@ -11,6 +11,7 @@ class AllSumReduce(Module):
     def __init__(self, P_x, axes_reduce=None, axes_keep=None, scale_backward=None):
         super().__init__()
         self.P_x = P_x
+        self.scale_backward = scale_backward
         if not P_x.active:
             self.P_allreduce = None
             return
@@ -32,4 +33,4 @@ class AllSumReduce(Module):
         if not self.P_x.active or self.identity:
             return input
         Function = self._distdl_backend.functional.all_sum_reduce.AllSumReduceFunction
-        return Function.apply(input, self.P_allreduce, None)
+        return Function.apply(input, self.P_allreduce, None, self.scale_backward)

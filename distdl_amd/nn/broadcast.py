@@ -14,6 +14,7 @@ class Broadcast(Module):
         self.transpose_src = transpose_src
         self.transpose_dest = transpose_dest
         self.preserve_batch = preserve_batch
+        self.scale_backward = scale_backward
         # Source and destination are the same team: nothing moves.
         self.identity = (P_x == P_y)
 
@@ -22,4 +23,4 @@ class Broadcast(Module):
             return input
         Function = self._distdl_backend.functional.broadcast.BroadcastFunction
         return Function.apply(input, self.P_x, self.P_y, self.preserve_batch, None,
-                              self.transpose_src, self.transpose_dest)
+                              self.transpose_src, self.transpose_dest, self.scale_backward)

@@ -12,13 +12,11 @@ from .module import Module
 
 class ReduceScatter(Module):
 
-    def __init__(self, P_x, axes_reduce_scatter=None, axes_keep=None, scale_backward=None):
+    def __init__(self, P_x, axes_reduce_scatter=None, axes_keep=None):
         super().__init__()
         self.P_x = P_x
         if not P_x.active:
             return
-        if scale_backward is not None:
-            raise NotImplementedError("scale_backward is not part of this build")
         if axes_reduce_scatter is None:
             axes_reduce_scatter = [d for d in range(P_x.dim) if d not in [int(a) for a in axes_keep]]
         self.axes = tuple(int(a) for a in axes_reduce_scatter)

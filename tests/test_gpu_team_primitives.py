@@ -381,3 +381,43 @@ def test_all_sum_reduce_reference_layouts(P_shape, shape, axes):
         assert len(group) == int(np.prod([P_shape[d] for d in axes])) if axes else group == [r]
         assert np.array_equal(outs[r][0], sum(xs[s] for s in group)), f"worker {r}"
         assert np.array_equal(outs[r][1], sum(dys[s] for s in group)), f"worker {r}"
+
+
+def test_scale_backward_divides_the_gradients_before_they_are_summed():
+    """Broadcast, AllGather and AllSumReduce with ``scale_backward`` (reference:
+    backends/mpi_numpy/functional/broadcast.py:208-209, all_gather.py:188-190,
+    all_sum_reduce.py:127-128): forward unchanged, every worker's gradient
+    divided by the scalar before the adjoint's sum.  Integers and a power of two,
+    so the quotients are exact."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import AllGather, AllSumReduce, Broadcast
+    xs = _integers(4, [2, 6], 21)
+    dys = _integers(4, [2, 6], 22)
+    dgs = _integers(4, [2, 24], 23)
+
+    def body(P_world):
+        r = P_world.rank
+        P_one = P_world.create_partition_inclusive([0]).create_cartesian_topology_partition([1, 1])
+        P_all = P_world.create_partition_inclusive([0, 1, 2, 3]).create_cartesian_topology_partition([1, 4])
+        x = torch.from_numpy(xs[r]).cuda().requires_grad_(True)
+        y = Broadcast(P_one, P_all, scale_backward=4)(x)
+        y.backward(torch.from_numpy(dys[r]).cuda())
+        xa = torch.from_numpy(xs[r]).cuda().requires_grad_(True)
+        ya = AllGather(P_all, axes_all_gather=(1,), scale_backward=2)(xa)
+        ya.backward(torch.from_numpy(dgs[r]).cuda())
+        xr = torch.from_numpy(xs[r]).cuda().requires_grad_(True)
+        yr = AllSumReduce(P_all, axes_reduce=(1,), scale_backward=8)(xr)
+        yr.backward(torch.from_numpy(dys[r]).cuda())
+        torch.cuda.synchronize()
+        return (y.detach().cpu().numpy(), x.grad.cpu().numpy(), ya.detach().cpu().numpy(), xa.grad.cpu().numpy(),
+                yr.detach().cpu().numpy(), xr.grad.cpu().numpy())
+
+    outs = SimWorld(4).run(body)
+    for r, (y, dx, ya, dxa, yr, dxr) in enumerate(outs):
+        assert np.array_equal(y, xs[0])
+        if r == 0:
+            assert np.array_equal(dx, sum(dys) / 4)
+        assert np.array_equal(ya, np.concatenate(xs, axis=1))
+        assert np.array_equal(dxa, (sum(dgs) / 2)[:, 6 * r:6 * (r + 1)])
+        assert np.array_equal(yr, sum(xs))
+        assert np.array_equal(dxr, sum(dys) / 8)
