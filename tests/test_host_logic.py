@@ -521,6 +521,11 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert rc == -5
     rc = lib.ddl_embedding_gather(16, 8, 8, 3, 16, 1, 4, 0, 4, 16, None)
     assert rc == -1
+    rc = lib.ddl_embedding_renorm(16, _lib.DDL_DT_F32, 8, 8, 16, 1, 4, 0, 4, -1.0, 2.0, 16, None)     # negative max_norm
+    assert rc == -1 and b"max_norm" in lib.ddl_last_error()
+    rc = lib.ddl_embedding_renorm(16, _lib.DDL_DT_F64, 8, 8, 16, 1, 4, 0, 4, 1.0, 2.0, 16, None)      # no float64 tables
+    assert rc == -5
+    assert lib.ddl_embedding_renorm(16, _lib.DDL_DT_F32, 8, 8, 16, 1, 0, 0, 4, 1.0, 2.0, 16, None) == 0   # no ids: nothing to do
     assert lib.ddl_pack_boxes(1, shape, shape, 2, 4, 0, shape, shape, _lib.ptr_array([]), None) == 0
 
 
