@@ -617,3 +617,14 @@ def test_sum_reduce_and_broadcast_layers_with_one_live_worker():
     assert torch.equal(y.detach(), x.detach())
     y.backward(2 * torch.ones_like(y))
     assert torch.equal(x.grad, 2 * torch.ones(2, 3))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """One GPU's share is what is measured; a request for more says so and
+    exits before anything touches a device."""
+    import subprocess
+    import sys
+    done = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                          timeout=300)
+    assert done.returncode != 0
+    assert "ONE GPU" in (done.stderr + done.stdout)
