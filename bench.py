@@ -1,6 +1,6 @@
 """Benchmark of the per-rank hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--skip-layers] [--only NAMES]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--skip-layers] [--only NAMES | --all]
 
 Headline workload (BASELINE.json configs[1]): Repartition pack + unpack of one
 rank, bf16 global tensor [8,4096,8192] moved from P_x=[1,8,1] to P_y=[1,1,8].
@@ -12,7 +12,12 @@ asserted equal to the oracle's before anything is timed.  Inputs are resident
 in HBM before the timed region; a step rotates over several buffer sets so that
 the 256 MB last-level cache cannot hold the working set.  The other hot-path
 kernels (LayerNorm, Embedding, Linear GEMM, halo staging) are measured the same
-way and reported under "workloads" of the same JSON line, each with
+way and reported under "workloads" of the same JSON line, and once more, one
+short entry each, under roofline["configs"] and cpu_baseline["configs"].  A run
+without --only / --all measures the five BASELINE configurations and the few
+workloads read next to them (DEFAULT_WORKLOADS); --all adds the backward
+kernels, fp32 GEMM, slab-only halo exchange, re-layouts and MFMA probes.  Each
+workload carries
 
   roofline      algorithmic work / HIP-event time of the step's launches
   layer         microseconds per forward call of the distdl_amd.nn module that
@@ -73,6 +78,8 @@ def parse_args():
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--skip-layers", action="store_true", help="skip the module-level (host path included) timings")
     ap.add_argument("--only", default=None, help="run only these workloads, comma-separated; see WORKLOADS")
+    ap.add_argument("--all", action="store_true", help="every workload of WORKLOADS except the comparison figures "
+                    "(backward kernels, fp32 GEMM, slab-only halo, MFMA probes, ...) instead of the default set")
     ap.add_argument("--no-graph", action="store_true", help="launch on the stream instead of replaying a HIP graph")
     return ap.parse_args()
 
@@ -195,21 +202,24 @@ def _call(lib, _lib, name, args):
     return fn
 
 
-def time_layer(torch, fn, calls=200, warm=10):
-    """Microseconds per call of a module's forward: the host loop alone, and
-    with the device drained at the end (the larger of the two is what a caller
-    sees per call in steady state)."""
-    with torch.no_grad():
-        for _ in range(warm):
-            fn()
+def time_layer(torch, fn, inputs, calls=200, warm=10, grad=False):
+    """Microseconds per call of a module's forward, `fn(x)` over the inputs in
+    turn (enough of them that the last-level cache cannot hold what one round
+    touches): the host loop alone, and with the device drained at the end (the
+    larger of the two is what a caller sees per call in steady state).  With
+    `grad` the calls record for autograd (the forward of a training step)."""
+    n = len(inputs)
+    with torch.enable_grad() if grad else torch.no_grad():
+        for i in range(warm):
+            fn(inputs[i % n])
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(calls):
-            fn()
+        for i in range(calls):
+            fn(inputs[i % n])
         t1 = time.perf_counter()
         torch.cuda.synchronize()
         t2 = time.perf_counter()
-    return {"host_us_per_call": 1e6 * (t1 - t0) / calls, "us_per_call": 1e6 * (t2 - t0) / calls, "calls": calls}
+    return {"host_us": 1e6 * (t1 - t0) / calls, "us": 1e6 * (t2 - t0) / calls, "calls": calls, "inputs": n}
 
 
 def timed_cpu(fn, budget_s):
@@ -291,9 +301,9 @@ def _build_repartition_half(which):
 
 def layer_repartition(torch):
     layer, x = repartition_layer(torch)
-    rec = time_layer(torch, lambda: layer(x))
-    rec["module"] = ("Repartition(P_x=[1,8,1], P_y=[1,1,8]).forward under no_grad, rank 0 of 8, solo transport "
-                     "(one launch for 7 packs + the self copy, one for 7 unpacks)")
+    xs = [x] + [torch.empty_like(x).copy_(x) for _ in range(5)]      # 6 x 64 MiB in, as much out
+    rec = time_layer(torch, layer, xs)
+    rec["module"] = "Repartition([1,8,1]->[1,1,8]).forward, no_grad, rank 0 of 8, solo transport"
     return rec
 
 
@@ -315,8 +325,7 @@ def cpu_repartition(budget_s=12.0):
         o_rep.unpack(recv0, rbufs, (8, 4096, 1024), np.uint16)
     n, dt = timed_cpu(step, budget_s)
     return {"value": 268435456 * n / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{n} full steps of config 2 (pack 8 boxes + zero-filled unpack of 8 boxes), "
-                      f"NumPy np.copyto on uint16 views, one process standing in for rank 0, {dt:.1f} s"}
+            "sample": f"{n} full steps of config 2, np.copyto per box + zero-filled output, one process as rank 0, {dt:.1f} s"}
 
 
 # ----------------------------------------------------------------------------
@@ -434,27 +443,12 @@ def layer_layernorm(torch):
     peers = [None] + [torch.from_numpy(o_ln.partial_stats(xg[..., 256 * p:256 * (p + 1)].numpy()).astype(np.float32)).cuda()
                       for p in range(1, 4)]
     world.transport.set_gather_provider(STATS_TAG, lambda P, t: list(peers))
-    rec = time_layer(torch, lambda: layer(x))
-    rec["module"] = "DistributedLayerNorm(P_x=[1,1,4], 1024).forward under no_grad, rank 0 of 4, peers' statistics seeded"
-    xr = x.clone().requires_grad_(True)
-    grad = time_layer_grad(torch, lambda: layer(xr))
-    rec["host_us_per_call_grad_mode"] = grad["host_us_per_call"]
-    rec["us_per_call_grad_mode"] = grad["us_per_call"]
+    xs = [x] + [torch.empty_like(x).copy_(x) for _ in range(63)]     # 64 x 8 MiB in, as much out
+    rec = time_layer(torch, layer, xs, calls=256)
+    rec["module"] = "DistributedLayerNorm([1,1,4], 1024).forward, no_grad, rank 0 of 4, peers' statistics seeded"
+    grad = time_layer(torch, layer, [t.requires_grad_(True) for t in xs], calls=256, grad=True)
+    rec["host_us_grad_mode"], rec["us_grad_mode"] = grad["host_us"], grad["us"]
     return rec
-
-
-def time_layer_grad(torch, fn, calls=200, warm=10):
-    """time_layer with autograd recording (the forward of a training step)."""
-    for _ in range(warm):
-        fn()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(calls):
-        fn()
-    t1 = time.perf_counter()
-    torch.cuda.synchronize()
-    t2 = time.perf_counter()
-    return {"host_us_per_call": 1e6 * (t1 - t0) / calls, "us_per_call": 1e6 * (t2 - t0) / calls, "calls": calls}
 
 
 def cpu_layernorm(budget_s=4.0):
@@ -473,8 +467,7 @@ def cpu_layernorm(budget_s=4.0):
     peer_var = sum(((xg[..., 256 * p:256 * (p + 1)] - mean) ** 2).mean(axis=-1, keepdims=True) for p in range(1, 4))
     n, dt = timed_cpu(lambda: o_ln.forward_rank(x, peer_mean, peer_var, 4, gamma, beta, 1e-5), budget_s)
     return {"value": 25298944 * n / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{n} full steps of config 1 on rank 0 ([16,512,256] fp32): the reference's op sequence in NumPy fp32, "
-                      f"all-reduces replaced by seeded sums of the three peers, {dt:.1f} s"}
+            "sample": f"{n} full steps of config 1 on rank 0, the reference's op sequence in NumPy fp32, seeded peer sums, {dt:.1f} s"}
 
 
 # ----------------------------------------------------------------------------
@@ -505,9 +498,9 @@ def layer_embedding(torch):
     world = SimWorld(1)
     P_x = world.partition(0).create_partition_inclusive([0]).create_cartesian_topology_partition([1, 1, 1])
     layer = DistributedEmbedding(P_x, 128256, 4096, dtype=torch.bfloat16, vocab_shard=(0, 16032))
-    ids = torch.randint(0, 128256, (32, 4096), generator=torch.Generator().manual_seed(2003)).cuda()
-    rec = time_layer(torch, lambda: layer(ids), calls=50, warm=5)
-    rec["module"] = "DistributedEmbedding(128256, 4096, bf16, vocab_shard=(0,16032)).forward under no_grad, ids [32,4096]"
+    ids = [torch.randint(0, 128256, (32, 4096), generator=torch.Generator().manual_seed(2003 + s)).cuda() for s in range(4)]
+    rec = time_layer(torch, layer, ids, calls=48, warm=4)            # every call writes a new 1 GiB
+    rec["module"] = "DistributedEmbedding(128256, 4096, bf16, vocab_shard=(0,16032)).forward, no_grad, ids [32,4096]"
     return rec
 
 
@@ -523,8 +516,7 @@ def cpu_embedding(budget_s=4.0):
     nbytes = ids.size * 4096 * 2 + ids.size * 8 + n_hit * 8192
     n, dt = timed_cpu(lambda: o_emb.gather(table, ids, 0, 16032), budget_s)
     return {"value": nbytes * n / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{n} gathers of 4096 of config 3's 131072 tokens (1/32 of a step) from the [16032,4096] shard, "
-                      f"NumPy indexing on uint16 views, {dt:.1f} s"}
+            "sample": f"{n} gathers of 4096 of config 3's 131072 tokens (1/32 step), NumPy indexing, {dt:.1f} s"}
 
 
 # ----------------------------------------------------------------------------
@@ -624,10 +616,10 @@ def layer_linear(torch):
     world = SimWorld(8)
     P_y = world.partition(0).create_partition_inclusive(list(range(8))).create_cartesian_topology_partition([1, 1, 8])
     layer = DistributedLinearAllGather(P_y, 8192, 28672, dtype=torch.bfloat16)
-    x = torch.randn(4, 2048, 8192, generator=torch.Generator().manual_seed(3004)).to(torch.bfloat16).cuda()
-    rec = time_layer(torch, lambda: layer(x), calls=50, warm=5)
-    rec["module"] = ("DistributedLinearAllGather(P_y=[1,1,8], 8192, 28672, bf16).forward under no_grad, rank 0 of 8, "
-                     "x [4,2048,8192] whole on every worker")
+    xs = [torch.randn(4, 2048, 8192, generator=torch.Generator().manual_seed(3004 + s)).to(torch.bfloat16).cuda()
+          for s in range(4)]                                         # 4 x 128 MiB
+    rec = time_layer(torch, layer, xs, calls=48, warm=4)
+    rec["module"] = "DistributedLinearAllGather([1,1,8], 8192, 28672, bf16).forward, no_grad, rank 0 of 8, x whole"
     return rec
 
 
@@ -649,8 +641,7 @@ def cpu_linear(budget_s=4.0):
     except Exception:
         pass
     return {"value": 2.0 * m * 3584 * 8192 * n / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": f"{n} products of 256 of config 4's 8192 rows (1/32 of a step) with the [3584,8192] weight shard, NumPy "
-                      f"fp32 matmul (BLAS, {threads} threads) on operands converted from bf16 beforehand, {dt:.1f} s"}
+            "sample": f"{n} products of 256 of config 4's 8192 rows (1/32 step), NumPy fp32 matmul (BLAS, {threads} threads), {dt:.1f} s"}
 
 
 # ----------------------------------------------------------------------------
@@ -775,11 +766,11 @@ def layer_halo(torch):
     world = SimWorld(8)
     P_x = world.partition(0).create_partition_inclusive(list(range(8))).create_cartesian_topology_partition([1, 1, 2, 2, 2])
     layer = DistributedConv3d(P_x, in_channels=32, out_channels=4, kernel_size=3, padding=1, bias=False)
-    x = torch.randn(1, 32, 128, 128, 128, generator=torch.Generator(device="cuda").manual_seed(1005), device="cuda")
-    layer._distdl_forward_pre_hook(layer, (x,))
-    rec = time_layer(torch, lambda: layer.stage_input(x), calls=50, warm=5)
-    rec["module"] = ("DistributedConv3d(P_x=[1,1,2,2,2], kernel 3, padding 1).stage_input under no_grad, rank 0 of 8 "
-                     "(pad + exchange + crop in front of the stock convolution)")
+    gen = torch.Generator(device="cuda").manual_seed(1005)
+    xs = [torch.randn(1, 32, 128, 128, 128, generator=gen, device="cuda") for _ in range(3)]     # 3 x 256 MiB
+    layer._distdl_forward_pre_hook(layer, (xs[0],))
+    rec = time_layer(torch, layer.stage_input, xs, calls=48, warm=6)
+    rec["module"] = "DistributedConv3d([1,1,2,2,2], kernel 3, padding 1).stage_input (pad + exchange + crop), no_grad, rank 0 of 8"
     return rec
 
 
@@ -798,8 +789,7 @@ def cpu_halo(budget_s=4.0):
         ghosts.append([None, rng.standard_normal([s.stop - s.start for s in rgs], dtype=np.float32) if RANK0[d][1] else None])
     n, dt = timed_cpu(lambda: o_halo.pad_exchange_single(x, PAD5, RANK0, RANK0, ghosts), budget_s)
     return {"value": 562531072 * n / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{n} full steps of config 5 on rank 0 ([1,32,128^3] fp32, 3 + 3 slabs): np.pad, then per dimension "
-                      f"pack the bulk slabs and unpack the ghost slabs, NumPy, {dt:.1f} s"}
+            "sample": f"{n} full steps of config 5 on rank 0 (3 + 3 slabs): np.pad, per dimension pack bulk / unpack ghosts, {dt:.1f} s"}
 
 
 # ----------------------------------------------------------------------------
@@ -958,29 +948,56 @@ def build_calib(torch, lib, _lib, nsets):
     return steps, keep, 2 * (64 << 20)
 
 
+_PROBES = [None]
+
+
+def probes_lib():
+    """The benchmark's own helper library (an empty kernel and an MFMA-only
+    kernel; distdl_amd/csrc/bench_probes.hip), not part of the product library."""
+    if _PROBES[0] is None:
+        path = os.path.join(ROOT, "distdl_amd", "libdistdl_bench_probes.so")
+        if not os.path.exists(path):
+            raise SystemExit(f"bench.py: {path} is not built; run `make -C distdl_amd/csrc`")
+        probes = ctypes.CDLL(path)
+        probes.bench_probe_launch.restype = ctypes.c_int
+        probes.bench_probe_launch.argtypes = [ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+        probes.bench_probe_mfma.restype = ctypes.c_int
+        probes.bench_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int64,
+                                            ctypes.POINTER(ctypes.c_int64), ctypes.c_void_p]
+        _PROBES[0] = probes
+    return _PROBES[0]
+
+
+def _probe_call(name, args):
+    def fn(a=args, f=getattr(probes_lib(), name), n=name):
+        rc = f(*a, STREAM[0])
+        if rc:
+            raise RuntimeError(f"{n} failed with code {rc}")
+    return fn
+
+
 def build_launch_floor(torch, lib, _lib, nsets):
     """A kernel that does nothing, launched with the grid of config 1's
     LayerNorm kernels (2048 workgroups of 256 threads) and replayed from the
     same kind of graph: the time a launch costs on its own.  `work` is zero
     bytes; only the time per launch means anything."""
-    steps = [[_call(lib, _lib, "ddl_probe_launch", (2048, 256)), _call(lib, _lib, "ddl_probe_launch", (2048, 256))]
+    steps = [[_probe_call("bench_probe_launch", (2048, 256)), _probe_call("bench_probe_launch", (2048, 256))]
              for _ in range(nsets)]
     return steps, [], 0
 
 
 def _build_mfma_probe(instruction, random):
     def build(torch, lib, _lib, nsets):
-        """Nothing but MFMAs on register operands (ddl_probe_mfma): what the matrix
+        """Nothing but MFMAs on register operands (bench_probe_mfma): what the matrix
         cores of this machine sustain with this instruction on this kind of data,
         the ceiling the shard GEMM's figure is read against."""
         sink = torch.empty(512 * 256, device="cuda")
         flop = ctypes.c_int64(0)
         iters = 4000
         args = (instruction, random, iters, sink.data_ptr(), sink.numel(), ctypes.byref(flop))
-        rc = lib.ddl_probe_mfma(*args, STREAM[0])
-        _lib.check(rc, "ddl_probe_mfma")
+        _probe_call("bench_probe_mfma", args)()
         torch.cuda.synchronize()
-        return [[_call(lib, _lib, "ddl_probe_mfma", args)] for _ in range(nsets)], [sink, flop], int(flop.value)
+        return [[_probe_call("bench_probe_mfma", args)] for _ in range(nsets)], [sink, flop], int(flop.value)
     return build
 
 
@@ -1020,6 +1037,10 @@ WORKLOADS = {
     "linear_f32_library": (_build_linear_f32(True), 2, 1, "mfma_f32", None, None, None, None),
     "calib": (build_calib, 4, 1, "hbm", None, None, None, None),
 }
+# What a run without --only / --all measures: the five BASELINE configurations and the secondaries read next to them.
+DEFAULT_WORKLOADS = ("repartition", "layernorm", "layernorm_joined", "embedding", "linear", "halo", "halo_interior",
+                     "launch_floor")
+# Never part of --all (comparison figures through other libraries, counter calibration): only with --only.
 ONLY_ON_REQUEST = ("layernorm_local_bwd_two_passes", "linear_library", "linear_bwd_transposed", "linear_f32_library", "calib")
 
 
@@ -1055,7 +1076,12 @@ def main():
     lib = _lib.load()
     use_graph = not args.no_graph
 
-    names = [n.strip() for n in args.only.split(",")] if args.only else [n for n in WORKLOADS if n not in ONLY_ON_REQUEST]
+    if args.only:
+        names = [n.strip() for n in args.only.split(",")]
+    elif args.all:
+        names = [n for n in WORKLOADS if n not in ONLY_ON_REQUEST]
+    else:
+        names = list(DEFAULT_WORKLOADS)
     for n in names:
         if n not in WORKLOADS:
             raise SystemExit(f"bench.py: unknown workload {n!r}; choose from {', '.join(WORKLOADS)}")
@@ -1083,24 +1109,53 @@ def main():
             "mode": m["mode"], "work_per_step": work, "launches_per_step": launches, "us_per_launch": 1e6 * m["launch_s"],
             "baseline_config": config,
             "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
-                         "traffic": traffic,
-                         "traffic_source": f"profiles/{name}_hbm_traffic_pmc.txt (earlier rocprofv3 --pmc runs, not this run)"
-                         if traffic is not None else None},
+                         "traffic": traffic},
         }
-        if name == "layernorm_joined":
-            # the same step counted with config 1's algorithmic bytes (x read by both halves), for comparison with `layernorm`
-            results[name]["roofline"]["frac_of_config1_bytes"] = 25298944 / (m["launch_s"] * launches) / 1e9 / HBM_PEAK_GBS
+        if traffic is not None:
+            results[name]["roofline"]["traffic_source"] = f"profiles/{name}_hbm_traffic_pmc.txt (not this run)"
         del step_fns, keep
         torch.cuda.empty_cache()
         if layer_fn is not None and not args.skip_layers:
             rec = layer_fn(torch)
-            rec["kernel_us_per_step"] = 1e6 * m["launch_s"] * launches
+            rec["kernel_us"] = 1e6 * m["launch_s"] * launches
             results[name]["layer"] = rec
             torch.cuda.empty_cache()
         if cpu_fn is not None and not args.skip_cpu:
             results[name]["cpu_baseline"] = cpu_fn()
 
+    # Config 1 is small enough that what a launch costs by itself is a large part of its time: next to the plain
+    # fraction, the one computed on (time of the step's launches - time of as many empty launches of the same grid).
+    if "launch_floor" in results:
+        floor_us = results["launch_floor"]["us_per_launch"]
+        for name in ("layernorm", "layernorm_joined"):
+            if name in results:
+                r = results[name]
+                us = r["us_per_launch"] * r["launches_per_step"]
+                above = us - floor_us * r["launches_per_step"]
+                r["roofline"]["launch_floor_us"] = floor_us
+                if above > 0:
+                    r["roofline"]["frac_above_launch_floor"] = r["work_per_step"] / (above * 1e-6) / 1e9 / HBM_PEAK_GBS
+    if "layernorm_joined" in results:
+        # The same step counted with config 1's algorithmic bytes (x read by both halves): the path the layer takes for
+        # config 1 under the solo transport, where the peers' statistics are in memory beforehand.
+        r = results["layernorm_joined"]
+        r["roofline"]["frac_of_config1_bytes"] = 25298944 / (r["us_per_launch"] * 1e-6) / 1e9 / HBM_PEAK_GBS
+
     head = results[head_name]
+    # One entry per workload, small enough to survive in a truncated record: fraction of the roofline, time of one
+    # step's launches by HIP events, throughput by wall clock.
+    table = {}
+    for name, r in results.items():
+        key = f"cfg{r['baseline_config']}_{name}" if r["baseline_config"] else name
+        table[key] = {"frac": r["roofline"]["frac"], "us": r["us_per_launch"] * r["launches_per_step"], "value": r["value"],
+                      "unit": r["unit"], "ms_per_step": r["ms_per_step"]}
+        for extra in ("frac_above_launch_floor", "frac_of_config1_bytes"):
+            if extra in r["roofline"]:
+                table[key][extra] = r["roofline"][extra]
+        if "layer" in r:
+            table[key]["layer_us"] = r["layer"]["us"]
+    roofline = dict(head["roofline"])
+    roofline["configs"] = table
     line = {
         "metric": "Repartition pack+unpack GB/s (rank 0, bf16 [8,4096,8192], P_x=[1,8,1] -> P_y=[1,1,8])"
         if head_name == "repartition" else head_name,
@@ -1112,14 +1167,28 @@ def main():
                    if head_name == "repartition" else head_name,
                    "launch_mode": head["mode"], "buffer_sets": WORKLOADS[head_name][1],
                    "box_lists": "distdl_amd.nn.Repartition set-up (rank 0 of 8), asserted equal to the oracle's plan"},
-        "roofline": head["roofline"],
-        "workloads": results,
+        "roofline": roofline,
     }
     if "cpu_baseline" in head:
-        line["cpu_baseline"] = head["cpu_baseline"]
+        cpu = dict(head["cpu_baseline"])
+        cpu["configs"] = {f"cfg{r['baseline_config']}_{name}": {k: r["cpu_baseline"][k] for k in ("value", "unit", "cores")}
+                          for name, r in results.items() if "cpu_baseline" in r}
+        line["cpu_baseline"] = cpu
     if not args.skip_cpu:
         line["cpu_host"] = cpu_host()
-    print(json.dumps(line))
+    line["workloads"] = results
+    print(json.dumps(compact(line)))
+
+
+def compact(obj):
+    """Floats to five significant digits: the line stays short enough to be kept whole."""
+    if isinstance(obj, float):
+        return float(f"{obj:.5g}")
+    if isinstance(obj, dict):
+        return {k: compact(v) for k, v in obj.items()}
+    if isinstance(obj, (list, tuple)):
+        return [compact(v) for v in obj]
+    return obj
 
 
 if __name__ == "__main__":

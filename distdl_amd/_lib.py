@@ -65,8 +65,6 @@ SIGNATURES = {
     "ddl_halo_pad_exchange": (c_int, [c_void_p, c_void_p, POINTER(c_int64), c_int, c_int, POINTER(c_int64),
                                       POINTER(c_int64), POINTER(c_int64), POINTER(c_void_p), POINTER(c_void_p),
                                       c_int, c_void_p]),
-    "ddl_probe_launch": (c_int, [c_int64, c_int, c_void_p]),
-    "ddl_probe_mfma": (c_int, [c_int, c_int, c_int, c_void_p, c_int64, POINTER(c_int64), c_void_p]),
     "ddl_ln_partial_stats": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "ddl_ln_normalize_affine": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, POINTER(c_int64),
                                         c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),

@@ -7,7 +7,7 @@ output by one launch of the box kernel, uneven pieces included.  The adjoint is
 a reduce-scatter: every worker sums its slab of all workers' gradients
 (strided reads, accumulating box copies)."""
 
-__all__ = ["AllGatherFunction", "gather_slabs", "reduce_scatter_slabs"]
+__all__ = ["AllGatherFunction", "gather_slabs", "reduce_scatter_slabs", "single_axis"]
 
 import numpy as np
 import torch
@@ -58,17 +58,31 @@ def reduce_scatter_slabs(P, full, axis, tag):
     return out
 
 
+def single_axis(axes, who):
+    """The one tensor axis a re-layout runs along (the reference's layers pass
+    a tuple of axes; its einops pattern handles one, all_gather.py:126-149)."""
+    axes = [int(a) for a in np.atleast_1d(np.asarray(axes))]
+    if len(axes) != 1:
+        raise NotImplementedError(f"{who} along several axes is not part of this build")
+    return axes[0]
+
+
 class AllGatherFunction(torch.autograd.Function):
+    """Positional arguments as in the reference
+    (backends/mpi_numpy/functional/all_gather.py:36-37).  The tensor structures
+    are accepted and not needed: the output shape follows from the gathered
+    pieces.  ``P_allgather`` None stands for a gather already done by the
+    caller (solo transport): only the scaling of the gradient remains."""
 
     @staticmethod
-    def forward(ctx, input, P_allgather, axis=None, tag=None, scale_backward=None):
+    def forward(ctx, input, P_allgather, input_tensor_structure, output_tensor_structure, axes, scale_backward):
         ctx.scale_backward = scale_backward
         if P_allgather is None or not P_allgather.active or P_allgather.size == 1:
             ctx.identity = True
             return input
         ctx.identity = False
-        ctx.P, ctx.axis, ctx.tag = P_allgather, int(axis), tag
-        return gather_slabs(P_allgather, input.detach(), int(axis), ("all_gather", tag))
+        ctx.P, ctx.axis = P_allgather, single_axis(axes, "AllGather")
+        return gather_slabs(P_allgather, input.detach(), ctx.axis, ("all_gather", None))
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -76,6 +90,6 @@ class AllGatherFunction(torch.autograd.Function):
         if ctx.scale_backward is not None:
             grad_output = grad_output / ctx.scale_backward      # before the sum (reference :188-190)
         if ctx.identity:
-            return grad_output, None, None, None, None
-        dx = reduce_scatter_slabs(ctx.P, grad_output, ctx.axis, ("all_gather_adjoint", ctx.tag))
-        return dx, None, None, None, None
+            return grad_output, None, None, None, None, None
+        dx = reduce_scatter_slabs(ctx.P, grad_output, ctx.axis, ("all_gather_adjoint", None))
+        return dx, None, None, None, None, None

@@ -5,20 +5,36 @@ transport (identity for a solo rank that owns the data; copies between rank
 threads, summed with the box kernel, under loopback) so that layers storing
 weights on a sub-grid work end to end, gradients included."""
 
-__all__ = ["BroadcastFunction"]
+__all__ = ["BroadcastFunction", "route_of"]
 
 import torch
 
 from ....utilities.torch import zero_volume_tensor
 
 
+def route_of(P_send, P_recv, kind):
+    """The two Cartesian partitions and transposes behind a (P_send, P_recv)
+    pair made by ``create_broadcast_partition_to`` / ``create_reduction_partition_to``."""
+    route = getattr(P_send, "_route", None) or getattr(P_recv, "_route", None)
+    if route is None or route.kind != kind:
+        raise ValueError(f"P_send / P_recv were not made by this backend's create_{kind}_partition_to")
+    return route
+
+
 class BroadcastFunction(torch.autograd.Function):
+    """Positional arguments as in the reference (:32-34).  ``P_send`` and
+    ``P_recv`` come from ``P_x.create_broadcast_partition_to(P_y, ...)`` and carry
+    the partitions and transposes the transport needs; the tensor structures
+    are accepted and not needed."""
 
     @staticmethod
-    def forward(ctx, input, P_send, P_recv, preserve_batch=False, tag=None, transpose_src=False, transpose_dest=False,
-                scale_backward=None):
+    def forward(ctx, input, P_send, P_recv, preserve_batch, input_tensor_structure, output_tensor_structure,
+                scale_backward):
         if not (P_send.active or P_recv.active):
             return input
+        route = route_of(P_send, P_recv, "broadcast")
+        P_send, P_recv, tag = route.P_src, route.P_dest, None
+        transpose_src, transpose_dest = route.transpose_src, route.transpose_dest
         ctx.P_send, ctx.P_recv, ctx.tag = P_send, P_recv, tag
         ctx.transposes = (transpose_src, transpose_dest)
         ctx.scale_backward = scale_backward
@@ -46,4 +62,4 @@ class BroadcastFunction(torch.autograd.Function):
         if grad is None:
             shape, dtype, device = ctx.input_like
             grad = torch.zeros(shape, dtype=dtype, device=device)
-        return grad, None, None, None, None, None, None, None
+        return grad, None, None, None, None, None, None

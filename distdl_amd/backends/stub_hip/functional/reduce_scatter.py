@@ -10,22 +10,26 @@ import torch
 
 from .all_gather import gather_slabs
 from .all_gather import reduce_scatter_slabs
+from .all_gather import single_axis
 
 
 class ReduceScatterFunction(torch.autograd.Function):
+    """Positional arguments as in the reference
+    (backends/mpi_numpy/functional/reduce_scatter.py:35-37); the tensor
+    structures are accepted and not needed."""
 
     @staticmethod
-    def forward(ctx, input, P_reducescatter, axis=None, tag=None):
+    def forward(ctx, input, P_reducescatter, input_tensor_structure, output_tensor_structure, axes):
         if not P_reducescatter.active or P_reducescatter.size == 1:
             ctx.identity = True
             return input
         ctx.identity = False
-        ctx.P, ctx.axis, ctx.tag = P_reducescatter, int(axis), tag
-        return reduce_scatter_slabs(P_reducescatter, input.detach(), int(axis), ("reduce_scatter", tag))
+        ctx.P, ctx.axis = P_reducescatter, single_axis(axes, "ReduceScatter")
+        return reduce_scatter_slabs(P_reducescatter, input.detach(), ctx.axis, ("reduce_scatter", None))
 
     @staticmethod
     def backward(ctx, grad_output):
         if ctx.identity:
-            return grad_output, None, None, None
-        dx = gather_slabs(ctx.P, grad_output.detach(), ctx.axis, ("reduce_scatter_adjoint", ctx.tag))
-        return dx, None, None, None
+            return grad_output, None, None, None, None
+        dx = gather_slabs(ctx.P, grad_output.detach(), ctx.axis, ("reduce_scatter_adjoint", None))
+        return dx, None, None, None, None

@@ -11,6 +11,7 @@ __all__ = ["SumReduceFunction"]
 import torch
 
 from ....utilities.torch import zero_volume_tensor
+from .broadcast import route_of
 
 
 def _world_of(P_send, P_recv):
@@ -18,11 +19,17 @@ def _world_of(P_send, P_recv):
 
 
 class SumReduceFunction(torch.autograd.Function):
+    """Positional arguments as in the reference (:32-34).  ``P_send`` and
+    ``P_recv`` come from ``P_x.create_reduction_partition_to(P_y, ...)``; the
+    tensor structures are accepted and not needed."""
 
     @staticmethod
-    def forward(ctx, input, P_send, P_recv, preserve_batch=True, tag=None, transpose_src=False, transpose_dest=False):
+    def forward(ctx, input, P_send, P_recv, preserve_batch, input_tensor_structure, output_tensor_structure):
         if not (P_send.active or P_recv.active):
             return input
+        route = route_of(P_send, P_recv, "reduction")
+        P_send, P_recv, tag = route.P_src, route.P_dest, None
+        transpose_src, transpose_dest = route.transpose_src, route.transpose_dest
         ctx.P_send, ctx.P_recv, ctx.tag = P_send, P_recv, tag
         ctx.transposes = (transpose_src, transpose_dest)
         ctx.input_like = (tuple(input.shape), input.dtype, input.device)
@@ -46,4 +53,4 @@ class SumReduceFunction(torch.autograd.Function):
             tag=("sum-reduce-adjoint", ctx.tag))
         if not P_send.active:
             grad = torch.zeros(shape, dtype=dtype, device=device)
-        return grad, None, None, None, None, None, None
+        return grad, None, None, None, None, None

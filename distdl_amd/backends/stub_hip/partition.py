@@ -143,6 +143,24 @@ class Partition:
             raise Exception(f"Cartesian shape {shape.tolist()} does not match a team of {len(self._ranks)}")
         return CartesianPartition(self._world, self._ranks, self._me, shape, device=self.device)
 
+    def create_broadcast_partition_to(self, P_dest, transpose_src=False, transpose_dest=False,
+                                      initialize_backend_comm=False):
+        """``(P_send, P_recv)`` of a broadcast from this partition to ``P_dest``
+        (reference :490-632).  The reference builds one communicator per source
+        worker; here both partitions are the union of the two teams seen from
+        this worker -- ``P_send`` active on the workers of the source, ``P_recv``
+        on those of the destination -- and carry the route (the two Cartesian
+        partitions and their transposes), from which the transport finds every
+        worker's partner by the reference's broadcast rule."""
+        return _route_partitions(Route("broadcast", self, P_dest, bool(transpose_src), bool(transpose_dest)))
+
+    def create_reduction_partition_to(self, P_dest, transpose_src=False, transpose_dest=False,
+                                      initialize_backend_comm=False):
+        """``(P_send, P_recv)`` of a sum-reduction from this partition onto
+        ``P_dest`` (reference :683-823): the broadcast rule read backwards, this
+        partition being the larger one."""
+        return _route_partitions(Route("reduction", self, P_dest, bool(transpose_src), bool(transpose_dest)))
+
     # -- small host data exchanges -------------------------------------------
 
     def _next_seq(self, kind):
@@ -232,7 +250,45 @@ class CartesianPartition(Partition):
             ranks.append(self._ranks[self._rank_of(full)])
         return CartesianPartition(self._world, tuple(ranks), self._me, sub_shape, device=self.device)
 
+    def create_allreduction_partition(self, axes_reduce, initialize_backend_comm=False):
+        """The workers that share this worker's index outside ``axes_reduce``,
+        in row-major order of the reduced axes, with extent 1 in every other
+        dimension (reference :634-681)."""
+        if not self.active:
+            return Partition(self._world, None, self._me, device=self.device)
+        axes = [int(a) for a in axes_reduce]
+        for a in axes:
+            if a >= self.dim:
+                raise ValueError(f"Dimension {a} in axes_reduce exceeds partition dimesion.")
+        sub = self.create_cartesian_subtopology_partition([d in axes for d in range(self.dim)])
+        shape = [int(self.shape[d]) if d in axes else 1 for d in range(self.dim)]
+        return CartesianPartition(self._world, sub._ranks, self._me, shape, device=self.device)
+
     # Geometry of the team seen from any member; used by the solo transport to
     # answer for absent peers.
     def index_of_rank(self, rank):
         return np.asarray(np.unravel_index(int(rank), tuple(int(s) for s in self.shape)), dtype=int)
+
+
+class Route:
+    """What a pair of broadcast / reduction partitions stands for: data moves
+    from ``P_src`` to ``P_dest`` (``kind`` "broadcast": copies from the smaller
+    partition; "reduction": sums onto the smaller one), either partition
+    transposed first."""
+
+    __slots__ = ("kind", "P_src", "P_dest", "transpose_src", "transpose_dest")
+
+    def __init__(self, kind, P_src, P_dest, transpose_src, transpose_dest):
+        self.kind, self.P_src, self.P_dest = kind, P_src, P_dest
+        self.transpose_src, self.transpose_dest = transpose_src, transpose_dest
+
+
+def _route_partitions(route):
+    P_src, P_dest = route.P_src, route.P_dest
+    world = P_src._world if P_src._world is not None else P_dest._world
+    me = P_src._me if P_src._me is not None else P_dest._me
+    union = tuple(P_src._group()) + tuple(r for r in P_dest._group() if r not in P_src._group())
+    P_send = Partition(world, union if P_src.active else None, me, device=P_src.device)
+    P_recv = Partition(world, union if P_dest.active else None, me, device=P_dest.device)
+    P_send._route = P_recv._route = route
+    return P_send, P_recv

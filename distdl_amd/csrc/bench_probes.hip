@@ -1,8 +1,25 @@
-// Measurement aids (no counterpart in the reference): kernels that isolate one
-// cost so that the figures the other kernels are judged against -- what a
-// launch costs by itself, what the matrix cores sustain on a given kind of data
-// -- are measured on the same machine, in the same way, as those kernels.
-#include "ddl_common.h"
+// Measurement aids of the benchmark (no counterpart in the reference, and not
+// part of libdistdl_hip or its header): kernels that isolate one cost so that
+// the figures the product's kernels are judged against -- what a launch costs
+// by itself, what the matrix cores sustain on a given kind of data -- are
+// measured on the same machine, in the same way, as those kernels.  Built as
+// libdistdl_bench_probes.so, which only bench.py loads.
+//
+//   int bench_probe_launch(int64_t workgroups, int threads, void* stream)
+//       enqueues a kernel that does nothing: the floor under every small kernel
+//   int bench_probe_mfma(int instruction, int random, int iters, float* sink,
+//                        int64_t sink_elems, int64_t* flop, void* stream)
+//       enqueues a kernel of nothing but bf16 MFMAs on register operands (512
+//       workgroups of 256 threads: two wavefronts per SIMD on 256 CUs);
+//       instruction 0: v_mfma_f32_32x32x16_bf16, 1: v_mfma_f32_16x16x32_bf16;
+//       random 0: every operand element 1.0, 1: N(0,1) x 0.02 N(0,1) operands
+//       (on random operands the chip runs against its power limit); `iters`
+//       loop iterations of 2^20 flop per wavefront, the flop count of the launch
+//       is stored to the host address `flop` (may be NULL); `sink`: device
+//       memory for 131072 floats that the kernel overwrites.
+// Both return 0, -2 for a bad argument, or the hipError_t of the launch.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
 namespace ddl {
 namespace {
@@ -100,25 +117,23 @@ __global__ __launch_bounds__(kProbeThreads) void mfma_probe_16x16x32(float* sink
 
 extern "C" {
 
-int ddl_probe_launch(int64_t workgroups, int threads, void* stream) {
-    if (workgroups < 1 || workgroups > 0x7FFFFFFFll || threads < 1 || threads > 1024)
-        return ddl::fail(DDL_E_ARG, "probe: %lld workgroups of %d threads", (long long)workgroups, threads);
+int bench_probe_launch(int64_t workgroups, int threads, void* stream) {
+    if (workgroups < 1 || workgroups > 0x7FFFFFFFll || threads < 1 || threads > 1024) return -2;
     hipLaunchKernelGGL(ddl::probe_kernel, dim3(static_cast<uint32_t>(workgroups)), dim3(threads), 0, static_cast<hipStream_t>(stream));
-    return ddl::check_launch("probe_kernel");
+    return static_cast<int>(hipGetLastError());
 }
 
-int ddl_probe_mfma(int instruction, int random, int iters, float* sink, int64_t sink_elems, int64_t* flop, void* stream) {
+int bench_probe_mfma(int instruction, int random, int iters, float* sink, int64_t sink_elems, int64_t* flop, void* stream) {
     using namespace ddl;
-    if ((instruction != 0 && instruction != 1) || iters < 1 || iters > (1 << 24)) return fail(DDL_E_ARG, "mfma probe: instruction %d, iters %d", instruction, iters);
-    if (!sink || sink_elems < static_cast<int64_t>(kProbeBlocks) * kProbeThreads)
-        return fail(DDL_E_ARG, "mfma probe: sink must hold %d floats", kProbeBlocks * kProbeThreads);
+    if ((instruction != 0 && instruction != 1) || iters < 1 || iters > (1 << 24)) return -2;
+    if (!sink || sink_elems < static_cast<int64_t>(kProbeBlocks) * kProbeThreads) return -2;
     if (flop) *flop = static_cast<int64_t>(kProbeBlocks) * (kProbeThreads / 64) * iters * kProbeFlopPerWaveIter;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (instruction == 0)
         hipLaunchKernelGGL(mfma_probe_32x32x16, dim3(kProbeBlocks), dim3(kProbeThreads), 0, s, sink, iters, random ? 1 : 0);
     else
         hipLaunchKernelGGL(mfma_probe_16x16x32, dim3(kProbeBlocks), dim3(kProbeThreads), 0, s, sink, iters, random ? 1 : 0);
-    return check_launch("mfma_probe");
+    return static_cast<int>(hipGetLastError());
 }
 
 }  // extern "C"

@@ -6,6 +6,7 @@ reduce-scatter adjoint)."""
 
 import numpy as np
 
+from ..utilities.torch import TensorStructure
 from .module import Module
 
 
@@ -20,8 +21,8 @@ class AllGather(Module):
         if axes_all_gather is None:
             axes_all_gather = [d for d in range(P_x.dim) if d not in [int(a) for a in axes_keep]]
         self.axes = tuple(int(a) for a in axes_all_gather)
-        keep = [d in self.axes for d in range(P_x.dim)]
-        self.P_allgather = P_x.create_cartesian_subtopology_partition(keep)
+        self.axes_all_gather = self.axes
+        self.P_allgather = P_x.create_allreduction_partition(self.axes)
         self.identity = int(np.prod(self.P_allgather.shape)) == 1
 
     def forward(self, input):
@@ -31,7 +32,8 @@ class AllGather(Module):
         Function = self._distdl_backend.functional.all_gather.AllGatherFunction
         if getattr(transport, "ghosts_preloaded", False):
             # solo: the input already is the gathered tensor; only the scaling of the gradient remains
-            return input if self.scale_backward is None else Function.apply(input, None, None, None, self.scale_backward)
-        if len(self.axes) != 1:
-            raise NotImplementedError("AllGather along several axes is not part of this build")
-        return Function.apply(input, self.P_allgather, self.axes[0], None, self.scale_backward)
+            if self.scale_backward is None:
+                return input
+            return Function.apply(input, None, TensorStructure(input), TensorStructure(input), self.axes, self.scale_backward)
+        # Positional arguments as in the reference (nn/all_gather.py:182-187).
+        return Function.apply(input, self.P_allgather, TensorStructure(input), None, self.axes, self.scale_backward)

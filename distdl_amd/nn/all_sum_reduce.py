@@ -3,6 +3,7 @@ tensor over the workers that share every Cartesian index outside ``axes_reduce``
 
 import numpy as np
 
+from ..utilities.torch import TensorStructure
 from .module import Module
 
 
@@ -23,14 +24,14 @@ class AllSumReduce(Module):
         if axes_reduce is None:
             axes_reduce = [d for d in dims if d not in [int(a) for a in axes_keep]]
         self.axes_reduce = tuple(int(a) for a in axes_reduce)
-        keep = [d in self.axes_reduce for d in dims]
-        # Sub-grid of the workers this worker reduces with, row-major over the
-        # reduced axes.
-        self.P_allreduce = P_x.create_cartesian_subtopology_partition(keep)
+        # The workers this worker reduces with, row-major over the reduced axes.
+        self.P_allreduce = P_x.create_allreduction_partition(self.axes_reduce)
         self.identity = int(np.prod(self.P_allreduce.shape)) == 1
 
     def forward(self, input):
         if not self.P_x.active or self.identity:
             return input
         Function = self._distdl_backend.functional.all_sum_reduce.AllSumReduceFunction
-        return Function.apply(input, self.P_allreduce, None, self.scale_backward)
+        # Positional arguments as in the reference (nn/all_sum_reduce.py:174-178).
+        structure = TensorStructure(input)
+        return Function.apply(input, self.P_allreduce, structure, structure, self.scale_backward)

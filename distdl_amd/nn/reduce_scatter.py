@@ -7,6 +7,7 @@ number of workers."""
 
 import numpy as np
 
+from ..utilities.torch import TensorStructure
 from .module import Module
 
 
@@ -20,14 +21,13 @@ class ReduceScatter(Module):
         if axes_reduce_scatter is None:
             axes_reduce_scatter = [d for d in range(P_x.dim) if d not in [int(a) for a in axes_keep]]
         self.axes = tuple(int(a) for a in axes_reduce_scatter)
-        keep = [d in self.axes for d in range(P_x.dim)]
-        self.P_reducescatter = P_x.create_cartesian_subtopology_partition(keep)
+        self.axes_reduce_scatter = self.axes
+        self.P_reducescatter = P_x.create_allreduction_partition(self.axes)
         self.identity = int(np.prod(self.P_reducescatter.shape)) == 1
 
     def forward(self, input):
         if not self.P_x.active or self.identity:
             return input
-        if len(self.axes) != 1:
-            raise NotImplementedError("ReduceScatter along several axes is not part of this build")
         Function = self._distdl_backend.functional.reduce_scatter.ReduceScatterFunction
-        return Function.apply(input, self.P_reducescatter, self.axes[0], None)
+        # Positional arguments as in the reference (nn/reduce_scatter.py:177-182).
+        return Function.apply(input, self.P_reducescatter, TensorStructure(input), None, self.axes)

@@ -3,6 +3,7 @@ held on ``P_x`` are summed onto ``P_y`` along the dimensions in which ``P_y`` ha
 one worker, by the reference's broadcast rules read backwards.  The collective
 itself is outside this build; see backends/stub_hip/functional/sum_reduce.py."""
 
+from ..utilities.torch import TensorStructure
 from .module import Module
 
 
@@ -17,10 +18,13 @@ class SumReduce(Module):
         self.preserve_batch = preserve_batch
         # Source and destination are the same team: nothing is added.
         self.identity = (P_x == P_y)
+        self.P_send = self.P_recv = None
+        if not self.identity and (P_x.active or P_y.active):
+            self.P_send, self.P_recv = P_x.create_reduction_partition_to(P_y, transpose_src, transpose_dest)
 
     def forward(self, input):
         if self.identity or not (self.P_x.active or self.P_y.active):
             return input
         Function = self._distdl_backend.functional.sum_reduce.SumReduceFunction
-        return Function.apply(input, self.P_x, self.P_y, self.preserve_batch, None,
-                              self.transpose_src, self.transpose_dest)
+        # Positional arguments as in the reference (nn/sum_reduce.py:205-211).
+        return Function.apply(input, self.P_send, self.P_recv, self.preserve_batch, TensorStructure(input), None)

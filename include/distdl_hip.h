@@ -42,24 +42,6 @@ const char* ddl_version(void);
 /* Message for the last non-zero return on the calling thread ("" if none). */
 const char* ddl_last_error(void);
 
-/* Enqueues a kernel that does nothing, `workgroups` workgroups of `threads`
- * threads (1..1024).  No counterpart in the reference: a measurement aid that
- * gives the time a launch of that size costs on its own, the floor under every
- * small kernel of this library. */
-int ddl_probe_launch(int64_t workgroups, int threads, void* stream);
-
-/* Enqueues a kernel of nothing but bf16 MFMAs on operands held in registers
- * (512 workgroups of 256 threads: two wavefronts per SIMD on 256 CUs), the
- * other measurement aid: what the matrix cores sustain on this machine with
- *   instruction 0: v_mfma_f32_32x32x16_bf16,  1: v_mfma_f32_16x16x32_bf16
- *   random      0: every operand element 1.0, 1: N(0,1) x 0.02 N(0,1) operands
- * which differ because on random operands the chip runs against its power
- * limit.  `iters` loop iterations of 2^20 flop per wavefront; the flop count
- * of the launch is stored to the host address `flop` (may be NULL).  `sink`:
- * device memory for 131072 floats that the kernel overwrites. */
-int ddl_probe_mfma(int instruction, int random, int iters, float* sink,
-                   int64_t sink_elems, int64_t* flop, void* stream);
-
 /* ------------------------------------------------------------------------ *
  * Box copies (Repartition / HaloExchange pack, unpack, self-copy)
  * ------------------------------------------------------------------------ */

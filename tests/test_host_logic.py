@@ -619,6 +619,70 @@ def test_sum_reduce_and_broadcast_layers_with_one_live_worker():
     assert torch.equal(x.grad, 2 * torch.ones(2, 3))
 
 
+def test_primitive_functions_take_the_reference_arguments():
+    """Every autograd Function of the backend is called by the reference's
+    layers with a fixed list of positional arguments
+    (backends/mpi_numpy/functional/all_gather.py:36-37, all_sum_reduce.py:32-33,
+    broadcast.py:32-34, reduce_scatter.py:35-37, sum_reduce.py:32-34,
+    repartition.py:33-36, halo_exchange.py:14); forward takes exactly those and
+    backward returns one gradient slot for each."""
+    import inspect
+    from distdl_amd import backends
+    fn = backends.backend.functional
+    expected = {
+        fn.all_gather.AllGatherFunction:
+            ["input", "P_allgather", "input_tensor_structure", "output_tensor_structure", "axes", "scale_backward"],
+        fn.all_sum_reduce.AllSumReduceFunction:
+            ["input", "P_allreduce", "input_tensor_structure", "output_tensor_structure", "scale_backward"],
+        fn.broadcast.BroadcastFunction:
+            ["input", "P_send", "P_recv", "preserve_batch", "input_tensor_structure", "output_tensor_structure",
+             "scale_backward"],
+        fn.reduce_scatter.ReduceScatterFunction:
+            ["input", "P_reducescatter", "input_tensor_structure", "output_tensor_structure", "axes"],
+        fn.sum_reduce.SumReduceFunction:
+            ["input", "P_send", "P_recv", "preserve_batch", "input_tensor_structure", "output_tensor_structure"],
+        fn.repartition.RepartitionFunction:
+            ["input", "P_union", "x_global_structure", "x_local_structure", "y_local_structure", "P_x",
+             "P_x_to_y_overlaps", "P_x_to_y_buffers", "P_y", "P_y_to_x_overlaps", "P_y_to_x_buffers", "preserve_batch"],
+        fn.halo_exchange.HaloExchangeFunction: ["input", "P_x", "slices", "buffers", "neighbor_ranks"],
+    }
+    for Function, names in expected.items():
+        params = list(inspect.signature(Function.forward).parameters.values())
+        assert [p.name for p in params] == ["ctx"] + names, Function.__name__
+        assert all(p.default is inspect.Parameter.empty for p in params), Function.__name__
+    # one live worker: identity paths hand back one gradient slot per argument
+    world = SimWorld(1, device=torch.device("cpu"))
+    P = world.partition(0).create_partition_inclusive([0]).create_cartesian_topology_partition([1, 1])
+    x = torch.arange(6.0).reshape(2, 3).requires_grad_(True)
+    s = TensorStructure(x)
+    y = fn.all_gather.AllGatherFunction.apply(x, P.create_allreduction_partition((1,)), s, s, (1,), 2.0)
+    y = fn.reduce_scatter.ReduceScatterFunction.apply(y, P.create_allreduction_partition((1,)), s, s, (1,))
+    y = fn.all_sum_reduce.AllSumReduceFunction.apply(y, P.create_allreduction_partition((0,)), s, s, 4.0)
+    y.backward(torch.ones_like(y))
+    assert torch.equal(x.grad, torch.full((2, 3), 0.125))
+
+
+def test_route_partitions_of_broadcast_and_reduction():
+    """create_broadcast_partition_to / create_reduction_partition_to hand back
+    (P_send, P_recv), active on the workers of the source resp. destination
+    (backends/common/partition.py:490-632, :683-823), and
+    create_allreduction_partition the workers that differ along the axes only."""
+    world = SimWorld(4, device=torch.device("cpu"))
+    for rank in range(4):
+        P_world = world.partition(rank)
+        P_x = P_world.create_partition_inclusive([0, 1]).create_cartesian_topology_partition([1, 2])
+        P_w = P_world.create_partition_inclusive([0, 1, 2, 3]).create_cartesian_topology_partition([2, 2])
+        P_send, P_recv = P_x.create_broadcast_partition_to(P_w)
+        assert P_send.active == (rank < 2) and P_recv.active
+        P_send, P_recv = P_w.create_reduction_partition_to(P_x, transpose_src=True)
+        assert P_send.active and P_recv.active == (rank < 2)
+        P_r = P_w.create_allreduction_partition((0,))
+        assert list(P_r.shape) == [2, 1] and P_r.size == 2
+        assert P_r._ranks == ((0, 2) if rank % 2 == 0 else (1, 3)) and P_r.rank == rank // 2
+    with pytest.raises(ValueError):
+        P_w.create_allreduction_partition((2,))
+
+
 def test_bench_refuses_more_than_one_gpu():
     """One GPU's share is what is measured; a request for more says so and
     exits before anything touches a device."""
