@@ -10,6 +10,7 @@ import ctypes
 import os
 from ctypes import POINTER
 from ctypes import c_char_p
+from ctypes import c_double
 from ctypes import c_float
 from ctypes import c_int
 from ctypes import c_int32
@@ -56,6 +57,7 @@ SIGNATURES = {
     "ddl_version": (c_char_p, []),
     "ddl_last_error": (c_char_p, []),
     "ddl_copy_boxes": (c_int, [POINTER(ddl_box_t), c_int, c_int, c_int, c_int, c_void_p]),
+    "ddl_sum_boxes": (c_int, [POINTER(ddl_box_t), POINTER(c_void_p), c_int, c_int, c_int, c_double, c_void_p]),
     "ddl_pack_boxes": (c_int, [c_void_p, POINTER(c_int64), POINTER(c_int64), c_int, c_int, c_int,
                                POINTER(c_int64), POINTER(c_int64), POINTER(c_void_p), c_void_p]),
     "ddl_unpack_boxes": (c_int, [c_void_p, POINTER(c_int64), POINTER(c_int64), c_int, c_int, c_int,

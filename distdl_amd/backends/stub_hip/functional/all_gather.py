@@ -4,8 +4,8 @@ itself belongs to the transport; what runs here is the local re-layout the
 reference does with einops (``p a b c -> a (p b) c``, zero-padding and stripping
 uneven shards): the P received pieces are unpacked into their slabs of the
 output by one launch of the box kernel, uneven pieces included.  The adjoint is
-a reduce-scatter: every worker sums its slab of all workers' gradients
-(strided reads, accumulating box copies)."""
+a reduce-scatter: every worker sums its slab of all workers' gradients in one
+launch of the sum kernel (strided reads of the P slabs, one write)."""
 
 __all__ = ["AllGatherFunction", "gather_slabs", "reduce_scatter_slabs", "single_axis"]
 
@@ -19,7 +19,7 @@ from ....utilities.slicing import compute_subshape
 def gather_slabs(P, local, axis, tag):
     """``local`` of every worker of ``P``, concatenated along ``axis`` in rank order."""
     transport = P._world.transport
-    x = local if local.is_contiguous() else local.contiguous()
+    x = hip_ops.contiguous(local)
     parts = transport.gather_list(P, x, tag=tag)
     extent = sum(int(p.shape[axis]) for p in parts)
     shape = list(x.shape)
@@ -36,11 +36,13 @@ def gather_slabs(P, local, axis, tag):
     return out
 
 
-def reduce_scatter_slabs(P, full, axis, tag):
-    """Sum over the workers of ``P`` of their ``full`` tensors, of which this
-    worker keeps its balanced slab along ``axis``."""
+def reduce_scatter_slabs(P, full, axis, tag, divisor=1):
+    """Sum over the workers of ``P``, in rank order, of their ``full`` tensors
+    (each divided by ``divisor`` first), of which this worker keeps its balanced
+    slab along ``axis``: one launch that reads the P slabs where they lie and
+    writes the result once."""
     transport = P._world.transport
-    g = full if full.is_contiguous() else full.contiguous()
+    g = hip_ops.contiguous(full)
     grads = transport.gather_list(P, g, tag=tag)
     me = int(P.rank)
     extent = int(g.shape[axis])
@@ -52,8 +54,8 @@ def reduce_scatter_slabs(P, full, axis, tag):
     src = [slice(0, int(n)) for n in g.shape]
     src[axis] = slice(start, start + sizes[me])
     dst = [slice(0, int(n)) for n in shape]
-    for q, gq in enumerate(grads):
-        hip_ops.copy_box(gq, src, out, dst, accumulate=q > 0)
+    if out.numel():
+        hip_ops.sum_boxes(grads, src, out, dst, divisor)
     transport.release(P, tag=tag)
     return out
 
@@ -87,9 +89,9 @@ class AllGatherFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         grad_output = grad_output.detach()
-        if ctx.scale_backward is not None:
-            grad_output = grad_output / ctx.scale_backward      # before the sum (reference :188-190)
+        # Every worker's gradient is divided before the sum (reference :188-190): the sum kernel divides as it reads.
+        divisor = 1 if ctx.scale_backward is None else ctx.scale_backward
         if ctx.identity:
-            return grad_output, None, None, None, None, None
-        dx = reduce_scatter_slabs(ctx.P, grad_output, ctx.axis, ("all_gather_adjoint", None))
+            return (grad_output if divisor == 1 else hip_ops.scaled(grad_output, divisor)), None, None, None, None, None
+        dx = reduce_scatter_slabs(ctx.P, grad_output, ctx.axis, ("all_gather_adjoint", None), divisor)
         return dx, None, None, None, None, None

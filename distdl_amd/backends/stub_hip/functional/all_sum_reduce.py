@@ -1,10 +1,25 @@
 """All-sum-reduce stand-in (reference: backends/mpi_numpy/functional/all_sum_reduce.py:77-92).
-A collective, hence outside this build: contributions are gathered through the
-transport and summed in rank order."""
+A collective, hence outside this build: the workers' tensors are handed over by
+the transport and summed in rank order by one launch of the sum kernel."""
 
 __all__ = ["AllSumReduceFunction"]
 
 import torch
+
+from .... import hip_ops
+
+
+def _sum_over(P, tensor, tag, divisor=1):
+    """Sum of ``tensor / divisor`` over the workers of ``P``, in rank order."""
+    transport = P._world.transport
+    mine = hip_ops.contiguous(tensor)
+    parts = transport.gather_list(P, mine, tag=tag)
+    out = torch.empty_like(mine)
+    if out.numel():
+        full = [slice(0, int(n)) for n in mine.shape]
+        hip_ops.sum_boxes(parts, full, out, full, divisor)
+    transport.release(P, tag=tag)
+    return out
 
 
 class AllSumReduceFunction(torch.autograd.Function):
@@ -18,17 +33,15 @@ class AllSumReduceFunction(torch.autograd.Function):
         tag = None
         if not P_reduce.active or P_reduce.size == 1:
             return input
-        parts = P_reduce._world.transport.allgather(P_reduce, input.detach(), tag=tag)
-        return parts.sum(dim=0)
+        return _sum_over(P_reduce, input.detach(), ("all_sum_reduce", tag))
 
     @staticmethod
     def backward(ctx, grad_output):
         # The all-sum-reduce is its own adjoint (reference :95-161).
         P_reduce = ctx.P_reduce
         grad_output = grad_output.detach()
-        if ctx.scale_backward is not None:
-            grad_output = grad_output / ctx.scale_backward      # before the sum (reference :127-128)
+        # Every worker's gradient is divided before the sum (reference :127-128): the sum kernel divides as it reads.
+        divisor = 1 if ctx.scale_backward is None else ctx.scale_backward
         if not P_reduce.active or P_reduce.size == 1:
-            return grad_output, None, None, None, None
-        parts = P_reduce._world.transport.allgather(P_reduce, grad_output.contiguous(), tag=("adjoint", ctx.tag))
-        return parts.sum(dim=0), None, None, None, None
+            return (grad_output if divisor == 1 else hip_ops.scaled(grad_output, divisor)), None, None, None, None
+        return _sum_over(P_reduce, grad_output, ("all_sum_reduce_adjoint", ctx.tag), divisor), None, None, None, None

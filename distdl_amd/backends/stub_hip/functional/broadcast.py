@@ -9,6 +9,7 @@ __all__ = ["BroadcastFunction", "route_of"]
 
 import torch
 
+from .... import hip_ops
 from ....utilities.torch import zero_volume_tensor
 
 
@@ -56,7 +57,7 @@ class BroadcastFunction(torch.autograd.Function):
         grad_output = grad_output.detach()
         if ctx.scale_backward is not None and P_recv.active:
             # Every receiver's gradient is divided before the sum (reference :208-209).
-            grad_output = grad_output / ctx.scale_backward
+            grad_output = hip_ops.scaled(grad_output, ctx.scale_backward)
         grad = world.transport.broadcast_adjoint(P_send, P_recv, grad_output, transpose_src=transpose_src,
                                                  transpose_dst=transpose_dest, tag=ctx.tag)
         if grad is None:

@@ -1,8 +1,8 @@
 """Reduce-scatter along one partitioned axis and its adjoint (reference:
 backends/mpi_numpy/functional/reduce_scatter.py:86-127, :130-200): every worker
 holds a full-length tensor and keeps its balanced slab of the sum.  The adjoint
-is the all-gather.  Local work: strided slab reads with accumulating box
-copies, resp. one unpack launch of the box kernel; see all_gather.py."""
+is the all-gather.  Local work: one launch of the sum kernel over the P slabs,
+resp. one unpack launch of the box kernel; see all_gather.py."""
 
 __all__ = ["ReduceScatterFunction"]
 

@@ -18,6 +18,7 @@ MPI or NCCL between those halves is supplied here by one of two transports:
 """
 
 import threading
+import weakref
 
 import numpy as np
 
@@ -68,17 +69,28 @@ class SoloTransport:
     def __init__(self, world):
         self.world = world
         self._gather_providers = {}
-        self._seeded = {}            # tag -> identity of the buffer whose peer slots a provider has filled
+        self._constant = set()       # tags whose provider stands for peers that contribute the same on every call
+        self._seeded = {}            # tag -> weak reference to the buffer whose peer slots a constant provider has filled
         self._shape_provider = None
 
     # -- configuration by tests / benchmarks --------------------------------
 
-    def set_gather_provider(self, tag, fn):
+    def set_gather_provider(self, tag, fn, constant=False):
         """``fn(P, tensor) -> list of P.size tensors`` supplies what the peers
         would contribute to a gather carrying ``tag`` (entry ``P.rank`` is
-        replaced by the live tensor)."""
+        replaced by the live tensor).  It is asked on every gather, unless
+        ``constant`` says that the peers' parts do not depend on the call: an
+        in-place gather then asks once per buffer and the parts stay in its
+        slots (seeded peers, as a benchmark of one rank's share has them)."""
         self._gather_providers[tag] = fn
+        self._constant.discard(tag)
+        if constant:
+            self._constant.add(tag)
         self._seeded.pop(tag, None)
+
+    def _is_seeded(self, tag, buffer):
+        ref = self._seeded.get(tag)
+        return ref is not None and ref() is buffer
 
     def set_peer_shape_provider(self, fn):
         """``fn(P, index, my_shape) -> shape`` of the shard held by the peer at
@@ -133,28 +145,34 @@ class SoloTransport:
 
     def allgather_into(self, P, buffer, tag=None):
         """In-place all-gather: ``buffer`` is ``[P.size, ...]`` and slot
-        ``P.rank`` already holds this worker's part.  The other slots hold what
-        the caller seeded them with; a gather provider registered for ``tag``
-        fills them once per buffer (it stands for peers whose contribution does
-        not change between calls)."""
+        ``P.rank`` already holds this worker's part.  Without a provider the
+        absent workers hold what the live one holds (as in :meth:`allgather`);
+        a provider supplies their parts on every call, a constant one once per
+        buffer object."""
         fn = self._gather_providers.get(tag)
-        if fn is not None and self._seeded.get(tag) != (buffer.data_ptr(), tuple(buffer.shape)):
-            parts = list(fn(P, buffer[P.rank]))
-            if len(parts) != P.size:
-                raise TransportError(f"gather provider for {tag!r} returned {len(parts)} parts for {P.size} workers")
-            for p, part in enumerate(parts):
+        if fn is None:
+            for p in range(P.size):
                 if p != P.rank:
-                    buffer[p].copy_(part)
-            self._seeded[tag] = (buffer.data_ptr(), tuple(buffer.shape))
+                    buffer[p].copy_(buffer[P.rank])
+            return buffer
+        if tag in self._constant and self._is_seeded(tag, buffer):
+            return buffer
+        parts = list(fn(P, buffer[P.rank]))
+        if len(parts) != P.size:
+            raise TransportError(f"gather provider for {tag!r} returned {len(parts)} parts for {P.size} workers")
+        for p, part in enumerate(parts):
+            if p != P.rank:
+                buffer[p].copy_(part)
+        if tag in self._constant:
+            self._seeded[tag] = weakref.ref(buffer)
         return buffer
 
     def peers_gathered_ahead(self, P, buffer, tag=None):
         """True when the slots of ``buffer`` other than ``P.rank`` hold the
-        peers' parts before the live rank's part exists (they were seeded, or a
-        provider has filled them on an earlier call), so that one kernel may
-        produce the live part and consume the others."""
-        fn = self._gather_providers.get(tag)
-        return fn is None or self._seeded.get(tag) == (buffer.data_ptr(), tuple(buffer.shape))
+        peers' parts before the live rank's part exists -- a constant provider
+        has filled them on an earlier call -- so that one kernel may produce the
+        live part and consume the others."""
+        return tag in self._constant and self._is_seeded(tag, buffer)
 
     def broadcast(self, P_src, P_dst, tensor, transpose_src=False, transpose_dst=False, tag=None):
         if P_src.active:

@@ -171,8 +171,9 @@ typedef const DevBox* DevBoxPtr;
 // entries beyond a box's own count hold extent 1 and stride 0).  Every table
 // field is fetched unconditionally at the top, so the scalar loads are issued
 // together and waited for once per tile.
-template <int OP, typename T, typename V, int ND>
-__device__ inline void move_tile(DevBoxPtr bx, uint32_t tile) {
+template <int ND>
+__device__ __forceinline__ void tile_offsets(DevBoxPtr bx, uint32_t tile, int64_t (&soff)[kUnroll], int64_t (&doff)[kUnroll],
+                                             bool (&live)[kUnroll]) {
     const uint32_t col_tiles = bx->col_tiles;
     const uint32_t tc_log = bx->tc_log;
     const uint32_t ct_mul = bx->ct_mul, ct_shr = bx->ct_shr;
@@ -192,8 +193,6 @@ __device__ inline void move_tile(DevBoxPtr bx, uint32_t tile) {
     const uint32_t col_tile = tile - row_tile * col_tiles;
     const uint32_t row0 = row_tile << (kTileLog - tc_log);
     const uint32_t col0 = col_tile << tc_log;
-    int64_t soff[kUnroll], doff[kUnroll];
-    bool live[kUnroll];
     const uint32_t tc = 1u << tc_log;
     const bool interior = col0 + tc <= cols && row0 + (kTileVecs >> tc_log) <= rows;   // wave-uniform
     if (ND <= 1 && interior) {
@@ -252,6 +251,13 @@ __device__ inline void move_tile(DevBoxPtr bx, uint32_t tile) {
             doff[u] = dof;
         }
     }
+}
+
+template <int OP, typename T, typename V, int ND>
+__device__ inline void move_tile(DevBoxPtr bx, uint32_t tile) {
+    int64_t soff[kUnroll], doff[kUnroll];
+    bool live[kUnroll];
+    tile_offsets<ND>(bx, tile, soff, doff, live);
     char* const dst = bx->dst;
     if constexpr (OP == OP_ZERO) {
         V z;
@@ -324,6 +330,159 @@ __global__ __launch_bounds__(kThreads) void box_kernel(const Batch bt_by_value) 
             case 2: move_tile_nd<OP, T, uint32_t>(bx, tile, nd); break;
             case 1: move_tile_nd<OP, T, uint16_t>(bx, tile, nd); break;
             default: move_tile_nd<OP, T, uint8_t>(bx, tile, nd); break;
+        }
+    }
+}
+
+// Sum of several sources into one destination, each source divided first.
+//
+// The quotient and every partial sum are rounded to the element type, in the
+// order of the sources: bit for bit what a chain of element-wise divisions and
+// accumulating box copies gives, in one pass that reads every source once and
+// writes the destination once.
+template <typename T>
+struct DivOp;
+template <>
+struct DivOp<float> {
+    static __device__ float apply(float a, double d) { return a / static_cast<float>(d); }
+};
+template <>
+struct DivOp<double> {
+    static __device__ double apply(double a, double d) { return a / d; }
+};
+template <>
+struct DivOp<bf16_bits> {
+    static __device__ bf16_bits apply(bf16_bits a, double d) {
+        const float q = __uint_as_float(static_cast<uint32_t>(a.u) << 16) / static_cast<float>(d);
+        uint32_t u = __float_as_uint(q);
+        bf16_bits r;
+        if (q != q) {
+            r.u = 0x7FC0;
+        } else {
+            u += 0x7FFFu + ((u >> 16) & 1u);
+            r.u = static_cast<uint16_t>(u >> 16);
+        }
+        return r;
+    }
+};
+template <>
+struct DivOp<f16_bits> {
+    static __device__ f16_bits apply(f16_bits a, double d) {
+        _Float16 ha;
+        __builtin_memcpy(&ha, &a.u, 2);
+        const _Float16 hq = static_cast<_Float16>(static_cast<float>(ha) / static_cast<float>(d));
+        f16_bits r;
+        __builtin_memcpy(&r.u, &hq, 2);
+        return r;
+    }
+};
+// Integers are only ever summed (the host refuses a divisor other than 1 for them).
+template <>
+struct DivOp<int32_t> {
+    static __device__ int32_t apply(int32_t a, double) { return a; }
+};
+template <>
+struct DivOp<int64_t> {
+    static __device__ int64_t apply(int64_t a, double) { return a; }
+};
+
+template <typename T, typename V>
+__device__ inline V div_vector(V s, double d) {
+    constexpr int n = sizeof(V) / sizeof(T);
+    T sv[n];
+    __builtin_memcpy(sv, &s, sizeof(V));
+#pragma unroll
+    for (int i = 0; i < n; ++i) sv[i] = DivOp<T>::apply(sv[i], d);
+    V out;
+    __builtin_memcpy(&out, sv, sizeof(V));
+    return out;
+}
+
+constexpr int kMaxSumSources = 64;
+
+struct SumArgs {
+    DevBox box;                        // src: the box in source 0
+    int64_t delta[kMaxSumSources];     // bytes from source 0 to source q (delta[0] = 0)
+    double divisor;
+    uint32_t nsrc;
+    uint32_t ntiles;
+    uint32_t divide;                   // 0: divisor is 1, sources are summed as they are
+    uint32_t pad;
+};
+
+#if defined(__HIP_DEVICE_COMPILE__)
+typedef const SumArgs __attribute__((address_space(4))) * SumArgsPtr;
+#else
+typedef const SumArgs* SumArgsPtr;
+#endif
+
+template <typename T, typename V, int ND>
+__device__ inline void sum_tile(SumArgsPtr sa, uint32_t tile) {
+    DevBoxPtr bx = &sa->box;
+    int64_t soff[kUnroll], doff[kUnroll];
+    bool live[kUnroll];
+    tile_offsets<ND>(bx, tile, soff, doff, live);
+    const char* const src = bx->src;
+    const uint32_t nsrc = sa->nsrc;
+    const bool divide = sa->divide != 0;
+    const double divisor = sa->divisor;
+    V acc[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) acc[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(src + soff[u]));
+    if (divide) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) acc[u] = div_vector<T, V>(acc[u], divisor);
+    }
+    for (uint32_t q = 1; q < nsrc; ++q) {
+        const char* const sq = src + sa->delta[q];
+        V val[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) val[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(sq + soff[u]));
+        if (divide) {
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) val[u] = div_vector<T, V>(val[u], divisor);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) acc[u] = add_vectors<T, V>(acc[u], val[u]);
+    }
+    // The destination may be one of the sources: an element is written by the one lane that owns it.
+    char* const dst = bx->dst;
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+        if (live[u]) __builtin_nontemporal_store(acc[u], reinterpret_cast<V*>(dst + doff[u]));
+}
+
+template <typename T, typename V>
+__device__ inline void sum_tile_nd(SumArgsPtr sa, uint32_t tile, uint32_t nd) {
+    if (nd == 0)
+        sum_tile<T, V, 0>(sa, tile);
+    else if (nd == 1)
+        sum_tile<T, V, 1>(sa, tile);
+    else if (nd == 2)
+        sum_tile<T, V, 2>(sa, tile);
+    else
+        sum_tile<T, V, kMaxDevDims>(sa, tile);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void sum_kernel(const SumArgs args_by_value) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    SumArgsPtr sa = (SumArgsPtr)__builtin_amdgcn_kernarg_segment_ptr();
+#else
+    SumArgsPtr sa = &args_by_value;
+#endif
+    const uint32_t ntiles = sa->ntiles;
+    const uint32_t nd = sa->box.nd, vlog = sa->box.vlog;
+    for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        // A vector holds whole elements: the host lowers the box with the element size as the narrowest vector.
+        if (vlog == 4)
+            sum_tile_nd<T, u32x4>(sa, tile, nd);
+        else if (vlog == 3) {
+            if constexpr (sizeof(T) <= 8) sum_tile_nd<T, u32x2>(sa, tile, nd);
+        } else if (vlog == 2) {
+            if constexpr (sizeof(T) <= 4) sum_tile_nd<T, uint32_t>(sa, tile, nd);
+        } else {
+            if constexpr (sizeof(T) <= 2) sum_tile_nd<T, uint16_t>(sa, tile, nd);
         }
     }
 }
@@ -579,10 +738,60 @@ int tensor_boxes(const void* tensor, const int64_t* tshape, const int64_t* tstri
     return 0;
 }
 
+
+template <typename T>
+int launch_sum(const std::vector<DevBox>& pieces, const void* const* srcs, int nsrc, double divisor, hipStream_t stream) {
+    for (const DevBox& db : pieces) {
+        SumArgs sa{};
+        sa.box = db;
+        for (int q = 0; q < nsrc; ++q) sa.delta[q] = static_cast<const char*>(srcs[q]) - static_cast<const char*>(srcs[0]);
+        sa.divisor = divisor;
+        sa.divide = divisor != 1.0 ? 1u : 0u;
+        sa.nsrc = static_cast<uint32_t>(nsrc);
+        const uint64_t tr = kTileVecs >> db.tc_log;
+        const uint64_t tiles = static_cast<uint64_t>(db.col_tiles) * ((db.rows + tr - 1) / tr);
+        sa.ntiles = static_cast<uint32_t>(tiles);
+        const uint32_t blocks = tiles < kPersistentBlocks ? static_cast<uint32_t>(tiles) : kPersistentBlocks;
+        hipLaunchKernelGGL((sum_kernel<T>), dim3(blocks), dim3(kThreads), 0, stream, sa);
+        if (int rc = check_launch("sum_kernel")) return rc;
+    }
+    return 0;
+}
+
 }  // namespace
 }  // namespace ddl
 
 extern "C" {
+
+int ddl_sum_boxes(const ddl_box_t* box, const void* const* srcs, int nsrc, int elem_size, int dtype, double divisor, void* stream) {
+    using namespace ddl;
+    if (!box || !srcs) return fail(DDL_E_ARG, "sum_boxes: null argument");
+    if (nsrc < 1 || nsrc > kMaxSumSources) return fail(DDL_E_UNSUPP, "sum_boxes: %d sources outside [1,%d]", nsrc, kMaxSumSources);
+    static const int dt_size[] = {0, 4, 8, 2, 2, 4, 8};
+    if (dtype < DDL_DT_F32 || dtype > DDL_DT_I64) return fail(DDL_E_ARG, "sum_boxes needs an arithmetic dtype, got %d", dtype);
+    if (dt_size[dtype] != elem_size) return fail(DDL_E_ARG, "dtype %d does not have element size %d", dtype, elem_size);
+    if (!(divisor == divisor) || divisor == 0.0) return fail(DDL_E_ARG, "sum_boxes: divisor %g", divisor);
+    if ((dtype == DDL_DT_I32 || dtype == DDL_DT_I64) && divisor != 1.0) return fail(DDL_E_UNSUPP, "sum_boxes: integers are summed, not divided");
+    for (int q = 0; q < nsrc; ++q) {
+        if (!srcs[q]) return fail(DDL_E_ARG, "sum_boxes: source %d is null", q);
+        // One vector width serves all sources: they must sit at the same offset from a 16-byte boundary.
+        if ((reinterpret_cast<uintptr_t>(srcs[q]) - reinterpret_cast<uintptr_t>(srcs[0])) % 16 != 0)
+            return fail(DDL_E_ALIGN, "sum_boxes: source %d is not a multiple of 16 bytes from source 0", q);
+    }
+    ddl_box_t in = *box;
+    in.src = srcs[0];
+    std::vector<DevBox> pieces;
+    if (int rc = lower_box(in, elem_size, true, &pieces)) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case DDL_DT_F32: return launch_sum<float>(pieces, srcs, nsrc, divisor, s);
+        case DDL_DT_F64: return launch_sum<double>(pieces, srcs, nsrc, divisor, s);
+        case DDL_DT_BF16: return launch_sum<bf16_bits>(pieces, srcs, nsrc, divisor, s);
+        case DDL_DT_I32: return launch_sum<int32_t>(pieces, srcs, nsrc, divisor, s);
+        case DDL_DT_I64: return launch_sum<int64_t>(pieces, srcs, nsrc, divisor, s);
+        default: return launch_sum<f16_bits>(pieces, srcs, nsrc, divisor, s);
+    }
+}
 
 int ddl_copy_boxes(const ddl_box_t* boxes, int nbox, int elem_size, int op, int dtype, void* stream) {
     if (op != DDL_OP_COPY && op != DDL_OP_ADD) return ddl::fail(DDL_E_ARG, "unknown box operation %d", op);

@@ -180,6 +180,83 @@ def copy_box(src, src_slices, dst, dst_slices, accumulate=False):
     _lib.check(rc, "ddl_copy_boxes")
 
 
+def sum_boxes(srcs, src_slices, dst, dst_slices, divisor=1):
+    """dst[dst_slices] = sum over q, in order, of srcs[q][src_slices] / divisor.
+
+    One launch that reads every source once and writes the destination once;
+    quotients and partial sums are rounded to the element type, as a chain of
+    divisions and accumulating copies would round them.  All sources share
+    shape and strides.  ``dst`` may be one of them when the slices coincide
+    (scaling in place).  Sources that do not sit a multiple of 16 bytes apart,
+    or more than 64 of them, are summed by accumulating box copies instead
+    (``divisor`` 1 only)."""
+    srcs = list(srcs)
+    if not srcs:
+        raise ValueError("sum_boxes: no sources")
+    first = srcs[0]
+    _require_gpu(dst, *srcs)
+    nd = first.dim()
+    for t in srcs:
+        if t.dtype != dst.dtype or tuple(t.shape) != tuple(first.shape) or t.stride() != first.stride():
+            raise ValueError("sum_boxes: sources must agree in dtype, shape and strides with each other (dtype: and with dst)")
+    if dst.dtype not in _ADD_DTYPES:
+        raise ValueError(f"sums are not available for {dst.dtype}")
+    if dst.dim() != nd or len(src_slices) != nd or len(dst_slices) != nd:
+        raise ValueError("sum_boxes: rank mismatch")
+    box = _lib.ddl_box_t()
+    box.ndim = nd
+    soff = doff = 0
+    for d in range(nd):
+        n = int(src_slices[d].stop) - int(src_slices[d].start)
+        if n != int(dst_slices[d].stop) - int(dst_slices[d].start):
+            raise ValueError("sum_boxes: source and destination boxes differ in shape")
+        if src_slices[d].start < 0 or src_slices[d].stop > first.shape[d] or \
+           dst_slices[d].start < 0 or dst_slices[d].stop > dst.shape[d]:
+            raise ValueError("sum_boxes: box outside tensor")
+        box.shape[d] = n
+        box.src_stride[d] = first.stride(d)
+        box.dst_stride[d] = dst.stride(d)
+        soff += int(src_slices[d].start) * first.stride(d)
+        doff += int(dst_slices[d].start) * dst.stride(d)
+    es = dst.element_size()
+    box.dst = dst.data_ptr() + doff * es
+    ptrs = [t.data_ptr() + soff * es for t in srcs]
+    one_launch = len(srcs) <= 64 and all((p - ptrs[0]) % 16 == 0 for p in ptrs)
+    if not one_launch:
+        if divisor != 1:
+            raise ValueError("sum_boxes: this layout of the sources is summed by accumulating copies, which cannot divide")
+        for q, t in enumerate(srcs):
+            copy_box(t, src_slices, dst, dst_slices, accumulate=q > 0)
+        return
+    rc = _lib.load().ddl_sum_boxes(ctypes.byref(box), _lib.ptr_array(ptrs), len(srcs), es, _ADD_DTYPES[dst.dtype],
+                                   float(divisor), _stream())
+    _lib.check(rc, "ddl_sum_boxes")
+
+
+def scaled(t, divisor):
+    """``t / divisor`` as a new tensor, through the sum kernel with one source
+    (the scaling of a gradient ahead of an adjoint's sum)."""
+    out = torch.empty(t.shape, dtype=t.dtype, device=t.device)
+    if t.numel() == 0:
+        return out
+    src = t if t.is_contiguous() else contiguous(t)
+    full = [slice(0, int(n)) for n in src.shape]
+    sum_boxes([src], full, out, full, divisor)
+    return out
+
+
+def contiguous(t):
+    """A row-major copy of a strided tensor, made by the box kernel."""
+    if t.is_contiguous():
+        return t
+    _require_gpu(t)
+    out = torch.empty(t.shape, dtype=t.dtype, device=t.device)
+    if t.numel():
+        full = [slice(0, int(n)) for n in t.shape]
+        copy_box(t, full, out, full)
+    return out
+
+
 class HaloPadPlan:
     """Geometry of the fused pad + ghost fill + bulk pack call for one shard shape."""
 
@@ -510,7 +587,7 @@ def embedding_gather(weight, ids, lo, hi, out=None):
         raise ValueError("embedding_gather: ids must be int32 or int64")
     if weight.shape[0] != hi - lo:
         raise ValueError(f"embedding_gather: table has {weight.shape[0]} rows but the window is [{lo},{hi})")
-    ids_c = ids.contiguous()
+    ids_c = contiguous(ids)
     dim = weight.shape[1]
     if out is None:
         out = torch.empty(tuple(ids.shape) + (dim,), dtype=weight.dtype, device=weight.device)
@@ -539,7 +616,7 @@ def embedding_renorm(weight, ids, lo, hi, max_norm, norm_type=2.0):
         raise ValueError(f"embedding_renorm: table has {weight.shape[0]} rows but the window is [{lo},{hi})")
     if weight.shape[0] == 0 or ids.numel() == 0:
         return weight
-    ids_c = ids.contiguous()
+    ids_c = contiguous(ids)
     dim = weight.shape[1]
     flags = torch.empty(weight.shape[0], dtype=torch.int32, device=weight.device)
     rc = _lib.load().ddl_embedding_renorm(weight.data_ptr(), _LN_DTYPES[weight.dtype], dim,
@@ -564,8 +641,8 @@ def embedding_backward(grad_output, ids, lo, hi, padding_idx=None, scale_grad_by
         raise ValueError("embedding_backward: gradient and ids disagree in shape")
     dy = grad_output.reshape(-1, dim)
     if dim > 1 and dy.stride(1) != 1:
-        dy = dy.contiguous()
-    ids_c = ids.contiguous()
+        dy = contiguous(dy)
+    ids_c = contiguous(ids)
     rows, n_ids = int(hi) - int(lo), ids_c.numel()
     dw = torch.empty((rows, dim), dtype=grad_output.dtype, device=grad_output.device)
     work = torch.empty(2 * rows + 1 + n_ids, dtype=torch.int32, device=grad_output.device)
@@ -610,9 +687,9 @@ def linear(x, weight, bias=None, out=None):
     n, k = weight.shape
     x2 = x.reshape(-1, k)
     if x2.stride(1) != 1 and k > 1:
-        x2 = x2.contiguous()
+        x2 = contiguous(x2)
     if weight.stride(1) != 1 and k > 1:
-        weight = weight.contiguous()
+        weight = contiguous(weight)
     if bias is not None and (bias.numel() != n or not bias.is_contiguous()):
         raise ValueError("linear: bias must be contiguous with out_features elements")
     m = x2.shape[0]
@@ -657,7 +734,7 @@ def transpose_2d(src, ld_dst=None):
     if src.dim() != 2 or src.element_size() != 2:
         raise ValueError("transpose_2d: a 2-D tensor of 16-bit elements is required")
     if src.stride(1) != 1 and src.shape[1] > 1:
-        src = src.contiguous()
+        src = contiguous(src)
     rows, cols = src.shape
     ld_dst = rows if ld_dst is None else ld_dst
     alloc = torch.empty if ld_dst == rows else torch.zeros
@@ -675,7 +752,7 @@ def colsum(a):
     if a.dim() != 2 or dt is None:
         raise ValueError("colsum: a 2-D bfloat16, float16 or float32 tensor is required")
     if a.stride(1) != 1 and a.shape[1] > 1:
-        a = a.contiguous()
+        a = contiguous(a)
     rows, cols = a.shape
     out = torch.empty(cols, dtype=a.dtype, device=a.device)
     splits = max(1, min(64, (rows + 127) // 128))
@@ -709,14 +786,14 @@ def linear_backward(x, weight, grad_output, need_input=True, need_weight=True, n
     x2 = x.reshape(-1, k)
     dy = grad_output.reshape(-1, n)
     if dy.stride(1) != 1 and n > 1:
-        dy = dy.contiguous()
+        dy = contiguous(dy)
     m = x2.shape[0]
     dx = dw = db = None
     if dt == _lib.DDL_DT_F32:
         if x2.stride(1) != 1 and k > 1:
-            x2 = x2.contiguous()
+            x2 = contiguous(x2)
         if weight.stride(1) != 1 and k > 1:
-            weight = weight.contiguous()
+            weight = contiguous(weight)
         lib = _lib.load()
         ld_dy, ld_x, ld_w = (dy.stride(0) if m > 1 else n), (x2.stride(0) if m > 1 else k), (weight.stride(0) if n > 1 else k)
         if need_input:
@@ -740,9 +817,9 @@ def linear_backward(x, weight, grad_output, need_input=True, need_weight=True, n
             db = colsum(dy)
         return dx, dw, db
     if x2.stride(1) != 1 and k > 1:
-        x2 = x2.contiguous()
+        x2 = contiguous(x2)
     if weight.stride(1) != 1 and k > 1:
-        weight = weight.contiguous()
+        weight = contiguous(weight)
     ld_dy, ld_x, ld_w = (dy.stride(0) if m > 1 else n), (x2.stride(0) if m > 1 else k), (weight.stride(0) if n > 1 else k)
     if need_input:
         # dx[m, j] = sum_n dy[m, n] w[n, j]: dy is read along n, w down its columns

@@ -37,7 +37,7 @@ class _HaloStaging(torch.autograd.Function):
     def forward(ctx, input, plan, ghost_bufs, bulk_bufs):
         x = input.detach()
         if not x.is_contiguous():
-            x = x.contiguous()
+            x = hip_ops.contiguous(x)
         ctx.plan = plan
         return plan.run(x, ghost_bufs, bulk_bufs)
 

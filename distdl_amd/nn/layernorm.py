@@ -42,7 +42,7 @@ def _shard_forward(input, weight, bias, P_reduce, part_cols, eps, part_cols_arr,
     cols = int(part_cols[P_reduce.rank if P_reduce.active else 0])
     x2d = x.reshape(-1, cols)
     if x2d.shape[1] > 1 and x2d.stride(1) != 1:
-        x2d = x2d.contiguous()
+        x2d = hip_ops.contiguous(x2d)
     gamma = None if weight is None else weight.detach().reshape(-1)
     beta = None if bias is None else bias.detach().reshape(-1)
     nparts = len(part_cols)
@@ -92,7 +92,7 @@ class _LayerNormShard(torch.autograd.Function):
         if dy2d.dtype != x2d.dtype:
             dy2d = dy2d.to(x2d.dtype)
         if dy2d.shape[1] > 1 and dy2d.stride(1) != 1:
-            dy2d = dy2d.contiguous()
+            dy2d = hip_ops.contiguous(dy2d)
         dx = dw = db = None
         w_shape, b_shape = ctx.param_shapes
         want_w, want_b = need_w and w_shape is not None, need_b and b_shape is not None

@@ -81,6 +81,26 @@ typedef struct ddl_box {
 int ddl_copy_boxes(const ddl_box_t* boxes, int nbox, int elem_size,
                    int op, int dtype, void* stream);
 
+/* One box summed over `nsrc` sources (1..64) in one pass:
+ *   dst[box] = (srcs[0][box] / divisor) + (srcs[1][box] / divisor) + ...
+ * added in the order of `srcs`, quotients and partial sums rounded to the
+ * element type, i.e. bit for bit what element-wise divisions followed by
+ * accumulating box copies give -- but every source is read once and the
+ * destination written once.  `box` supplies dst, shape, dst_stride and the
+ * src_stride shared by all sources (its src field is ignored); srcs[q] points
+ * at the first element of the box in source q, all a multiple of 16 bytes
+ * apart.  dst may be one of the sources (same strides) but must not overlap
+ * them otherwise.  Integer dtypes take divisor 1 only.
+ *
+ * Replaces the local reduction and re-layout of ReduceScatter,
+ *   backends/mpi_numpy/functional/reduce_scatter.py:86-119 (rearrange + MPI.SUM
+ *   into the own slab), the sum of AllSumReduce, all_sum_reduce.py:77-92, and
+ * the scaling of gradients ahead of the adjoint sums,
+ *   all_gather.py:188-190, all_sum_reduce.py:127-128, broadcast.py:208-209
+ *   (grad_output / scale_backward). */
+int ddl_sum_boxes(const ddl_box_t* box, const void* const* srcs, int nsrc,
+                  int elem_size, int dtype, double divisor, void* stream);
+
 /* Pack: for b in [0,nbox): bufs[b] (contiguous, C order, shape box_shape[b])
  *       = tensor[box_start[b] : box_start[b]+box_shape[b]].
  * `tensor_strides` are the element strides of the (possibly non-contiguous)

@@ -487,3 +487,102 @@ def test_box_accumulate_integers_wrap_around(dtype):
     hip_ops.copy_box(src.cuda(), [slice(0, 5), slice(0, 37), slice(0, 19)], d, [slice(1, 6), slice(2, 39), slice(3, 22)],
                      accumulate=True)
     assert torch.equal(d.cpu(), want)
+
+
+# ------------------------------------------------------------- sum of boxes --
+
+def _sequential_sum(srcs, divisor):
+    """What ddl_sum_boxes promises: every source divided (true division, in
+    fp32 for the 16-bit types, rounded to the element type), then added in
+    order with a rounding after every addition -- torch on the CPU, step by step."""
+    acc = None
+    for s in srcs:
+        t = s if divisor == 1 else (s / divisor).to(s.dtype)
+        acc = t.clone() if acc is None else (acc + t).to(s.dtype)
+    return acc
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16, torch.float16, torch.int32, torch.int64])
+@pytest.mark.parametrize("nsrc,divisor", [(1, 1), (1, 3), (3, 1), (8, 7), (64, 2)])
+def test_sum_boxes_matches_step_by_step_arithmetic(ops, dtype, nsrc, divisor):
+    """One launch = the chain of divisions and additions, bit for bit, on a
+    strided box of every source into a strided box of the destination."""
+    if not dtype.is_floating_point and divisor != 1:
+        pytest.skip("integers are summed, not divided")
+    gen = torch.Generator().manual_seed(nsrc * 100 + divisor)
+    shape, box = (5, 9, 44), (slice(1, 5), slice(2, 9), slice(4, 41))
+    if dtype.is_floating_point:
+        srcs = [(torch.randn(shape, generator=gen) * 3).to(dtype) for _ in range(nsrc)]
+    else:
+        srcs = [torch.randint(-2 ** 30, 2 ** 30, shape, generator=gen).to(dtype) for _ in range(nsrc)]
+        srcs[0][1, 2, 4] = torch.iinfo(dtype).max          # wraps around with the next addend
+        if nsrc > 1:
+            srcs[1][1, 2, 4] = 9
+    dst = torch.full((6, 8, 50), 5, dtype=dtype)
+    dbox = (slice(2, 6), slice(0, 7), slice(10, 47))
+    want = dst.clone()
+    want[dbox] = _sequential_sum([s[box] for s in srcs], divisor)
+    d = dst.cuda()
+    ops.sum_boxes([s.cuda() for s in srcs], box, d, dbox, divisor)
+    assert torch.equal(bits(d.cpu()), bits(want))
+
+
+def test_sum_boxes_in_place_and_fallbacks(ops):
+    """The destination may be one of the sources (scaling a gradient in place);
+    sources that are not 16 bytes apart, or more than 64 of them, go through
+    accumulating copies; what neither path can do is refused."""
+    gen = torch.Generator().manual_seed(5)
+    x = torch.randn(7, 33, generator=gen)
+    full = (slice(0, 7), slice(0, 33))
+    d = x.cuda()
+    ops.sum_boxes([d], full, d, full, 3)
+    assert torch.equal(d.cpu(), x / 3)
+    assert torch.equal(ops.scaled(x.cuda().t(), 5).cpu(), (x / 5).t())
+    pool = torch.randn(3 * 7 * 33 + 8, generator=gen).cuda()
+    odd = [pool[1 + q * 231: 1 + (q + 1) * 231].view(7, 33) for q in range(3)]       # 4 bytes past a 16-byte boundary, 924 apart
+    odd[1] = pool[2 + 231: 2 + 2 * 231].view(7, 33)
+    out = torch.empty(7, 33, device="cuda")
+    ops.sum_boxes(odd, full, out, full)
+    assert torch.equal(out.cpu(), _sequential_sum([t.cpu() for t in odd], 1))
+    with pytest.raises(ValueError):
+        ops.sum_boxes(odd, full, out, full, 2)
+    many = [torch.full((4, 8), float(q), device="cuda") for q in range(70)]
+    out = torch.empty(4, 8, device="cuda")
+    ops.sum_boxes(many, (slice(0, 4), slice(0, 8)), out, (slice(0, 4), slice(0, 8)))
+    assert torch.equal(out.cpu(), torch.full((4, 8), float(sum(range(70)))))
+    with pytest.raises(ValueError):
+        ops.sum_boxes([x.cuda(), x.cuda().double()], full, out, full)
+    from distdl_amd import _lib
+    lib = _lib.load()
+    box = _lib.ddl_box_t()
+    box.ndim = 1
+    box.shape[0], box.src_stride[0], box.dst_stride[0] = 8, 1, 1
+    box.dst = out.data_ptr()
+    ptrs = _lib.ptr_array([x.cuda().data_ptr()])
+    assert lib.ddl_sum_boxes(box, ptrs, 0, 4, _lib.DDL_DT_F32, 1.0, None) == -5
+    assert lib.ddl_sum_boxes(box, ptrs, 1, 4, _lib.DDL_DT_F32, 0.0, None) == -1
+    assert lib.ddl_sum_boxes(box, ptrs, 1, 4, _lib.DDL_DT_I32, 2.0, None) == -5
+    assert lib.ddl_sum_boxes(box, ptrs, 1, 2, _lib.DDL_DT_F32, 1.0, None) == -1
+
+
+def test_reduce_scatter_relayout_at_config4_activation_size(ops):
+    """The local half of a reduce-scatter over 8 workers at the activation
+    shape of configuration 4 ([4,2048,8192] bf16, split along the features):
+    the own slab of the sum of eight full tensors in one launch, against the
+    step-by-step sum on sampled rows and against linearity (the sum of A and of
+    B, scaled by powers of two, is exact)."""
+    gen = torch.Generator(device="cuda").manual_seed(77)
+    fulls = [torch.randn(4, 2048, 8192, generator=gen, device="cuda").to(torch.bfloat16) for _ in range(8)]
+    src = (slice(0, 4), slice(0, 2048), slice(3072, 4096))           # worker 3's slab
+    dst = (slice(0, 4), slice(0, 2048), slice(0, 1024))
+    out = torch.empty(4, 2048, 1024, dtype=torch.bfloat16, device="cuda")
+    ops.sum_boxes(fulls, src, out, dst)
+    rows = [0, 1, 777, 2047]
+    want = _sequential_sum([f[:, rows, 3072:4096].cpu() for f in fulls], 1)
+    assert torch.equal(bits(out[:, rows].cpu()), bits(want))
+    doubled = torch.empty_like(out)
+    ops.sum_boxes([ops.scaled(f, 0.5) for f in fulls], src, doubled, dst)        # every addend times two
+    quartered = torch.empty_like(out)
+    ops.sum_boxes(fulls, src, quartered, dst, 4)
+    assert torch.equal(bits(doubled.cpu()), bits((out.float() * 2).to(torch.bfloat16).cpu()))
+    assert torch.equal(bits(quartered.cpu()), bits((out.float() / 4).to(torch.bfloat16).cpu()))

@@ -49,7 +49,7 @@ def test_layernorm_layer_forward_replays_from_a_graph():
     whole = torch.randn(4, 64, 512, generator=gen)
     peers = [None] + [torch.from_numpy(o_ln.partial_stats(whole[..., 128 * p:128 * (p + 1)].numpy()).astype(np.float32)).cuda()
                       for p in range(1, 4)]
-    world.transport.set_gather_provider(STATS_TAG, lambda P, t: list(peers))
+    world.transport.set_gather_provider(STATS_TAG, lambda P, t: list(peers), constant=True)
 
     def make_input(i):
         g = torch.Generator().manual_seed(100 + i)

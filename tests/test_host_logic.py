@@ -208,8 +208,9 @@ def test_loopback_transport_moves_data_between_rank_threads():
 
 def test_allgather_into_fills_the_other_slots_in_place():
     """In-place all-gather: every worker writes its own slot, the transport fills
-    the rest (loopback), or leaves seeded slots alone and consults a provider
-    once per buffer (solo)."""
+    the rest (loopback); solo, the absent workers mirror the live one unless a
+    provider speaks for them, on every call or -- declared constant -- once per
+    buffer object."""
     world = SimWorld(3, device=torch.device("cpu"))
 
     def body(P):
@@ -228,19 +229,31 @@ def test_allgather_into_fills_the_other_slots_in_place():
     solo = SimWorld(3, device=torch.device("cpu"))
     P = solo.partition(1)
     buf = torch.zeros(3, 2)
-    buf[0], buf[2] = torch.tensor([7.0, 7.0]), torch.tensor([9.0, 9.0])      # seeded by the caller
+    buf[0], buf[2] = torch.tensor([7.0, 7.0]), torch.tensor([9.0, 9.0])
     buf[1] = 1.0
-    assert solo.transport.allgather_into(P, buf, tag="s") is buf and buf.tolist() == [[7, 7], [1, 1], [9, 9]]
+    assert not solo.transport.peers_gathered_ahead(P, buf, tag="s")
+    assert solo.transport.allgather_into(P, buf, tag="s") is buf and buf.tolist() == [[1, 1], [1, 1], [1, 1]]
+    assert torch.equal(solo.transport.allgather(P, buf[1], tag="s"), buf)      # the two gathers agree about the peers
     calls = []
 
     def provider(P_, mine):
         calls.append(1)
-        return [torch.full((2,), 3.0), None, torch.full((2,), 4.0)]
+        return [mine + 2.0, None, mine + 3.0]
     solo.transport.set_gather_provider("s", provider)
     solo.transport.allgather_into(P, buf, tag="s")
     buf[1] = 2.0
+    assert not solo.transport.peers_gathered_ahead(P, buf, tag="s")
     solo.transport.allgather_into(P, buf, tag="s")
-    assert buf.tolist() == [[3, 3], [2, 2], [4, 4]] and len(calls) == 1
+    assert buf.tolist() == [[4, 4], [2, 2], [5, 5]] and len(calls) == 2      # asked on every gather
+    solo.transport.set_gather_provider("s", provider, constant=True)
+    assert not solo.transport.peers_gathered_ahead(P, buf, tag="s")
+    solo.transport.allgather_into(P, buf, tag="s")
+    buf[1] = 6.0
+    assert solo.transport.peers_gathered_ahead(P, buf, tag="s")
+    solo.transport.allgather_into(P, buf, tag="s")
+    assert buf.tolist() == [[4, 4], [6, 6], [5, 5]] and len(calls) == 3      # once per buffer
+    other = torch.zeros(3, 2)                                                # another buffer object: asked again
+    assert not solo.transport.peers_gathered_ahead(P, other, tag="s")
 
 
 def test_loopback_transport_propagates_failures():
