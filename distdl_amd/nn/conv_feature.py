@@ -51,6 +51,32 @@ class _HaloStaging(torch.autograd.Function):
         return dx, None, None, None
 
 
+class _Crop(torch.autograd.Function):
+    """``padded[slices]`` as a contiguous tensor (reference :410, where the
+    slice is a view and the stock convolution makes the copy): one pass of the
+    box kernel over the window.  Adjoint: the gradient placed into a zeroed
+    tensor of the padded shape."""
+
+    @staticmethod
+    def forward(ctx, padded, slices):
+        src = padded.detach()
+        ctx.padded_shape, ctx.slices = tuple(src.shape), slices
+        out = torch.empty([int(s.stop) - int(s.start) for s in slices], dtype=src.dtype, device=src.device)
+        if out.numel():
+            hip_ops.copy_box(src, slices, out, [slice(0, n) for n in out.shape])
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        g = grad_output.detach()
+        dp = torch.empty(ctx.padded_shape, dtype=g.dtype, device=g.device)
+        whole = hip_ops.BoxPlan(dp.shape, dp.stride(), [([0] * dp.dim(), list(dp.shape))])
+        whole.zero(dp)
+        if g.numel():
+            hip_ops.copy_box(g, [slice(0, n) for n in g.shape], dp, ctx.slices)
+        return dp, None
+
+
 class DistributedFeatureConvBase(Module, HaloMixin, ConvMixin):
     r"""Convolution over a tensor partitioned in feature space only:
     ``P_x ~ 1 x 1 x P_{d-1} x ... x P_0``; the output reuses ``P_x``.  Weights
@@ -214,7 +240,12 @@ class DistributedFeatureConvBase(Module, HaloMixin, ConvMixin):
         else:
             padded = _HaloStaging.apply(input, self._pad_only_plan, None, None)
             exchanged = self.halo_layer(padded)
-        return exchanged[self.needed_slices]
+        crop = tuple(slice(int(sl.start), int(sl.stop)) for sl in self.needed_slices)
+        if all(sl.start == 0 and sl.stop == n for sl, n in zip(crop, exchanged.shape)):
+            return exchanged
+        # A window smaller than the padded tensor (strided or unbalanced
+        # geometries): handed to the convolution as a contiguous tensor.
+        return _Crop.apply(exchanged, crop)
 
     def _fused_slabs(self, input):
         """Ghost and bulk slabs of the fused pass as ``[dim][side]`` tables of
@@ -223,21 +254,39 @@ class DistributedFeatureConvBase(Module, HaloMixin, ConvMixin):
         when dimensions are exchanged one after the other; one pass over all
         dimensions needs a slab per (dimension, side, kind), so it asks the
         same buffer manager for that many buffers (the first four are the halo
-        layer's own: the two ways of staging never run together)."""
+        layer's own: the two ways of staging never run together).  A slab's
+        place in the pool is fixed by (dimension, side, kind), whether or not
+        the slab exists, so two layers of one manager agree on which buffer
+        is, say, the right ghost of dimension 3.  Pooled buffers are scratch:
+        another layer of the same manager overwrites them, so ghost slabs that
+        a caller seeds (solo transport) must be seeded again before each call
+        unless this layer has the manager to itself.  Ghost views are zeroed
+        when the layer first takes them, so slabs nobody seeded read as zeros."""
         plan = self._staging_plan
         slabs = getattr(self, "_fused_slab_cache", None)
         key = (tuple(input.shape), input.dtype, _buffer.reallocations())
         if slabs is None or slabs[0] != key:
+            first_time = slabs is None
             wanted = [(d, s, kind, plan.slab_shape(d, s, kind))
                       for d in range(plan.ndim) for s in range(2) for kind in ("ghost", "bulk")]
-            wanted = [w for w in wanted if w[3] is not None]
+            # dimensions in front of the first exchanged one take no place in the pool
+            first = next((i for i, w in enumerate(wanted) if w[3] is not None), len(wanted)) // 4 * 4
+            wanted = wanted[first:]
+            while wanted and wanted[-1][3] is None:
+                wanted.pop()
             pool = self.buffer_manager.request_buffers(len(wanted), dtype=input.dtype)
             for buf, w in zip(pool, wanted):
-                buf.allocate_view(w[3])        # may reallocate: take the views only afterwards
+                if w[3] is not None:
+                    buf.allocate_view(w[3])        # may reallocate: take the views only afterwards
             ghost = [[None, None] for _ in range(plan.ndim)]
             bulk = [[None, None] for _ in range(plan.ndim)]
             for buf, (d, s, kind, shape) in zip(pool, wanted):
-                (ghost if kind == "ghost" else bulk)[d][s] = buf.get_view(shape)
+                if shape is None:
+                    continue
+                view = buf.get_view(shape)
+                if kind == "ghost" and first_time:
+                    hip_ops.BoxPlan(view.shape, view.stride(), [([0] * view.dim(), list(view.shape))]).zero(view)
+                (ghost if kind == "ghost" else bulk)[d][s] = view
             key = (tuple(input.shape), input.dtype, _buffer.reallocations())
             slabs = self._fused_slab_cache = (key, ghost, bulk)
         return slabs[1], slabs[2]

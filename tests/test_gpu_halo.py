@@ -469,3 +469,144 @@ def test_solo_conv_staging_uses_fused_kernel_and_matches_oracle(ops):
         for s in range(2):
             if bulk[d][s] is not None:
                 assert np.array_equal(bulk[d][s].cpu().numpy(), want_bulks[d][s])
+
+
+# ------------------------------------- layers sharing one buffer manager --
+
+def _adjoint_tight(results):
+    """The reference's criterion (tests/adjoint_test.py:11-56) over the per-rank
+    tensors (x, dx, y, dy): <F x, dy> and <x, F* dy>, each divided by the larger
+    product of norms, agree to np.isclose."""
+    sums = np.zeros(6)
+    for x, dx, y, dy in results:
+        x, dx, y, dy = (t.double() for t in (x, dx, y, dy))
+        sums += [float((x * x).sum()), float((dx * dx).sum()), float((y * y).sum()), float((dy * dy).sum()),
+                 float((x * dx).sum()), float((y * dy).sum())]
+    nx1, nx2, ny1, ny2 = np.sqrt(sums[:4])
+    d = max(ny1 * ny2, nx1 * nx2)
+    assert d > 0 and np.isclose(sums[4] / d, sums[5] / d), (sums[4] / d, sums[5] / d)
+
+
+@pytest.mark.parametrize("repartitions_share_the_manager,counts_by_rank", [
+    # tests/utilities/test_buffer.py:226-343: only the convolutions use the manager
+    (False, {"c1": (4, 4, 4, 4), "c2": (4, 4, 4, 4), "c3": (4, 4, 4, 4), "backward": (4, 4, 4, 4)}),
+    # tests/utilities/test_buffer.py:346-466: the two repartitions use it too
+    (True, {"tr1": (3, 1, 1, 1), "c1": (4, 4, 4, 4), "c2": (4, 4, 4, 4), "c3": (4, 4, 4, 4), "tr2": (4, 4, 4, 4),
+            "backward": (4, 4, 4, 4)}),
+])
+def test_buffer_manager_shared_by_a_network_of_layers(repartitions_share_the_manager, counts_by_rank):
+    """The reference's networks of a scatter, three 3x3 convolutions over a 2x2
+    partition and a gather with ONE buffer manager, four workers moving real
+    data: the number of pooled float32 buffers after every layer's forward and
+    after the backward pass is the reference's, the output equals the three
+    stock convolutions on the whole tensor, and the chain passes the tight
+    adjoint test."""
+    from distdl_amd.backends.stub_hip import BufferManager
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedConv2d
+    from distdl_amd.nn import Repartition
+    from distdl_amd.utilities.torch import zero_volume_tensor
+    gen = torch.Generator().manual_seed(226)
+    x0 = torch.randn(1, 1, 5, 5, generator=gen)
+    dy0 = torch.randn(1, 20, 5, 5, generator=gen)
+    weights = [torch.randn(o, i, 3, 3, generator=gen) * 0.3 for i, o in ((1, 5), (5, 10), (10, 20))]
+
+    def body(P_world):
+        manager = BufferManager()
+        P_1 = P_world.create_partition_inclusive([0]).create_cartesian_topology_partition([1, 1, 1, 1])
+        P_22 = P_world.create_partition_inclusive([0, 1, 2, 3]).create_cartesian_topology_partition([1, 1, 2, 2])
+        shared = {"buffer_manager": manager} if repartitions_share_the_manager else {}
+        tr1 = Repartition(P_1, P_22, **shared)
+        convs = [DistributedConv2d(P_22, in_channels=i, out_channels=o, kernel_size=[3, 3], padding=[1, 1], bias=False,
+                                   buffer_manager=manager) for i, o in ((1, 5), (5, 10), (10, 20))]
+        tr2 = Repartition(P_22, P_1, **shared)
+        if P_22.rank == 0:
+            with torch.no_grad():
+                for conv, w in zip(convs, weights):
+                    conv.weight.copy_(w.cuda())
+        x = zero_volume_tensor(1, device="cuda")
+        if P_1.active:
+            x = x0.cuda()
+        x.requires_grad = True
+        counts = {}
+
+        def count():
+            return len(manager.buffers_map.get(torch.float32, []))
+        h = tr1(x)
+        counts["tr1"] = count()
+        for name, conv in zip(("c1", "c2", "c3"), convs):
+            h = conv(h)
+            counts[name] = count()
+        y = tr2(h)
+        counts["tr2"] = count()
+        dy = zero_volume_tensor(1, device="cuda")
+        if P_1.active:
+            dy = dy0.cuda()
+        y.backward(dy)
+        counts["backward"] = count()
+        torch.cuda.synchronize()
+        return counts, x.detach().cpu(), x.grad.cpu(), y.detach().cpu(), dy.cpu()
+
+    res = SimWorld(4).run(body)
+    for rank, (counts, *_) in enumerate(res):
+        for name, by_rank in counts_by_rank.items():
+            assert counts[name] == by_rank[rank], (name, rank, counts)
+    want = x0
+    for w in weights:
+        want = F.conv2d(want, w, padding=1)
+    assert torch.allclose(res[0][3], want, atol=1e-4, rtol=1e-4)
+    _adjoint_tight([r[1:] for r in res])
+
+
+K2S2_1D = {"id": "kernel-2-stride-2-1d", "P_x_shape": [1, 1, 4], "x_global_shape": [1, 1, 10], "kernel_size": [2],
+           "stride": [2], "padding": [0], "dilation": [1]}
+
+
+@pytest.mark.parametrize("geom_id", ["kernel-needs-offset", "kernel-2-stride-2-1d"])
+def test_feature_conv_with_cropped_staging_forward_and_backward(golden, geom_id):
+    """Strided geometries in which the needed range of some worker is smaller
+    than its padded shard (reference nn/conv_feature.py:410) -- one of the
+    reference's feature-conv test (tests/layers/test_conv_feature.py:9-247) and
+    the kernel 2 / stride 2 case of tests/utilities/test_halo_mixin.py:46-87:
+    the crop hands the convolution a contiguous window, and the output and the
+    input gradient equal those of the stock convolution on the whole tensor."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd import nn as dnn
+    geom = next(g for g in golden("layer_geometries.json")["conv_feature"] + [K2S2_1D] if g["id"] == geom_id)
+    P, gshape, k = geom["P_x_shape"], geom["x_global_shape"], geom["kernel_size"]
+    nd, n = len(k), int(np.prod(P))
+    Conv = {1: dnn.DistributedConv1d, 2: dnn.DistributedConv2d, 3: dnn.DistributedConv3d}[nd]
+    conv = {1: F.conv1d, 2: F.conv2d, 3: F.conv3d}[nd]
+    rng = np.random.default_rng(410)
+    x = rng.standard_normal(gshape).astype(np.float32)
+    w = torch.from_numpy(rng.standard_normal([4, gshape[1]] + k).astype(np.float32))
+    xr = torch.from_numpy(x).requires_grad_(True)
+    yr = conv(xr, w, None, stride=geom["stride"], padding=geom["padding"], dilation=geom["dilation"])
+    dy = rng.standard_normal(tuple(yr.shape)).astype(np.float32)
+    yr.backward(torch.from_numpy(dy))
+    shards, dys = o_rep.scatter(x, P), o_rep.scatter(dy, P)
+
+    def body(P_world):
+        P_x = P_world.create_partition_inclusive(list(range(n))).create_cartesian_topology_partition(P)
+        layer = Conv(P_x, in_channels=gshape[1], out_channels=4, kernel_size=k, stride=geom["stride"],
+                     padding=geom["padding"], dilation=geom["dilation"], bias=False)
+        if P_x.rank == 0:
+            with torch.no_grad():
+                layer.weight.copy_(w.cuda())
+        xin = torch.from_numpy(shards[P_x.rank]).cuda().requires_grad_(True)
+        layer._distdl_forward_pre_hook(layer, (xin,))
+        staged = layer.stage_input(xin)
+        padded_shape = [int(v) for v in np.asarray(xin.shape) + (layer.local_padding + layer.halo_shape).sum(axis=1)]
+        cropped = list(staged.shape) != padded_shape
+        assert staged.is_contiguous()
+        y = layer(xin)
+        y.backward(torch.from_numpy(dys[P_x.rank]).cuda())
+        torch.cuda.synchronize()
+        return y.detach().cpu().numpy(), xin.grad.cpu().numpy(), cropped
+
+    outs = SimWorld(n).run(body)
+    assert any(cropped for _, _, cropped in outs), "no worker of this geometry crops: the test would prove nothing"
+    for (y, _, _), part in zip(outs, o_rep.scatter(yr.detach().numpy(), P)):
+        assert np.allclose(y, part, atol=1e-4, rtol=1e-4)
+    for (_, dx, _), part in zip(outs, o_rep.scatter(xr.grad.numpy(), P)):
+        assert np.allclose(dx, part, atol=1e-4, rtol=1e-4)

@@ -1212,6 +1212,86 @@ def test_linear_backward_small_integer_cases_are_exact(ops, M, N, K):
     assert np.array_equal(db.cpu().double().numpy(), want_db)
 
 
+def test_linear_backward_config4_rank0(ops):
+    """The adjoint of configuration 4 at its full size (M 8192, N 3584, K 8192):
+    dx = dy w [8192, 8192], dw = dy^T x [3584, 8192], db = column sums, on the
+    operands where they lie.  Sampled rows (tile borders and both ends) against
+    the oracle's exact sums; on the whole outputs, linearity in dy (a factor of
+    two is exact in bf16) and agreement with the same products by the vendor
+    GEMM in fp32."""
+    gen = torch.Generator().manual_seed(1404)
+    x = torch.randn(8192, 8192, generator=gen).to(torch.bfloat16)
+    w = (0.02 * torch.randn(3584, 8192, generator=gen)).to(torch.bfloat16)
+    dy = torch.randn(8192, 3584, generator=gen).to(torch.bfloat16)
+    xg, wg, dyg = x.cuda(), w.cuda(), dy.cuda()
+    dx, dw, db = ops.linear_bf16_backward(xg, wg, dyg)
+    torch.cuda.synchronize()
+    assert dx.shape == (8192, 8192) and dw.shape == (3584, 8192) and db.shape == (3584,)
+    xb, wb, dyb = bits16(x), bits16(w), bits16(dy)
+    rows = np.r_[0:16, 255:258, 4094:4098, 8176:8192]
+    want_dx = o_lin.bf16_bits_to_f32(dyb[rows]).astype(np.float64) @ o_lin.bf16_bits_to_f32(wb).astype(np.float64)
+    err = np.abs(dx[rows].cpu().double().numpy() - want_dx)
+    assert (err <= LIN_RTOL * (np.abs(want_dx) + np.abs(want_dx).mean())).all()
+    nrows = np.r_[0:16, 191:194, 2046:2050, 3568:3584]
+    want_dw = o_lin.bf16_bits_to_f32(dyb[:, nrows]).astype(np.float64).T @ o_lin.bf16_bits_to_f32(xb).astype(np.float64)
+    err = np.abs(dw[nrows].cpu().double().numpy() - want_dw)
+    assert (err <= LIN_RTOL * (np.abs(want_dw) + np.abs(want_dw).mean())).all()
+    want_db = o_lin.bf16_bits_to_f32(dyb).astype(np.float64).sum(axis=0)
+    err = np.abs(db.cpu().double().numpy() - want_db)
+    assert (err <= LIN_RTOL * (np.abs(want_db) + np.abs(want_db).mean())).all()
+    dx2, dw2, db2 = ops.linear_bf16_backward(xg, wg, 2 * dyg)
+    assert torch.equal(dx2, 2 * dx) and torch.equal(dw2, 2 * dw) and torch.equal(db2, 2 * db)
+    ref_dx = dyg.float() @ wg.float()
+    assert float(((dx.float() - ref_dx).abs() / (ref_dx.abs() + ref_dx.abs().mean())).max()) <= LIN_RTOL
+    del ref_dx
+    ref_dw = dyg.float().t() @ xg.float()
+    assert float(((dw.float() - ref_dw).abs() / (ref_dw.abs() + ref_dw.abs().mean())).max()) <= LIN_RTOL
+
+
+def test_layernorm_backward_config1_rank0(ops):
+    """The adjoint of configuration 1 at its full size: rank 0's shard
+    [8192, 256] of rows of 1024 over four workers, the other workers' row sums
+    seeded from the oracle's fp64 quantities.  dx, dgamma, dbeta of both the
+    two-launch and the one-pass form against the fp64 closed form."""
+    rng = np.random.default_rng(1401)
+    rows, cols, P, eps = 16 * 512, 256, 4, 1e-5
+    xg = rng.standard_normal((rows, P * cols)).astype(np.float32)
+    dyg = rng.standard_normal((rows, P * cols)).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(P * cols)).astype(np.float32)
+    shards = [np.ascontiguousarray(xg[:, cols * p:cols * (p + 1)]) for p in range(P)]
+    dys = [np.ascontiguousarray(dyg[:, cols * p:cols * (p + 1)]) for p in range(P)]
+    gammas = [gamma[cols * p:cols * (p + 1)] for p in range(P)]
+    want_dx, want_dg, want_db = o_ln.backward_shards(shards, gammas, dys, eps)
+    x2d, dy2d, g = torch.from_numpy(shards[0]).cuda(), torch.from_numpy(dys[0]).cuda(), torch.from_numpy(gammas[0]).cuda()
+    parts = [torch.from_numpy(o_ln.partial_stats(s).astype(np.float32)).cuda() for s in shards]
+    parts[0] = ops.ln_partial_stats(x2d)
+    beta = torch.zeros(cols, device="cuda")
+    _, mean, rstd = ops.ln_normalize_affine(x2d, torch.stack(parts).contiguous(), [cols] * P, g, beta, eps, want_stats=True)
+    m64 = xg.astype(np.float64).mean(axis=1)
+    r64 = 1.0 / np.sqrt(xg.astype(np.float64).var(axis=1) + eps)
+    gathered = []
+    for p in range(P):
+        gp = dys[p].astype(np.float64) * gammas[p].astype(np.float64)
+        xh = (shards[p].astype(np.float64) - m64[:, None]) * r64[:, None]
+        gathered.append(torch.from_numpy(np.stack([gp.sum(axis=1), (gp * xh).sum(axis=1)], axis=1).astype(np.float32)).cuda())
+    sums, work = ops.ln_backward_partial_params(dy2d, x2d, mean, rstd, g)
+    assert np.allclose(sums.cpu().numpy(), gathered[0].cpu().numpy(), rtol=1e-4, atol=1e-3)
+    gathered[0] = sums
+    table = torch.stack(gathered).contiguous()
+    dx, dg, db = ops.ln_backward_input_params(dy2d, x2d, mean, rstd, g, table, 1.0 / (P * cols), work)
+    torch.cuda.synchronize()
+    tol = 1e-5 * max(1.0, np.abs(want_dx[0]).max())
+    assert np.abs(dx.cpu().numpy() - want_dx[0]).max() <= 4 * tol
+    # column sums over 8192 rows of O(1) terms: 1e-5 of the sum of magnitudes
+    assert np.abs(dg.cpu().numpy() - want_dg[0]).max() <= 1e-5 * np.abs(dys[0]).sum(axis=0).max() * 4
+    assert np.abs(db.cpu().numpy() - want_db[0]).max() <= 1e-5 * np.abs(dys[0]).sum(axis=0).max()
+    poisoned = table.clone()
+    poisoned[0] = float("nan")
+    dx1, dg1, db1 = ops.ln_backward_one_pass(dy2d, x2d, mean, rstd, g, 1.0 / (P * cols), poisoned, 0)
+    torch.cuda.synchronize()
+    assert torch.equal(poisoned, table) and torch.equal(dx1, dx) and torch.equal(dg1, dg) and torch.equal(db1, db)
+
+
 def test_linear_shard_autograd_matches_torch(ops):
     """The reference's layer runs torch autograd through F.linear; the same
     gradients must come out of the HIP path (bf16 tolerance), including through
