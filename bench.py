@@ -1100,8 +1100,6 @@ WORKLOADS = {
     "mfma_32x32x16_random": (_build_mfma_probe(0, 1), 1, 1, "mfma", None, None, None, None),
     "mfma_16x16x32_constant": (_build_mfma_probe(1, 0), 1, 1, "mfma", None, None, None, None),
     "mfma_16x16x32_random": (_build_mfma_probe(1, 1), 1, 1, "mfma", None, None, None, None),
-    "mfma_16x16x32_lds_constant": (_build_mfma_probe(2, 0), 1, 1, "mfma", None, None, None, None),
-    "mfma_16x16x32_lds_random": (_build_mfma_probe(2, 1), 1, 1, "mfma", None, None, None, None),
     # only with --only:
     "layernorm_local_bwd_two_passes": (build_layernorm_local_bwd_two_passes, 8, 2, "hbm", None, None, None, None),
     "linear_library": (build_linear_library, 4, 1, "mfma", None, None, None, None),

@@ -11,8 +11,7 @@
 //                        int64_t sink_elems, int64_t* flop, void* stream)
 //       enqueues a kernel of nothing but bf16 MFMAs on register operands (512
 //       workgroups of 256 threads: two wavefronts per SIMD on 256 CUs);
-//       instruction 0: v_mfma_f32_32x32x16_bf16, 1: v_mfma_f32_16x16x32_bf16,
-//       2: the latter with fresh operands read from LDS for every k-step;
+//       instruction 0: v_mfma_f32_32x32x16_bf16, 1: v_mfma_f32_16x16x32_bf16;
 //       random 0: every operand element 1.0, 1: N(0,1) x 0.02 N(0,1) operands
 //       (on random operands the chip runs against its power limit); `iters`
 //       loop iterations of 2^20 flop per wavefront, the flop count of the launch
@@ -113,55 +112,6 @@ __global__ __launch_bounds__(kProbeThreads) void mfma_probe_16x16x32(float* sink
     sink[t] = sum;
 }
 
-// The same 64 MFMAs of 16x16x32 per iteration, but every k-step's operands are
-// fresh: 4 + 8 fragments of 1 KiB read from LDS (filled once with the same kind
-// of data) at an offset that moves with the k-step, the next k-step's reads
-// issued under the current one's MFMAs -- the operand traffic of the shard
-// GEMM's inner loop without its global loads, barriers and epilogue.  What
-// the matrix cores sustain when their operands change with every instruction,
-// as they do in a real product.
-constexpr int kProbeLdsBytes = 60 * 1024;   // five k-steps of 12 KiB per workgroup, two workgroups per CU
-
-__global__ __launch_bounds__(kProbeThreads) void mfma_probe_16x16x32_lds(float* sink, int iters, int random) {
-    constexpr int TN = 4, TM = 8;
-    __shared__ __attribute__((aligned(16))) char lds[kProbeLdsBytes];
-    const uint32_t t = blockIdx.x * kProbeThreads + threadIdx.x;
-    for (int i = threadIdx.x; i < kProbeLdsBytes / 16; i += kProbeThreads) {
-        const int frag = (i / 64) % 12;   // fragments 0..3 of a k-step feed the A port, 4..11 the B port
-        *reinterpret_cast<bf16x8*>(lds + i * 16) = operand(blockIdx.x * 8192u + i, frag < TN ? 0.02f : 1.0f, random);
-    }
-    __syncthreads();
-    const char* mine = lds + (threadIdx.x & 63) * 16;
-    bf16x8 a[2][TN], b[2][TM];
-    auto fetch = [&](int buf, int step) {
-        const char* p = mine + (step % 5) * (12 * 1024);
-#pragma unroll
-        for (int i = 0; i < TN; ++i) a[buf][i] = *reinterpret_cast<const bf16x8*>(p + i * 1024);
-#pragma unroll
-        for (int j = 0; j < TM; ++j) b[buf][j] = *reinterpret_cast<const bf16x8*>(p + (TN + j) * 1024);
-    };
-    floatx4 acc[TN][TM];
-    for (int i = 0; i < TN; ++i)
-        for (int j = 0; j < TM; ++j)
-            for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
-    fetch(0, 0);
-    for (int it = 0; it < iters; ++it) {
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            fetch(s ^ 1, 2 * it + s + 1);
-#pragma unroll
-            for (int i = 0; i < TN; ++i)
-#pragma unroll
-                for (int j = 0; j < TM; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][i], b[s][j], acc[i][j], 0, 0, 0);
-        }
-    }
-    float sum = 0.f;
-    for (int i = 0; i < TN; ++i)
-        for (int j = 0; j < TM; ++j)
-            for (int e = 0; e < 4; ++e) sum += acc[i][j][e];
-    sink[t] = sum;
-}
-
 }  // namespace
 }  // namespace ddl
 
@@ -175,16 +125,14 @@ int bench_probe_launch(int64_t workgroups, int threads, void* stream) {
 
 int bench_probe_mfma(int instruction, int random, int iters, float* sink, int64_t sink_elems, int64_t* flop, void* stream) {
     using namespace ddl;
-    if (instruction < 0 || instruction > 2 || iters < 1 || iters > (1 << 24)) return -2;
+    if ((instruction != 0 && instruction != 1) || iters < 1 || iters > (1 << 24)) return -2;
     if (!sink || sink_elems < static_cast<int64_t>(kProbeBlocks) * kProbeThreads) return -2;
     if (flop) *flop = static_cast<int64_t>(kProbeBlocks) * (kProbeThreads / 64) * iters * kProbeFlopPerWaveIter;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (instruction == 0)
         hipLaunchKernelGGL(mfma_probe_32x32x16, dim3(kProbeBlocks), dim3(kProbeThreads), 0, s, sink, iters, random ? 1 : 0);
-    else if (instruction == 1)
-        hipLaunchKernelGGL(mfma_probe_16x16x32, dim3(kProbeBlocks), dim3(kProbeThreads), 0, s, sink, iters, random ? 1 : 0);
     else
-        hipLaunchKernelGGL(mfma_probe_16x16x32_lds, dim3(kProbeBlocks), dim3(kProbeThreads), 0, s, sink, iters, random ? 1 : 0);
+        hipLaunchKernelGGL(mfma_probe_16x16x32, dim3(kProbeBlocks), dim3(kProbeThreads), 0, s, sink, iters, random ? 1 : 0);
     return static_cast<int>(hipGetLastError());
 }
 

@@ -22,7 +22,7 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def _both(lib, dy, ids, lo, hi, padding_idx):
+def _both(lib, dy, ids, lo, hi, padding_idx, by_freq=0):
     """(static result, workspace result) of one gradient call; dy [n, dim], ids [n]."""
     n, dim = dy.shape
     rows = hi - lo
@@ -32,13 +32,22 @@ def _both(lib, dy, ids, lo, hi, padding_idx):
     got = torch.full((rows, dim), 7, dtype=dy.dtype, device="cuda")
     ref = torch.full((rows, dim), 9, dtype=dy.dtype, device="cuda")
     work = torch.full((2 * rows + 1 + n,), -1, dtype=torch.int32, device="cuda")
+    # The call is made twice and the second one is watched: the first call on a device looks up the built-in array's
+    # address, and the first launch of a kernel may make the runtime grow its own pools -- neither is the entry point's doing.
+    rc = lib.ddl_embedding_backward_static(dy.data_ptr(), dt, dim, dim, ids.data_ptr(), i64, n, lo, hi, padding_idx,
+                                           by_freq, got.data_ptr(), dim, _stream())
+    _lib.check(rc, "ddl_embedding_backward_static")
+    got.fill_(7)
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
-    rc = lib.ddl_embedding_backward_static(dy.data_ptr(), dt, dim, dim, ids.data_ptr(), i64, n, lo, hi, padding_idx, 0,
+    free_before, _ = torch.cuda.mem_get_info()          # the driver's own count: sees allocations torch's allocator does not
+    rc = lib.ddl_embedding_backward_static(dy.data_ptr(), dt, dim, dim, ids.data_ptr(), i64, n, lo, hi, padding_idx, by_freq,
                                            got.data_ptr(), dim, _stream())
     _lib.check(rc, "ddl_embedding_backward_static")
+    torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
-    rc = lib.ddl_embedding_backward(dy.data_ptr(), dt, dim, dim, ids.data_ptr(), i64, n, lo, hi, padding_idx, 0,
+    assert torch.cuda.mem_get_info()[0] == free_before
+    rc = lib.ddl_embedding_backward(dy.data_ptr(), dt, dim, dim, ids.data_ptr(), i64, n, lo, hi, padding_idx, by_freq,
                                     ref.data_ptr(), dim, work.data_ptr(), work.numel(), _stream())
     _lib.check(rc, "ddl_embedding_backward")
     torch.cuda.synchronize()
@@ -66,6 +75,29 @@ def test_static_entry_matches_workspace_entry_on_two_calls_in_a_row(dtype):
         exact = o_emb.backward(dy.double().numpy(), ids.numpy(), lo, lo + rows, padding_idx=pad)
         err = np.abs(got.cpu().double().numpy() - exact)
         assert (err <= 2.0 ** -7 * np.abs(exact) + 1e-5).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_static_entry_long_buckets_and_frequency_scaling_on_the_shared_array(dtype):
+    """Two calls in a row on the built-in array whose buckets take the sorted
+    paths -- a row with a few hundred tokens (sorted in LDS) and one with more
+    than 8192 (sorted in place) -- the first with scale_grad_by_freq, the second
+    smaller and without: bit for bit the workspace entry point's results."""
+    lib = _lib.load()
+    gen = torch.Generator().manual_seed(78)
+    for rows, tokens, dim, hot, by_freq in ((500, 30000, 64, (9000, 300), 1), (120, 12000, 40, (8300, 70), 0)):
+        lo = 3
+        ids = torch.randint(0, rows + 40, (tokens,), generator=gen)
+        order = torch.randperm(tokens, generator=gen)
+        ids[order[:hot[0]]] = lo + 7                     # more than 8192 tokens on one row
+        ids[order[hot[0]:hot[0] + hot[1]]] = lo + 8      # more than 64 on another
+        dy = torch.randn(tokens, dim, generator=gen).to(dtype)
+        got, ref = _both(lib, dy.cuda(), ids.cuda(), lo, lo + rows, -1, by_freq)
+        assert np.array_equal(_bits(got), _bits(ref))
+        exact = o_emb.backward(dy.double().numpy(), ids.numpy(), lo, lo + rows, scale_grad_by_freq=bool(by_freq))
+        err = np.abs(got.cpu().double().numpy() - exact)
+        tol = 2.0 ** -7 if dtype == torch.bfloat16 else 1e-5
+        assert (err <= tol * (np.abs(exact) + np.abs(exact).max())).all()
 
 
 def test_static_entry_exact_small_integers():
