@@ -1086,8 +1086,8 @@ WORKLOADS = {
     "halo_interior": (build_halo_interior, 4, 1, "hbm", None, None, None, None),
     "halo_slabs": (build_halo_slabs, 8, 6, "hbm", None, None, None, None),
     "halo_slabs_interior": (build_halo_slabs_interior, 8, 6, "hbm", None, None, None, None),
-    "all_gather_relayout": (build_all_gather_relayout, 3, 1, "hbm", None, None, None, None),
-    "reduce_scatter_relayout": (build_reduce_scatter_relayout, 2, 1, "hbm", None, None, None, None),
+    "all_gather_relayout": (build_all_gather_relayout, 3, 1, "hbm", "sum", None, None, None),
+    "reduce_scatter_relayout": (build_reduce_scatter_relayout, 2, 1, "hbm", "sum", None, None, None),
     "layernorm_bwd": (build_layernorm_bwd, 32, 2, "hbm", None, None, None, None),
     "layernorm_bwd_one_pass": (_build_layernorm_bwd_one_pass(16 * 512, 256, 4), 32, 2, "hbm", None, None, None, None),
     "layernorm_local_bwd": (_build_layernorm_bwd_one_pass(16 * 512, 1024, 1), 8, 2, "hbm", None, None, None, None),
