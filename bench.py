@@ -640,7 +640,7 @@ def layer_linear(torch):
     layer = DistributedLinearAllGather(P_y, 8192, 28672, dtype=torch.bfloat16)
     xs = [torch.randn(4, 2048, 8192, generator=torch.Generator().manual_seed(3004 + s)).to(torch.bfloat16).cuda()
           for s in range(4)]                                         # 4 x 128 MiB
-    rec = time_layer(torch, layer, xs, calls=48, warm=4)
+    rec = time_layer(torch, layer, xs, calls=120, warm=20)           # as many steps as the kernel's own timing: the clock settles
     rec["module"] = "DistributedLinearAllGather([1,1,8], 8192, 28672, bf16).forward, no_grad, rank 0 of 8, x whole"
     return rec
 
