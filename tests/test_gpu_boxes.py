@@ -85,6 +85,46 @@ def test_pack_unpack_random_boxes(ops, dtype, shape):
     assert torch.equal(bits(y.cpu()), want)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.uint8])
+@pytest.mark.parametrize("rows,strip,nbox,axis", [
+    (64, 1024, 8, 1),      # equal column strips of 2 KiB (bf16): whole tiles of 8 rows, box after box
+    (64, 1024, 16, 1),     # a full batch of sixteen boxes
+    (16, 1024, 17, 1),     # one more than a launch holds: a batch of sixteen equal boxes and one of one
+    (60, 1024, 4, 1),      # rows that are no whole number of tiles: the general kernel
+    (64, 1000, 4, 1),      # strips that are no whole number of 16-byte vectors per tile row
+    (8, 64, 3, 1),         # tiny
+    (4, 40960, 1, 1),      # one box of long contiguous rows
+    (6, 32768, 8, 0),      # equal slabs of long runs (64 KiB and more): boxes take turns, 4 KiB per wavefront
+    (6, 16384, 2, 0),      # runs of 16 KiB to 64 KiB: box after box, 4 KiB per wavefront
+    (3, 8200, 5, 0),       # long runs that are no whole number of tiles
+])
+def test_equal_boxes_pack_and_unpack_bit_exact(ops, dtype, rows, strip, nbox, axis):
+    """Batches of boxes that differ only in their base addresses take a kernel
+    of their own when their extents are whole tiles, the general kernel
+    otherwise; either way every bit arrives.  Column strips of a matrix
+    (axis 1: the pack of a Repartition along the last dimension) and slabs of
+    rows (axis 0: its unpack), random bit patterns."""
+    gen = torch.Generator().manual_seed(rows * 7 + strip + nbox)
+    shape = (rows, strip * nbox) if axis == 1 else (nbox, rows, strip)
+    x_cpu = random_bits(shape, dtype, gen)
+    x = x_cpu.cuda()
+    if axis == 1:
+        boxes = [(slice(0, rows), slice(strip * j, strip * (j + 1))) for j in range(nbox)]
+    else:
+        boxes = [(slice(j, j + 1), slice(0, rows), slice(0, strip)) for j in range(nbox)]
+    plan = ops.BoxPlan.from_slices(x, boxes)
+    bufs = [torch.zeros([s.stop - s.start for s in sl], dtype=dtype, device="cuda") for sl in boxes]
+    plan.pack(x, bufs)
+    for sl, buf in zip(boxes, bufs):
+        assert np.array_equal(to_np_bits(buf), to_np_bits(x_cpu[sl]))
+    y = torch.zeros_like(x)
+    plan.unpack(y, bufs[::-1])                         # buffers in reverse: every box lands where its slot says
+    want = torch.zeros_like(bits(x_cpu))
+    for sl, src in zip(boxes, boxes[::-1]):
+        want[sl] = bits(x_cpu)[src]
+    assert torch.equal(bits(y.cpu()), want)
+
+
 def test_pack_from_non_contiguous_tensor(ops):
     gen = torch.Generator().manual_seed(11)
     base = random_bits((9, 12, 10), torch.float32, gen).cuda()

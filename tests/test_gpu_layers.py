@@ -248,6 +248,41 @@ def test_layernorm_layer_takes_one_launch_once_the_peers_are_seeded(ops):
     assert torch.equal(y_first, y_second) and torch.equal(y_first, y_grad.detach())
 
 
+def test_layernorm_layer_solo_without_a_provider_is_consistent(ops):
+    """One live worker of four and nobody speaking for the others: the absent
+    workers hold what the live one holds, in the forward's gather and in the
+    backward's alike, so the layer is the layer norm of the live shard over its
+    own columns and its gradients are that function's (torch autograd)."""
+    from distdl_amd.backends.stub_hip import SimWorld
+    from distdl_amd.nn import DistributedLayerNorm
+    world = SimWorld(4)
+    P_x = world.partition(0).create_partition_inclusive(list(range(4))).create_cartesian_topology_partition([1, 1, 4])
+    layer = DistributedLayerNorm(P_x, [1024])
+    gen = torch.Generator().manual_seed(151)
+    with torch.no_grad():
+        layer.weight.copy_((1 + 0.1 * torch.randn(layer.weight.shape, generator=gen)).cuda())
+        layer.bias.copy_((0.1 * torch.randn(layer.bias.shape, generator=gen)).cuda())
+    x = torch.randn(3, 37, 256, generator=gen)
+    dy = torch.randn(3, 37, 256, generator=gen)
+    for _ in range(2):                                  # the second call finds the statistics buffer of the first
+        xg = x.cuda().requires_grad_(True)
+        y = layer(xg)
+        y.backward(dy.cuda())
+        xr = x.double().requires_grad_(True)
+        w = layer.weight.detach().cpu().double().reshape(-1).requires_grad_(True)
+        b = layer.bias.detach().cpu().double().reshape(-1).requires_grad_(True)
+        yr = F.layer_norm(xr, (256,), w, b, layer.eps)
+        yr.backward(dy.double())
+        assert torch.allclose(y.detach().cpu().double(), yr.detach(), rtol=1e-5, atol=1e-5)
+        assert torch.allclose(xg.grad.cpu().double(), xr.grad, rtol=1e-4, atol=1e-5)
+        assert torch.allclose(layer.weight.grad.cpu().double().reshape(-1), w.grad, rtol=1e-4, atol=1e-4)
+        assert torch.allclose(layer.bias.grad.cpu().double().reshape(-1), b.grad, rtol=1e-4, atol=1e-4)
+        layer.weight.grad = layer.bias.grad = None
+        with torch.no_grad():
+            y2 = layer(x.cuda())                        # the path without autograd: the same numbers
+        assert torch.equal(y2, y.detach())
+
+
 def test_layernorm_layer_single_worker_and_bf16(ops):
     """The layer on one worker takes the single-launch kernel (the reference's
     F.layer_norm branch) and is differentiable; a bf16 forward beside it."""
