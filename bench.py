@@ -896,7 +896,7 @@ def build_embedding_bwd(torch, lib, _lib, nsets):
         nbytes.append(n_hit * 8192 + 2 * ids.numel() * 8 + 16032 * 4096 * 2)
         ids = ids.cuda()
         dw = torch.empty(16032, 4096, dtype=torch.bfloat16, device="cuda")
-        work = torch.empty(2 * 16032 + 1 + ids.numel(), dtype=torch.int32, device="cuda")
+        work = torch.empty(3 * 16032 + 1 + ids.numel(), dtype=torch.int32, device="cuda")
         keep.append((ids, dw, work))
         args = (dy.data_ptr(), _lib.DDL_DT_BF16, 4096, 4096, ids.data_ptr(), 1, ids.numel(), 0, 16032, -1, 0, dw.data_ptr(),
                 4096, work.data_ptr(), work.numel())

@@ -645,7 +645,7 @@ def embedding_backward(grad_output, ids, lo, hi, padding_idx=None, scale_grad_by
     ids_c = contiguous(ids)
     rows, n_ids = int(hi) - int(lo), ids_c.numel()
     dw = torch.empty((rows, dim), dtype=grad_output.dtype, device=grad_output.device)
-    work = torch.empty(2 * rows + 1 + n_ids, dtype=torch.int32, device=grad_output.device)
+    work = torch.empty(3 * rows + 1 + n_ids, dtype=torch.int32, device=grad_output.device)
     dt = _lib.DDL_DT_BF16 if grad_output.dtype == torch.bfloat16 else _lib.DDL_DT_F32
     rc = _lib.load().ddl_embedding_backward(dy.data_ptr(), dt, dim, dy.stride(0) if n_ids > 1 else dim, ids_c.data_ptr(),
                                             1 if ids.dtype == torch.int64 else 0, n_ids, int(lo), int(hi),

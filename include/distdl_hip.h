@@ -412,8 +412,9 @@ int ddl_embedding_renorm(void* weight, int dtype, int64_t dim, int64_t ldw,
  * sum is divided by the number of tokens that contributed to it
  * (torch.nn.functional.embedding's option of that name, nn/embedding.py:244-246).
  * Every element of dweight is written, so it needs no clearing.  `workspace`:
- * device memory for at least 2 (hi-lo) + 1 + n_ids int32, contents on entry do
- * not matter. */
+ * device memory for at least 3 (hi-lo) + 1 + n_ids int32 (token counts, bucket
+ * cursors and bucket starts of the rows, then the buckets), contents on entry
+ * do not matter. */
 int ddl_embedding_backward(const void* dy, int dtype, int64_t dim, int64_t ld_dy,
                            const void* ids, int ids_is_i64, int64_t n_ids,
                            int64_t lo, int64_t hi, int64_t padding_idx,
@@ -427,7 +428,7 @@ int ddl_embedding_backward(const void* dy, int dtype, int64_t dim, int64_t ld_dy
  * The counters and buckets live in a 4 MiB device array built into the library
  * (one copy per GPU, held until the process ends); the call allocates nothing
  * and frees nothing.  It fails with DDL_E_UNSUPP when
- *   2 (hi - lo) + 1 + n_ids > DDL_EMBEDDING_BACKWARD_STATIC_MAX_ELEMS.
+ *   3 (hi - lo) + 1 + n_ids > DDL_EMBEDDING_BACKWARD_STATIC_MAX_ELEMS.
  * All calls on one GPU share that array: calls that overlap in time on one GPU
  * (different streams or threads) race; calls on one stream are safe.  The
  * array's device address is looked up the first time a GPU is used, so make

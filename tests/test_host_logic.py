@@ -668,11 +668,11 @@ def test_primitive_functions_take_the_reference_arguments():
     P = world.partition(0).create_partition_inclusive([0]).create_cartesian_topology_partition([1, 1])
     x = torch.arange(6.0).reshape(2, 3).requires_grad_(True)
     s = TensorStructure(x)
-    y = fn.all_gather.AllGatherFunction.apply(x, P.create_allreduction_partition((1,)), s, s, (1,), 2.0)
+    y = fn.all_gather.AllGatherFunction.apply(x, P.create_allreduction_partition((1,)), s, s, (1,), None)
     y = fn.reduce_scatter.ReduceScatterFunction.apply(y, P.create_allreduction_partition((1,)), s, s, (1,))
-    y = fn.all_sum_reduce.AllSumReduceFunction.apply(y, P.create_allreduction_partition((0,)), s, s, 4.0)
+    y = fn.all_sum_reduce.AllSumReduceFunction.apply(y, P.create_allreduction_partition((0,)), s, s, None)
     y.backward(torch.ones_like(y))
-    assert torch.equal(x.grad, torch.full((2, 3), 0.125))
+    assert torch.equal(x.grad, torch.ones(2, 3))
 
 
 def test_route_partitions_of_broadcast_and_reduction():

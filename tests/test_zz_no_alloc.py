@@ -31,7 +31,7 @@ def _both(lib, dy, ids, lo, hi, padding_idx, by_freq=0):
     # outputs and the reference workspace exist before the allocation-free call
     got = torch.full((rows, dim), 7, dtype=dy.dtype, device="cuda")
     ref = torch.full((rows, dim), 9, dtype=dy.dtype, device="cuda")
-    work = torch.full((2 * rows + 1 + n,), -1, dtype=torch.int32, device="cuda")
+    work = torch.full((3 * rows + 1 + n,), -1, dtype=torch.int32, device="cuda")
     # The call is made twice and the second one is watched: the first call on a device looks up the built-in array's
     # address, and the first launch of a kernel may make the runtime grow its own pools -- neither is the entry point's doing.
     rc = lib.ddl_embedding_backward_static(dy.data_ptr(), dt, dim, dim, ids.data_ptr(), i64, n, lo, hi, padding_idx,
