@@ -85,6 +85,7 @@ def parse_args():
     ap.add_argument("--all", action="store_true", help="every workload of WORKLOADS except the comparison figures "
                     "(backward kernels, fp32 GEMM, slab-only halo, MFMA probes, ...) instead of the default set")
     ap.add_argument("--no-graph", action="store_true", help="launch on the stream instead of replaying a HIP graph")
+    ap.add_argument("--cpu-worker", default=None, help=argparse.SUPPRESS)
     return ap.parse_args()
 
 
@@ -329,24 +330,60 @@ def layer_repartition(torch):
     return rec
 
 
-def cpu_repartition(budget_s=12.0):
-    """One rank's pack + unpack of config 2 with the oracle's NumPy code
-    (np.copyto per box, zero-filled output), single thread, uint16 views of the
-    bf16 payload."""
+def _cpu_repartition_rank(rank, budget_s):
+    """(steps, seconds) of one rank's pack + unpack of config 2 with the
+    oracle's NumPy code (np.copyto per box, zero-filled output), single thread,
+    uint16 views of the bf16 payload."""
     import numpy as np
     from oracle import repartition as o_rep
     send, recv, _, _ = o_rep.plan([8, 4096, 8192], [1, 8, 1], [1, 1, 8])
-    send0 = [(sl, sh, 99 if p == "self" else p) for sl, sh, p in send[0]]
-    recv0 = [(sl, sh, 99 if p == "self" else p) for sl, sh, p in recv[0]]
-    rng = np.random.default_rng(1002)
+    send_r = [(sl, sh, 99 if p == "self" else p) for sl, sh, p in send[rank]]
+    recv_r = [(sl, sh, 99 if p == "self" else p) for sl, sh, p in recv[rank]]
+    rng = np.random.default_rng(1002 + rank)
     x = rng.integers(0, 2 ** 16, size=(8, 512, 8192), dtype=np.uint16)
     rbufs = [rng.integers(0, 2 ** 16, size=(8, 512, 1024), dtype=np.uint16) for _ in range(8)]
 
     def step():
-        o_rep.pack(x, send0)
-        o_rep.unpack(recv0, rbufs, (8, 4096, 1024), np.uint16)
-    n, dt = timed_cpu(step, budget_s)
-    return {"value": 268435456 * n / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+        o_rep.pack(x, send_r)
+        o_rep.unpack(recv_r, rbufs, (8, 4096, 1024), np.uint16)
+    return timed_cpu(step, budget_s)
+
+
+def cpu_worker(spec):
+    """`bench.py --cpu-worker repartition:RANK:SECONDS`: one rank of the CPU
+    baseline as a process of its own (NumPy only, nothing touches the GPU);
+    prints {"steps", "seconds"}."""
+    what, rank, seconds = spec.split(":")
+    if what != "repartition":
+        raise SystemExit(f"bench.py: no CPU worker for {what!r}")
+    n, dt = _cpu_repartition_rank(int(rank), float(seconds))
+    print(json.dumps({"steps": n, "seconds": dt}))
+
+
+def cpu_repartition_all_ranks(budget_s=6.0, ranks=8):
+    """The eight ranks of config 2 at once, one process each, as `mpirun -np 8`
+    would run the reference's CPU backend (without its messages): what the box's
+    cores sustain together, next to the one rank the GPU's figure stands for."""
+    import subprocess
+    procs = [subprocess.Popen([sys.executable, os.path.abspath(__file__), "--cpu-worker", f"repartition:{r}:{budget_s}"],
+                              stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True) for r in range(ranks)]
+    rates = []
+    for p in procs:
+        out, _ = p.communicate(timeout=120 + 10 * budget_s)
+        if p.returncode != 0:
+            return None
+        rec = json.loads(out.strip().splitlines()[-1])
+        rates.append(268435456 * rec["steps"] / rec["seconds"] / 1e9)
+    return {"processes": ranks, "value": sum(rates), "unit": "GB/s", "per_process": sum(rates) / len(rates),
+            "what": f"{ranks} rank processes running config 2's pack + unpack at the same time, {budget_s:.0f} s each, summed"}
+
+
+def cpu_repartition(budget_s=12.0):
+    """One rank's pack + unpack of config 2 on one core, and all eight ranks at
+    once on eight processes."""
+    n, dt = _cpu_repartition_rank(0, budget_s)
+    return {"all_ranks": cpu_repartition_all_ranks(),
+            "value": 268435456 * n / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": f"{n} full steps of config 2, np.copyto per box + zero-filled output, one process as rank 0, {dt:.1f} s"}
 
 
@@ -1126,11 +1163,15 @@ def cpu_host():
     except OSError:
         pass
     return {"nproc": os.cpu_count(), "affinity": len(os.sched_getaffinity(0)), "torch_threads": torch.get_num_threads(),
-            "cpu_model": model, "launch": "single process standing in for rank 0 (no mpirun: mpi4py is not installed)"}
+            "cpu_model": model, "launch": "one process standing in for rank 0 (no mpirun: mpi4py is not installed); "
+                                          "cpu_baseline.all_ranks: the headline's eight ranks as eight processes at once"}
 
 
 def main():
     args = parse_args()
+    if args.cpu_worker:
+        cpu_worker(args.cpu_worker)
+        return
     if args.gpus != 1:
         sys.stderr.write("bench.py measures one rank's share on ONE GPU; --gpus N with N > 1 is not part of this build "
                          "(no collectives, no cross-GPU sharding).\n")
