@@ -188,8 +188,8 @@ def sum_boxes(srcs, src_slices, dst, dst_slices, divisor=1):
     divisions and accumulating copies would round them.  All sources share
     shape and strides.  ``dst`` may be one of them when the slices coincide
     (scaling in place).  Sources that do not sit a multiple of 16 bytes apart,
-    or more than 64 of them, are summed by accumulating box copies instead
-    (``divisor`` 1 only)."""
+    or more than 64 of them, go through the same arithmetic one source at a
+    time (divided into a temporary, added by an accumulating box copy)."""
     srcs = list(srcs)
     if not srcs:
         raise ValueError("sum_boxes: no sources")
@@ -222,15 +222,25 @@ def sum_boxes(srcs, src_slices, dst, dst_slices, divisor=1):
     box.dst = dst.data_ptr() + doff * es
     ptrs = [t.data_ptr() + soff * es for t in srcs]
     one_launch = len(srcs) <= 64 and all((p - ptrs[0]) % 16 == 0 for p in ptrs)
-    if not one_launch:
-        if divisor != 1:
-            raise ValueError("sum_boxes: this layout of the sources is summed by accumulating copies, which cannot divide")
-        for q, t in enumerate(srcs):
-            copy_box(t, src_slices, dst, dst_slices, accumulate=q > 0)
+    lib = _lib.load()
+    dt = _ADD_DTYPES[dst.dtype]
+    if one_launch:
+        rc = lib.ddl_sum_boxes(ctypes.byref(box), _lib.ptr_array(ptrs), len(srcs), es, dt, float(divisor), _stream())
+        _lib.check(rc, "ddl_sum_boxes")
         return
-    rc = _lib.load().ddl_sum_boxes(ctypes.byref(box), _lib.ptr_array(ptrs), len(srcs), es, _ADD_DTYPES[dst.dtype],
-                                   float(divisor), _stream())
+    # The same arithmetic source by source: the first one divided into dst, every other one divided into a
+    # temporary of the box's shape and added to dst by an accumulating copy.
+    rc = lib.ddl_sum_boxes(ctypes.byref(box), _lib.ptr_array(ptrs[:1]), 1, es, dt, float(divisor), _stream())
     _lib.check(rc, "ddl_sum_boxes")
+    shape = [int(box.shape[d]) for d in range(nd)]
+    whole = [slice(0, n) for n in shape]
+    for t in srcs[1:]:
+        if divisor == 1:
+            copy_box(t, src_slices, dst, dst_slices, accumulate=True)
+            continue
+        tmp = torch.empty(shape, dtype=dst.dtype, device=dst.device)
+        sum_boxes([t], src_slices, tmp, whole, divisor)
+        copy_box(tmp, whole, dst, dst_slices, accumulate=True)
 
 
 def scaled(t, divisor):

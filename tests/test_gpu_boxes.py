@@ -571,7 +571,7 @@ def test_sum_boxes_matches_step_by_step_arithmetic(ops, dtype, nsrc, divisor):
 def test_sum_boxes_in_place_and_fallbacks(ops):
     """The destination may be one of the sources (scaling a gradient in place);
     sources that are not 16 bytes apart, or more than 64 of them, go through
-    accumulating copies; what neither path can do is refused."""
+    the same arithmetic one source at a time; bad arguments are refused."""
     gen = torch.Generator().manual_seed(5)
     x = torch.randn(7, 33, generator=gen)
     full = (slice(0, 7), slice(0, 33))
@@ -585,8 +585,8 @@ def test_sum_boxes_in_place_and_fallbacks(ops):
     out = torch.empty(7, 33, device="cuda")
     ops.sum_boxes(odd, full, out, full)
     assert torch.equal(out.cpu(), _sequential_sum([t.cpu() for t in odd], 1))
-    with pytest.raises(ValueError):
-        ops.sum_boxes(odd, full, out, full, 2)
+    ops.sum_boxes(odd, full, out, full, 3)
+    assert torch.equal(out.cpu(), _sequential_sum([t.cpu() for t in odd], 3))
     many = [torch.full((4, 8), float(q), device="cuda") for q in range(70)]
     out = torch.empty(4, 8, device="cuda")
     ops.sum_boxes(many, (slice(0, 4), slice(0, 8)), out, (slice(0, 4), slice(0, 8)))
