@@ -306,7 +306,7 @@ __device__ __forceinline__ void gemm_tile(const Part& part, int tile_id, char* l
     auto k_step = [&](int cur, const char* wt, const char* xt, int ks_next, int first, int gap, int nreq, auto request) {
 #pragma unroll
         for (int q = 0; q < NMFMA; ++q) {
-            const int o = q / NI, i = q % NI;
+            const int o = q / NI, i = (o & 1) ? NI - 1 - q % NI : q % NI;   // back and forth: the inner piece stays across a change of the outer one
             const int a = kOuterX ? i : o, b = kOuterX ? o : i;
             mfma_16x16x32<F16>(acc[a][b], fa[cur][a], fb[cur][b]);
             if ((q & 1) && (q >> 1) < NREAD) read_frag(wt, xt, ks_next, fa[cur ^ 1], fb[cur ^ 1], q >> 1);
