@@ -1222,8 +1222,6 @@ def main():
             "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
                          "traffic": traffic},
         }
-        if traffic is not None:
-            results[name]["roofline"]["traffic_source"] = f"profiles/{name}_hbm_traffic_pmc.txt (not this run)"
         del step_fns, keep
         torch.cuda.empty_cache()
         if layer_fn is not None and not args.skip_layers:
@@ -1266,6 +1264,7 @@ def main():
         if "layer" in r:
             table[key]["layer_us"] = r["layer"]["us"]
     roofline = dict(head["roofline"])
+    roofline["traffic_source"] = "profiles/<workload>_hbm_traffic_pmc.txt: rocprofv3 --pmc runs of the same workloads, not this run"
     roofline["configs"] = table
     line = {
         "metric": "Repartition pack+unpack GB/s (rank 0, bf16 [8,4096,8192], P_x=[1,8,1] -> P_y=[1,1,8])"
