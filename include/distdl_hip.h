@@ -90,7 +90,10 @@ int ddl_copy_boxes(const ddl_box_t* boxes, int nbox, int elem_size,
  * src_stride shared by all sources (its src field is ignored); srcs[q] points
  * at the first element of the box in source q, all a multiple of 16 bytes
  * apart.  dst may be one of the sources (same strides) but must not overlap
- * them otherwise.  Integer dtypes take divisor 1 only.
+ * them otherwise.  Integer dtypes take divisor 1 only.  The 16-bit types are
+ * divided and added in fp32 and rounded to nearest even after every operation
+ * (a NaN stays a NaN, whatever its payload); a divisor that is a power of two
+ * is applied as a product with its exact reciprocal, which gives the same bits.
  *
  * Replaces the local reduction and re-layout of ReduceScatter,
  *   backends/mpi_numpy/functional/reduce_scatter.py:86-119 (rearrange + MPI.SUM

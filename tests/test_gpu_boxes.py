@@ -606,6 +606,69 @@ def test_sum_boxes_in_place_and_fallbacks(ops):
     assert lib.ddl_sum_boxes(box, ptrs, 1, 2, _lib.DDL_DT_F32, 1.0, None) == -1
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("divisor", [2, 8, 0.25, -4, 2.0 ** 40, 2.0 ** -40, 3, 7, 10, -6, 1e-3])
+def test_sum_boxes_divides_every_16_bit_pattern_like_true_division(ops, dtype, divisor):
+    """All 65 536 bit patterns of a 16-bit type, zeros, subnormals, infinities
+    and NaNs included, divided by powers of two (which the kernel multiplies by
+    the exact reciprocal) and by other numbers (which it divides by): the bits
+    of the quotient computed in fp32 and rounded once to the element type.  NaNs
+    are compared as NaNs: the CPU's own conversions do not agree on their bits."""
+    x = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16).view(dtype)
+    want = (x.float() / divisor).to(dtype)
+    got = ops.scaled(x.cuda(), divisor).cpu()
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(got), nan)
+    assert torch.equal(bits(got)[~nan], bits(want)[~nan])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_box_add_of_every_16_bit_pattern(ops, dtype):
+    """All 65 536 bit patterns of a 16-bit type plus a handful of partners
+    (zeros, the smallest subnormal, numbers that cancel or tie, the largest
+    finite one, infinity): the sum computed in fp32 and rounded once to nearest
+    even, through the accumulating copy and through the sum of two sources."""
+    x = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16).view(dtype)
+    info = torch.finfo(dtype)
+    partners = torch.tensor([0.0, -0.0, 1.0, -1.0, 1.0 + info.eps, 3 * info.eps / 2, info.tiny, -info.tiny * 0.5, info.max, -info.max,
+                             float("inf"), 0.3, -255.0], dtype=torch.float32).to(dtype)
+    smallest = torch.tensor([1], dtype=torch.int16).view(dtype)
+    full = (slice(0, 65536),)
+    for p in list(partners) + [smallest[0]]:
+        y = p.expand(65536).contiguous()
+        want = (x.float() + y.float()).to(dtype)
+        nan = torch.isnan(want)
+        d = y.cuda()
+        ops.copy_box(x.cuda(), full, d, full, accumulate=True)
+        got = d.cpu()
+        assert torch.equal(torch.isnan(got), nan)
+        assert torch.equal(bits(got)[~nan], bits(want)[~nan])
+        out = torch.empty(65536, dtype=dtype, device="cuda")
+        ops.sum_boxes([x.cuda(), y.cuda()], full, out, full)
+        assert torch.equal(bits(out.cpu())[~nan], bits(want)[~nan])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("divisor", [2, 0.125, -16, 2.0 ** 60, 2.0 ** -60, 3, 1e-3])
+def test_sum_boxes_divides_special_values_like_true_division(ops, dtype, divisor):
+    """Subnormal, tiny, huge and non-finite inputs and quotients in fp32 and
+    fp64: the product with the reciprocal of a power of two is the quotient
+    itself, also where it underflows or overflows."""
+    info = torch.finfo(dtype)
+    gen = torch.Generator().manual_seed(17)
+    special = torch.tensor([0.0, -0.0, info.tiny, -info.tiny, info.tiny / 8, info.tiny * 0.75, info.tiny * 1.5, info.max, -info.max,
+                            info.max / 3, info.eps, 1.0, -1.0, float("inf"), float("-inf"), float("nan"),
+                            info.smallest_normal * (1 + info.eps), 5e-324 if dtype == torch.float64 else 1.4e-45], dtype=dtype)
+    spread = (torch.randn(4096, generator=gen, dtype=torch.float64)
+              * torch.exp2(torch.randint(-140, 128, (4096,), generator=gen).double())).to(dtype)
+    x = torch.cat([special, spread])
+    want = x / divisor
+    got = ops.scaled(x.cuda(), divisor).cpu()
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(got), nan)
+    assert torch.equal(bits(got)[~nan], bits(want)[~nan])
+
+
 def test_reduce_scatter_relayout_at_config4_activation_size(ops):
     """The local half of a reduce-scatter over 8 workers at the activation
     shape of configuration 4 ([4,2048,8192] bf16, split along the features):
