@@ -521,6 +521,7 @@ struct DivOp<int64_t> {
 
 template <typename T, typename V, uint32_t MODE>
 __device__ inline V div_vector(V s, double d, double r) {
+    if constexpr (MODE == kDivNone) return s;
     constexpr int n = sizeof(V) / sizeof(T);
     if constexpr (std::is_same<T, bf16_bits>::value && sizeof(V) >= 4) {
         constexpr int words = sizeof(V) / 4;
@@ -542,6 +543,8 @@ __device__ inline V div_vector(V s, double d, double r) {
 }
 
 constexpr int kMaxSumSources = 64;
+constexpr int kSumPiecesSources = 5;        // from this many sources on, whole-tile boxes take sum_pieces_kernel
+constexpr uint32_t kXcdAddressBit = 19;     // lowest address bit that may tell the XCDs apart, see sum_pieces_kernel
 constexpr uint32_t kSumGroup = 2;   // 2: 27.6 us for eight [4,2048,1024] bf16 slabs, 1: 29.5 us, 4: 31.0 us (registers cost more wavefronts than the loads gain)
 
 struct SumArgs {
@@ -550,7 +553,7 @@ struct SumArgs {
     double divisor, reciprocal;
     uint32_t nsrc;
     uint32_t ntiles;
-    uint32_t divide;                   // kDivNone, kDivDivide or kDivReciprocal
+    uint32_t divide;                   // kDivNone, kDivDivide or kDivReciprocal (host side: which instantiation is launched)
     uint32_t pad;
 };
 
@@ -560,7 +563,7 @@ typedef const SumArgs __attribute__((address_space(4))) * SumArgsPtr;
 typedef const SumArgs* SumArgsPtr;
 #endif
 
-template <typename T, typename V, int ND>
+template <typename T, typename V, int ND, uint32_t MODE>
 __device__ inline void sum_tile(SumArgsPtr sa, uint32_t tile) {
     DevBoxPtr bx = &sa->box;
     int64_t soff[kUnroll], doff[kUnroll];
@@ -568,7 +571,6 @@ __device__ inline void sum_tile(SumArgsPtr sa, uint32_t tile) {
     tile_offsets<ND>(bx, tile, soff, doff, live);
     const char* const src = bx->src;
     const uint32_t nsrc = sa->nsrc;
-    const uint32_t divide = sa->divide;
     const double divisor = sa->divisor, reciprocal = sa->reciprocal;
     // Sources are fetched kSumGroup at a time (all their loads issued before the first addition) and added in order.
     V acc[kUnroll];
@@ -584,13 +586,8 @@ __device__ inline void sum_tile(SumArgsPtr sa, uint32_t tile) {
 #pragma unroll
         for (uint32_t g = 0; g < kSumGroup; ++g) {
             if (q0 + g >= nsrc) break;
-            if (divide == kDivReciprocal) {
 #pragma unroll
-                for (int u = 0; u < kUnroll; ++u) val[g][u] = div_vector<T, V, kDivReciprocal>(val[g][u], divisor, reciprocal);
-            } else if (divide == kDivDivide) {
-#pragma unroll
-                for (int u = 0; u < kUnroll; ++u) val[g][u] = div_vector<T, V, kDivDivide>(val[g][u], divisor, reciprocal);
-            }
+            for (int u = 0; u < kUnroll; ++u) val[g][u] = div_vector<T, V, MODE>(val[g][u], divisor, reciprocal);
             if (q0 + g == 0) {
 #pragma unroll
                 for (int u = 0; u < kUnroll; ++u) acc[u] = val[g][u];
@@ -607,19 +604,19 @@ __device__ inline void sum_tile(SumArgsPtr sa, uint32_t tile) {
         if (live[u]) __builtin_nontemporal_store(acc[u], reinterpret_cast<V*>(dst + doff[u]));
 }
 
-template <typename T, typename V>
+template <typename T, typename V, uint32_t MODE>
 __device__ inline void sum_tile_nd(SumArgsPtr sa, uint32_t tile, uint32_t nd) {
     if (nd == 0)
-        sum_tile<T, V, 0>(sa, tile);
+        sum_tile<T, V, 0, MODE>(sa, tile);
     else if (nd == 1)
-        sum_tile<T, V, 1>(sa, tile);
+        sum_tile<T, V, 1, MODE>(sa, tile);
     else if (nd == 2)
-        sum_tile<T, V, 2>(sa, tile);
+        sum_tile<T, V, 2, MODE>(sa, tile);
     else
-        sum_tile<T, V, kMaxDevDims>(sa, tile);
+        sum_tile<T, V, kMaxDevDims, MODE>(sa, tile);
 }
 
-template <typename T>
+template <typename T, uint32_t MODE>
 __global__ __launch_bounds__(kThreads) void sum_kernel(const SumArgs args_by_value) {
 #if defined(__HIP_DEVICE_COMPILE__)
     SumArgsPtr sa = (SumArgsPtr)__builtin_amdgcn_kernarg_segment_ptr();
@@ -631,15 +628,121 @@ __global__ __launch_bounds__(kThreads) void sum_kernel(const SumArgs args_by_val
     for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         // A vector holds whole elements: the host lowers the box with the element size as the narrowest vector.
         if (vlog == 4)
-            sum_tile_nd<T, u32x4>(sa, tile, nd);
+            sum_tile_nd<T, u32x4, MODE>(sa, tile, nd);
         else if (vlog == 3) {
-            if constexpr (sizeof(T) <= 8) sum_tile_nd<T, u32x2>(sa, tile, nd);
+            if constexpr (sizeof(T) <= 8) sum_tile_nd<T, u32x2, MODE>(sa, tile, nd);
         } else if (vlog == 2) {
-            if constexpr (sizeof(T) <= 4) sum_tile_nd<T, uint32_t>(sa, tile, nd);
+            if constexpr (sizeof(T) <= 4) sum_tile_nd<T, uint32_t, MODE>(sa, tile, nd);
         } else {
-            if constexpr (sizeof(T) <= 2) sum_tile_nd<T, uint16_t>(sa, tile, nd);
+            if constexpr (sizeof(T) <= 2) sum_tile_nd<T, uint16_t, MODE>(sa, tile, nd);
         }
     }
+}
+
+// The addend that leaves every partial sum as it is, bit for bit: -0.0 for the
+// floating-point types (x + -0.0 is x for every x, -0.0 included), 0 for integers.
+template <typename T, typename V>
+__device__ inline V sum_identity() {
+    constexpr int n = sizeof(V) / sizeof(T);
+    T e[n];
+    for (int i = 0; i < n; ++i) {
+        if constexpr (std::is_same<T, float>::value) e[i] = -0.0f;
+        else if constexpr (std::is_same<T, double>::value) e[i] = -0.0;
+        else if constexpr (std::is_integral<T>::value) e[i] = 0;
+        else e[i].u = 0x8000;
+    }
+    V out;
+    __builtin_memcpy(&out, e, sizeof(V));
+    return out;
+}
+
+// The same sum for many sources (five and more) over a box of whole tiles with
+// 16-byte vectors and at most one outer dimension: a workgroup takes a quarter
+// tile -- one vector per lane -- and has eight sources in flight, where
+// sum_kernel has four vectors of two.  Measured on the slab [4,2048,1024] of
+// eight [4,2048,8192] bf16 tensors (rows of 2 KiB, 16 KiB apart): 28.4 us in
+// sum_kernel's shape, 26.2 us in this one.  What the figures of a stand-alone
+// harness say about why: a workgroup that touches few rows of many tensors
+// does better than one that touches many rows of two, as long as the rows are
+// shorter than 4 KiB; from 4 KiB on the shapes are within 2 % of each other.
+//
+// Workgroups go to the eight XCDs in turn, so the three low bits of the
+// workgroup number name the XCD; which address bits they end up as is the
+// second thing that matters.  With one row of 2 KiB per 128 threads the same
+// sum takes 25.2 us when those bits are address bits 19-21 or higher, 25.9-26.4
+// at 14-16 and 15-17, 32.6 at 16-18, 28.2 at 17-19 and 18-20, and 29.9 when
+// every XCD has a contiguous eighth: an XCD whose requests all agree in bits
+// 16-18 is served by a part of the memory system only.  The host therefore
+// moves the three bits up (turn_log) until the sources' addresses differ at
+// bit 19 between neighbouring workgroups, for as many workgroups as fill whole
+// groups of 8 << turn_log.
+//
+// The geometry arrives as scalar arguments -- the first sixteen dwords of the
+// argument segment are in scalar registers when a wavefront starts -- and the
+// table of the sources follows as a structure read with one wide scalar load
+// per eight sources: a workgroup that lives for one round of loads cannot
+// afford the five rounds of dependent scalar loads a structure read field by
+// field costs it.
+struct SumSources {
+    double divisor, reciprocal;
+    int64_t delta[kMaxSumSources];     // bytes from source 0 to source q, padded to a multiple of eight with the last source
+};
+constexpr int kSumPiecesScalarBytes = 64;   // what precedes the SumSources argument of sum_pieces_kernel
+
+#if defined(__HIP_DEVICE_COMPILE__)
+typedef const SumSources __attribute__((address_space(4))) * SumSourcesPtr;
+typedef const char __attribute__((address_space(4))) * KernargBytes;
+#else
+typedef const SumSources* SumSourcesPtr;
+#endif
+
+template <typename T, uint32_t MODE>
+__global__ __launch_bounds__(kThreads) void sum_pieces_kernel(const char* src0, char* dst0, int64_t srow, int64_t drow, uint32_t col_tiles,
+                                                              uint32_t ct_mul, uint32_t shifts, uint32_t turn_items, uint32_t nsrc,
+                                                              uint32_t unused0, uint32_t unused1, uint32_t unused2,
+                                                              const SumSources sources_by_value) {
+    // shifts: tc_log, the shift of the division by col_tiles, turn_log -- a byte each (fourteen dwords are preloaded, not sixteen)
+    const uint32_t tc_log = shifts & 0xFFu, ct_shr = (shifts >> 8) & 0xFFu, turn_log = shifts >> 16;
+#if defined(__HIP_DEVICE_COMPILE__)
+    SumSourcesPtr ss = (SumSourcesPtr)((KernargBytes)__builtin_amdgcn_kernarg_segment_ptr() + kSumPiecesScalarBytes);
+#else
+    SumSourcesPtr ss = &sources_by_value;
+#endif
+    typedef u32x4 V;
+    uint32_t item = blockIdx.x;
+    if (item < turn_items) {
+        const uint32_t low = item & 7u, rest = item >> 3;
+        item = ((rest >> turn_log) << (turn_log + 3)) | (low << turn_log) | (rest & ((1u << turn_log) - 1u));
+    }
+    const uint32_t tile = item / kUnroll, part = item % kUnroll;
+    const uint32_t row_tile = col_tiles == 1 ? tile : (__umulhi(tile, ct_mul) >> ct_shr);
+    const uint32_t col_tile = tile - row_tile * col_tiles;
+    const uint32_t v = threadIdx.x + part * kThreads;              // vector number inside the tile
+    const uint32_t col = (col_tile << tc_log) + (v & ((1u << tc_log) - 1u));
+    const uint32_t r = (row_tile << (kTileLog - tc_log)) + (v >> tc_log);
+    const char* const src = src0 + static_cast<int64_t>(col) * 16 + static_cast<int64_t>(r) * srow;
+    char* const dst = dst0 + static_cast<int64_t>(col) * 16 + static_cast<int64_t>(r) * drow;
+    // Eight sources at a time, all requested before the first addition.  Beyond the last source the table repeats it;
+    // what is fetched there is replaced by the element that changes no sum (-0.0, integer 0) rather than skipped, so
+    // that no load hangs on a condition and the compiler keeps the eight together.
+    constexpr uint32_t G = 8;
+    const V nothing = sum_identity<T, V>();
+    V acc = nothing;
+    for (uint32_t q0 = 0; q0 < nsrc; q0 += G) {
+        int64_t delta[G];
+#pragma unroll
+        for (uint32_t g = 0; g < G; ++g) delta[g] = ss->delta[q0 + g];
+        V val[G];
+#pragma unroll
+        for (uint32_t g = 0; g < G; ++g) val[g] = __builtin_nontemporal_load(reinterpret_cast<const V*>(src + delta[g]));
+#pragma unroll
+        for (uint32_t g = 0; g < G; ++g) {
+            const V quotient = div_vector<T, V, MODE>(val[g], ss->divisor, ss->reciprocal);
+            const V sum = add_vectors<T, V>(acc, q0 + g < nsrc ? quotient : nothing);
+            acc = q0 + g == 0 ? quotient : sum;              // the first source as it is: -0.0 + 0.0 would lose its sign
+        }
+    }
+    __builtin_nontemporal_store(acc, reinterpret_cast<V*>(dst));
 }
 
 // ------------------------------------------------------------------ host --
@@ -976,8 +1079,43 @@ int launch_sum(const std::vector<DevBox>& pieces, const void* const* srcs, int n
         const uint64_t tr = kTileVecs >> db.tc_log;
         const uint64_t tiles = static_cast<uint64_t>(db.col_tiles) * ((db.rows + tr - 1) / tr);
         sa.ntiles = static_cast<uint32_t>(tiles);
+        const bool whole_tiles = db.cols % (1u << db.tc_log) == 0 && db.rows % tr == 0;
+        if (nsrc >= kSumPiecesSources && db.vlog == 4 && db.nd <= 1 && db.css == 16 && db.cds == 16 && whole_tiles &&
+            tiles * kUnroll <= 0x7FFFFFFFull) {
+            const uint32_t items = static_cast<uint32_t>(tiles * kUnroll);
+            // Bytes between the sources of neighbouring workgroups: a quarter tile further down the rows, or along the row.
+            const uint64_t rows_apart = kThreads >> db.tc_log;
+            const uint64_t apart = rows_apart >= 1 && db.nd == 1 ? rows_apart * static_cast<uint64_t>(std::llabs(db.dim[0].ss)) : kThreads * 16;
+            uint32_t apart_log = 0;
+            while ((2ull << apart_log) <= apart) ++apart_log;
+            uint32_t turn_log = apart_log < kXcdAddressBit ? kXcdAddressBit - apart_log : 0;
+            while (turn_log > 0 && (8u << turn_log) > items) --turn_log;
+            const uint32_t turn_items = items - items % (8u << turn_log);
+            SumSources ss{};
+            ss.divisor = sa.divisor, ss.reciprocal = sa.reciprocal;
+            for (int q = 0; q < kMaxSumSources; ++q) ss.delta[q] = sa.delta[q < nsrc ? q : nsrc - 1];
+            const int64_t srow = db.nd == 1 ? db.dim[0].ss : 0, drow = db.nd == 1 ? db.dim[0].ds : 0;
+#define DDL_LAUNCH_SUM_PIECES(MODE)                                                                                              \
+    hipLaunchKernelGGL((sum_pieces_kernel<T, MODE>), dim3(items), dim3(kThreads), 0, stream, db.src, db.dst, srow, drow,            \
+                       db.col_tiles, db.ct_mul, db.tc_log | (db.ct_shr << 8) | (turn_log << 16), turn_items,                      \
+                       static_cast<uint32_t>(nsrc), 0u, 0u, 0u, ss)
+            if (sa.divide == kDivNone)
+                DDL_LAUNCH_SUM_PIECES(kDivNone);
+            else if (sa.divide == kDivReciprocal)
+                DDL_LAUNCH_SUM_PIECES(kDivReciprocal);
+            else
+                DDL_LAUNCH_SUM_PIECES(kDivDivide);
+#undef DDL_LAUNCH_SUM_PIECES
+            if (int rc = check_launch("sum_pieces_kernel")) return rc;
+            continue;
+        }
         const uint32_t blocks = tiles < kPersistentBlocks ? static_cast<uint32_t>(tiles) : kPersistentBlocks;
-        hipLaunchKernelGGL((sum_kernel<T>), dim3(blocks), dim3(kThreads), 0, stream, sa);
+        if (sa.divide == kDivNone)
+            hipLaunchKernelGGL((sum_kernel<T, kDivNone>), dim3(blocks), dim3(kThreads), 0, stream, sa);
+        else if (sa.divide == kDivReciprocal)
+            hipLaunchKernelGGL((sum_kernel<T, kDivReciprocal>), dim3(blocks), dim3(kThreads), 0, stream, sa);
+        else
+            hipLaunchKernelGGL((sum_kernel<T, kDivDivide>), dim3(blocks), dim3(kThreads), 0, stream, sa);
         if (int rc = check_launch("sum_kernel")) return rc;
     }
     return 0;

@@ -568,6 +568,42 @@ def test_sum_boxes_matches_step_by_step_arithmetic(ops, dtype, nsrc, divisor):
     assert torch.equal(bits(d.cpu()), bits(want))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.int32])
+@pytest.mark.parametrize("nsrc", [5, 8, 13])
+@pytest.mark.parametrize("rows,row_elems,pitch_elems", [
+    (64, 128, 128 * 3),        # rows of 256 / 512 B: eight or four rows per quarter tile
+    (24, 1024, 8192),          # the re-layout's rows (2 KiB in bf16), 8 rows per tile
+    (6, 4096, 4096 * 2),       # rows longer than a quarter tile
+    (1, 16384 * 3, 16384 * 3), # one contiguous run
+])
+def test_sum_boxes_of_many_sources_over_whole_tiles(ops, dtype, nsrc, rows, row_elems, pitch_elems):
+    """Five and more sources over boxes made of whole tiles take the kernel
+    that has eight sources in flight per quarter tile and reorders its
+    workgroups: the same step-by-step arithmetic, also divided, also into one of
+    the sources, on row lengths on either side of a quarter tile."""
+    gen = torch.Generator().manual_seed(nsrc * 7 + rows)
+    es = torch.empty((), dtype=dtype).element_size()
+    row_elems, pitch_elems = row_elems * 4 // es, pitch_elems * 4 // es
+    if dtype.is_floating_point:
+        srcs = [(torch.randn(rows, pitch_elems, generator=gen) * 3).to(dtype) for _ in range(nsrc)]
+    else:
+        srcs = [torch.randint(-2 ** 30, 2 ** 30, (rows, pitch_elems), generator=gen).to(dtype) for _ in range(nsrc)]
+    first = pitch_elems - row_elems if pitch_elems > row_elems else 0
+    box = (slice(0, rows), slice(first, first + row_elems))
+    full = (slice(0, rows), slice(0, row_elems))
+    for divisor in ((1, 4, 3) if dtype.is_floating_point else (1,)):
+        want = _sequential_sum([t[box] for t in srcs], divisor)
+        out = torch.zeros(rows, row_elems, dtype=dtype, device="cuda")
+        dev = [t.cuda() for t in srcs]
+        ops.sum_boxes(dev, box, out, full, divisor)
+        assert torch.equal(bits(out.cpu()), bits(want))
+        ops.sum_boxes(dev, box, dev[2], box, divisor)                  # into the third source
+        assert torch.equal(bits(dev[2].cpu()[box]), bits(want))
+        untouched = torch.ones(rows, pitch_elems, dtype=torch.bool)
+        untouched[box] = False
+        assert torch.equal(bits(dev[2].cpu())[untouched], bits(srcs[2])[untouched])
+
+
 def test_sum_boxes_in_place_and_fallbacks(ops):
     """The destination may be one of the sources (scaling a gradient in place);
     sources that are not 16 bytes apart, or more than 64 of them, go through
