@@ -544,7 +544,6 @@ __device__ inline V div_vector(V s, double d, double r) {
 
 constexpr int kMaxSumSources = 64;
 constexpr int kSumPiecesSources = 5;        // from this many sources on, whole-tile boxes take sum_pieces_kernel
-constexpr uint32_t kXcdAddressBit = 19;     // lowest address bit that may tell the XCDs apart, see sum_pieces_kernel
 constexpr uint32_t kSumGroup = 2;   // 2: 27.6 us for eight [4,2048,1024] bf16 slabs, 1: 29.5 us, 4: 31.0 us (registers cost more wavefronts than the loads gain)
 
 struct SumArgs {
@@ -667,15 +666,14 @@ __device__ inline V sum_identity() {
 // shorter than 4 KiB; from 4 KiB on the shapes are within 2 % of each other.
 //
 // Workgroups go to the eight XCDs in turn, so the three low bits of the
-// workgroup number name the XCD; which address bits they end up as is the
-// second thing that matters.  With one row of 2 KiB per 128 threads the same
-// sum takes 25.2 us when those bits are address bits 19-21 or higher, 25.9-26.4
-// at 14-16 and 15-17, 32.6 at 16-18, 28.2 at 17-19 and 18-20, and 29.9 when
-// every XCD has a contiguous eighth: an XCD whose requests all agree in bits
-// 16-18 is served by a part of the memory system only.  The host therefore
-// moves the three bits up (turn_log) until the sources' addresses differ at
-// bit 19 between neighbouring workgroups, for as many workgroups as fill whole
-// groups of 8 << turn_log.
+// workgroup number name the XCD, and which address bits they coincide with
+// matters too: in the harness, with one row of 2 KiB per 128 threads, the sum
+// takes 25.9-26.4 us when they are address bits 14-16 or 15-17 (the natural
+// order of quarter tiles here), 32.6 at 16-18, 28.2 at 17-19 (whole tiles of
+// eight such rows: sum_kernel's order) and 18-20, 29.9 when every XCD has a
+// contiguous eighth.  Orders that move them to bit 19 and above measured
+// 25.2 us in one process and 26.5-29 us in the next -- above the page size the
+// bits that matter are physical -- so the natural order stays.
 //
 // The geometry arrives as scalar arguments -- the first sixteen dwords of the
 // argument segment are in scalar registers when a wavefront starts -- and the
@@ -698,23 +696,16 @@ typedef const SumSources* SumSourcesPtr;
 
 template <typename T, uint32_t MODE>
 __global__ __launch_bounds__(kThreads) void sum_pieces_kernel(const char* src0, char* dst0, int64_t srow, int64_t drow, uint32_t col_tiles,
-                                                              uint32_t ct_mul, uint32_t shifts, uint32_t turn_items, uint32_t nsrc,
+                                                              uint32_t ct_mul, uint32_t ct_shr, uint32_t tc_log, uint32_t nsrc,
                                                               uint32_t unused0, uint32_t unused1, uint32_t unused2,
                                                               const SumSources sources_by_value) {
-    // shifts: tc_log, the shift of the division by col_tiles, turn_log -- a byte each (fourteen dwords are preloaded, not sixteen)
-    const uint32_t tc_log = shifts & 0xFFu, ct_shr = (shifts >> 8) & 0xFFu, turn_log = shifts >> 16;
 #if defined(__HIP_DEVICE_COMPILE__)
     SumSourcesPtr ss = (SumSourcesPtr)((KernargBytes)__builtin_amdgcn_kernarg_segment_ptr() + kSumPiecesScalarBytes);
 #else
     SumSourcesPtr ss = &sources_by_value;
 #endif
     typedef u32x4 V;
-    uint32_t item = blockIdx.x;
-    if (item < turn_items) {
-        const uint32_t low = item & 7u, rest = item >> 3;
-        item = ((rest >> turn_log) << (turn_log + 3)) | (low << turn_log) | (rest & ((1u << turn_log) - 1u));
-    }
-    const uint32_t tile = item / kUnroll, part = item % kUnroll;
+    const uint32_t tile = blockIdx.x / kUnroll, part = blockIdx.x % kUnroll;
     const uint32_t row_tile = col_tiles == 1 ? tile : (__umulhi(tile, ct_mul) >> ct_shr);
     const uint32_t col_tile = tile - row_tile * col_tiles;
     const uint32_t v = threadIdx.x + part * kThreads;              // vector number inside the tile
@@ -1083,22 +1074,13 @@ int launch_sum(const std::vector<DevBox>& pieces, const void* const* srcs, int n
         if (nsrc >= kSumPiecesSources && db.vlog == 4 && db.nd <= 1 && db.css == 16 && db.cds == 16 && whole_tiles &&
             tiles * kUnroll <= 0x7FFFFFFFull) {
             const uint32_t items = static_cast<uint32_t>(tiles * kUnroll);
-            // Bytes between the sources of neighbouring workgroups: a quarter tile further down the rows, or along the row.
-            const uint64_t rows_apart = kThreads >> db.tc_log;
-            const uint64_t apart = rows_apart >= 1 && db.nd == 1 ? rows_apart * static_cast<uint64_t>(std::llabs(db.dim[0].ss)) : kThreads * 16;
-            uint32_t apart_log = 0;
-            while ((2ull << apart_log) <= apart) ++apart_log;
-            uint32_t turn_log = apart_log < kXcdAddressBit ? kXcdAddressBit - apart_log : 0;
-            while (turn_log > 0 && (8u << turn_log) > items) --turn_log;
-            const uint32_t turn_items = items - items % (8u << turn_log);
             SumSources ss{};
             ss.divisor = sa.divisor, ss.reciprocal = sa.reciprocal;
             for (int q = 0; q < kMaxSumSources; ++q) ss.delta[q] = sa.delta[q < nsrc ? q : nsrc - 1];
             const int64_t srow = db.nd == 1 ? db.dim[0].ss : 0, drow = db.nd == 1 ? db.dim[0].ds : 0;
 #define DDL_LAUNCH_SUM_PIECES(MODE)                                                                                              \
     hipLaunchKernelGGL((sum_pieces_kernel<T, MODE>), dim3(items), dim3(kThreads), 0, stream, db.src, db.dst, srow, drow,            \
-                       db.col_tiles, db.ct_mul, db.tc_log | (db.ct_shr << 8) | (turn_log << 16), turn_items,                      \
-                       static_cast<uint32_t>(nsrc), 0u, 0u, 0u, ss)
+                       db.col_tiles, db.ct_mul, db.ct_shr, db.tc_log, static_cast<uint32_t>(nsrc), 0u, 0u, 0u, ss)
             if (sa.divide == kDivNone)
                 DDL_LAUNCH_SUM_PIECES(kDivNone);
             else if (sa.divide == kDivReciprocal)
