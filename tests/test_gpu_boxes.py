@@ -568,7 +568,7 @@ def test_sum_boxes_matches_step_by_step_arithmetic(ops, dtype, nsrc, divisor):
     assert torch.equal(bits(d.cpu()), bits(want))
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.int32])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16, torch.float16, torch.int32, torch.int64])
 @pytest.mark.parametrize("nsrc", [5, 8, 13])
 @pytest.mark.parametrize("rows,row_elems,pitch_elems", [
     (64, 128, 128 * 3),        # rows of 256 / 512 B: eight or four rows per quarter tile
@@ -578,12 +578,12 @@ def test_sum_boxes_matches_step_by_step_arithmetic(ops, dtype, nsrc, divisor):
 ])
 def test_sum_boxes_of_many_sources_over_whole_tiles(ops, dtype, nsrc, rows, row_elems, pitch_elems):
     """Five and more sources over boxes made of whole tiles take the kernel
-    that has eight sources in flight per quarter tile and reorders its
-    workgroups: the same step-by-step arithmetic, also divided, also into one of
-    the sources, on row lengths on either side of a quarter tile."""
+    that has eight sources in flight per quarter tile: the same step-by-step
+    arithmetic, also divided, also into one of the sources, on row lengths on
+    either side of a quarter tile."""
     gen = torch.Generator().manual_seed(nsrc * 7 + rows)
     es = torch.empty((), dtype=dtype).element_size()
-    row_elems, pitch_elems = row_elems * 4 // es, pitch_elems * 4 // es
+    row_elems, pitch_elems = max(row_elems * 4 // es, 16 // es), pitch_elems * 4 // es
     if dtype.is_floating_point:
         srcs = [(torch.randn(rows, pitch_elems, generator=gen) * 3).to(dtype) for _ in range(nsrc)]
     else:
