@@ -1758,3 +1758,29 @@ def test_linear_reduce_scatter_layer_matches_torch(ops, P, x_shape, c_out, use_b
         if db is not None:
             assert r == 0 and np.allclose(db.numpy().reshape(-1), br.grad.numpy(), rtol=1e-5, atol=1e-4)
     assert seen_w == M
+
+
+def test_empty_inputs_give_empty_or_zero_outputs(ops):
+    """No rows, no tokens: every entry point returns without a launch of size
+    zero; gradients that are sums over nothing are zeros."""
+    dev = "cuda"
+    x = torch.empty(0, 256, device=dev)
+    g, b = torch.ones(256, device=dev), torch.zeros(256, device=dev)
+    assert ops.layer_norm(x, g, b, 1e-5).shape == (0, 256)
+    stats = ops.ln_partial_stats(x)
+    assert stats.shape == (0, 2)
+    assert ops.ln_normalize_affine(x, stats.unsqueeze(0), [256], g, b, 1e-5).shape == (0, 256)
+    mean = rstd = torch.empty(0, device=dev)
+    dx, dg, db = ops.ln_backward_one_pass(x, x, mean, rstd, g, 1.0 / 256)
+    assert dx.shape == (0, 256) and float(dg.abs().max()) == 0 and float(db.abs().max()) == 0
+    table = torch.randn(16, 64, device=dev).to(torch.bfloat16)
+    ids = torch.empty(0, dtype=torch.int64, device=dev)
+    assert ops.embedding_gather(table, ids, 0, 16).shape == (0, 64)
+    dw = ops.embedding_backward(torch.empty(0, 64, dtype=torch.bfloat16, device=dev), ids, 0, 16)
+    assert dw.shape == (16, 64) and float(dw.float().abs().max()) == 0
+    w = torch.randn(24, 64, device=dev).to(torch.bfloat16)
+    bias = torch.randn(24, device=dev).to(torch.bfloat16)
+    assert ops.linear(torch.empty(0, 64, dtype=torch.bfloat16, device=dev), w, bias).shape == (0, 24)
+    dx, dw, db = ops.linear_backward(torch.empty(0, 64, dtype=torch.bfloat16, device=dev), w,
+                                     torch.empty(0, 24, dtype=torch.bfloat16, device=dev))
+    assert dx.shape == (0, 64) and float(dw.float().abs().max()) == 0 and float(db.float().abs().max()) == 0
