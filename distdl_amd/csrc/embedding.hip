@@ -18,16 +18,22 @@ constexpr int kWave = 64;
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr int kInFlight = 8;
+// The gather runs two tokens per workgroup.  Workgroups go to the eight XCDs in
+// turn, so a workgroup's bytes decide which address bits an XCD's stores agree
+// in: with rows of 8 KiB, four tokens per workgroup (bits 15-17) take 200.0 us on
+// configuration 3, two (14-16) 199.0, one 198.0 -- and eight (16-18) 210.
+constexpr int kGatherBlock = 128;
+constexpr int kGatherWaves = kGatherBlock / kWave;
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 template <typename V, typename IdT>
-__global__ __launch_bounds__(kBlock) void gather_rows(const char* __restrict__ weight, int64_t ldw_bytes, int64_t nvec,
+__global__ __launch_bounds__(kGatherBlock) void gather_rows(const char* __restrict__ weight, int64_t ldw_bytes, int64_t nvec,
                                                       const IdT* __restrict__ ids, int64_t n_ids, int64_t lo, int64_t hi,
                                                       char* __restrict__ out) {
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t t = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + threadIdx.x / kWave;
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kGatherWaves + threadIdx.x / kWave;
     if (t >= n_ids) return;
     const int64_t id = static_cast<int64_t>(ids[t]);
     const bool hit = id >= lo && id < hi;
@@ -58,14 +64,14 @@ template <typename V>
 int launch_gather(const void* w, int64_t ldw_bytes, int64_t row_bytes, const void* ids, int i64, int64_t n, int64_t lo,
                   int64_t hi, void* out, hipStream_t s) {
     const int64_t nvec = row_bytes / static_cast<int64_t>(sizeof(V));
-    const int64_t blocks = (n + kWavesPerBlock - 1) / kWavesPerBlock;
-    if (blocks > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "embedding gather: more than 2^33 ids in one call");
+    const int64_t blocks = (n + kGatherWaves - 1) / kGatherWaves;
+    if (blocks > 0x7FFFFFFFll) return fail(DDL_E_UNSUPP, "embedding gather: more than 2^32 ids in one call");
     if (i64)
-        hipLaunchKernelGGL((gather_rows<V, int64_t>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, s,
+        hipLaunchKernelGGL((gather_rows<V, int64_t>), dim3(static_cast<uint32_t>(blocks)), dim3(kGatherBlock), 0, s,
                            static_cast<const char*>(w), ldw_bytes, nvec, static_cast<const int64_t*>(ids), n, lo, hi,
                            static_cast<char*>(out));
     else
-        hipLaunchKernelGGL((gather_rows<V, int32_t>), dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, s,
+        hipLaunchKernelGGL((gather_rows<V, int32_t>), dim3(static_cast<uint32_t>(blocks)), dim3(kGatherBlock), 0, s,
                            static_cast<const char*>(w), ldw_bytes, nvec, static_cast<const int32_t*>(ids), n, lo, hi,
                            static_cast<char*>(out));
     return check_launch("gather_rows");
