@@ -14,6 +14,7 @@ from oracle import halo as o_halo
 from oracle import layernorm as o_ln
 from oracle import linear as o_lin
 from oracle import partition_math as pm
+from oracle import relayout as o_rl
 from oracle import repartition as o_rep
 
 
@@ -456,3 +457,89 @@ def test_embedding_renorm_oracle_matches_torch(norm_type):
     assert np.allclose(part[[4, 10]], want_table.numpy()[[9, 15]], rtol=1e-12, atol=1e-12)
     rest = [r for r in range(15) if r not in (4, 10)]
     assert np.array_equal(part[rest], table.numpy()[5:20][rest])
+
+
+# ------------------------------------------- all-gather / reduce-scatter re-layouts --
+
+RELAYOUT_CASES = [((3, 10), 1, 4), ((7, 2, 5), 0, 3), ((2, 9, 4), 1, 2), ((2, 3, 8), 2, 4), ((5,), 0, 5), ((4, 6), 0, 6)]
+
+
+def test_relayout_shard_extents_known_answers(golden):
+    """The split the re-layouts assume is the balanced split of the reference's
+    own known answers (10 over 4 -> 3,3,2,2; 10 over 3 -> 4,3,3)."""
+    assert o_rl.shard_extents(10, 4) == [3, 3, 2, 2]
+    assert o_rl.shard_extents(10, 3) == [4, 3, 3]
+    for n, P in ((10, 4), (7, 3), (8, 8), (5, 6)):
+        assert o_rl.shard_extents(n, P) == [pm.subshape_1d(P, i, n) for i in range(P)]
+
+
+@pytest.mark.parametrize("shape,axis,P", RELAYOUT_CASES)
+def test_all_gather_oracle_closed_form_and_brute_force(shape, axis, P):
+    """A gather of the balanced split of x is x; and element by element: the
+    element j of the gathered axis comes from the worker whose range holds j."""
+    rng = np.random.default_rng(sum(shape) * 7 + axis + P)
+    x = rng.standard_normal(shape).astype(np.float32)
+    extents = o_rl.shard_extents(shape[axis], P)
+    starts = np.concatenate([[0], np.cumsum(extents)])
+    parts = [np.take(x, range(starts[r], starts[r + 1]), axis=axis) for r in range(P)]
+    got = o_rl.all_gather(parts, axis)
+    assert np.array_equal(got, x)
+    marked = [np.full(p.shape, 10 * r, dtype=np.int64) + np.arange(p.shape[axis]).reshape(
+        [-1 if d == axis else 1 for d in range(p.ndim)]) for r, p in enumerate(parts)]
+    tagged = o_rl.all_gather(marked, axis)
+    for j in range(shape[axis]):
+        r = int(np.searchsorted(starts, j, side="right") - 1)
+        assert np.all(np.take(tagged, j, axis=axis) == 10 * r + (j - starts[r]))
+    with pytest.raises(ValueError):
+        o_rl.all_gather(parts[::-1] if extents != extents[::-1] else [parts[0][..., :0]] + parts[1:], axis)
+
+
+@pytest.mark.parametrize("shape,axis,P", RELAYOUT_CASES)
+def test_reduce_scatter_oracle_closed_form_and_brute_force(shape, axis, P):
+    """Worker r ends with slab r of the element-wise sum; P copies of x give P
+    times the split of x; written out element by element on integers."""
+    rng = np.random.default_rng(sum(shape) * 11 + axis + P)
+    fulls = [rng.integers(-5, 6, size=shape).astype(np.int64) for _ in range(P)]
+    extents = o_rl.shard_extents(shape[axis], P)
+    starts = np.concatenate([[0], np.cumsum(extents)])
+    got = o_rl.reduce_scatter(fulls, axis)
+    total = np.zeros(shape, dtype=np.int64)
+    for idx in np.ndindex(*shape):
+        total[idx] = sum(int(f[idx]) for f in fulls)
+    for r in range(P):
+        want = np.take(total, range(starts[r], starts[r + 1]), axis=axis)
+        assert got[r].shape == want.shape and np.array_equal(got[r], want)
+    x = rng.standard_normal(shape).astype(np.float32)
+    same = o_rl.reduce_scatter([x] * P, axis)
+    if P & (P - 1) == 0:                                   # a power of two: the repeated additions are exact
+        for r in range(P):
+            assert np.array_equal(same[r], P * np.take(x, range(starts[r], starts[r + 1]), axis=axis))
+
+
+@pytest.mark.parametrize("shape,axis,P", RELAYOUT_CASES)
+def test_relayout_oracle_adjoint_identity(shape, axis, P):
+    """<A x, y> = <x, A* y> over all workers, exactly (integers), for the
+    gather with its reduce-scatter adjoint and the other way round; with
+    scale_backward the adjoint is divided by it."""
+    rng = np.random.default_rng(sum(shape) * 13 + axis + P)
+    extents = o_rl.shard_extents(shape[axis], P)
+
+    def shard_like(r):
+        s = list(shape)
+        s[axis] = extents[r]
+        return rng.integers(-4, 5, size=s).astype(np.int64)
+
+    xs = [shard_like(r) for r in range(P)]
+    ys = [rng.integers(-4, 5, size=shape).astype(np.int64) for _ in range(P)]
+    Ax = o_rl.all_gather(xs, axis)                         # every worker holds Ax
+    lhs = sum(int(np.sum(Ax * y)) for y in ys)
+    Aty = o_rl.all_gather_adjoint(ys, axis)
+    assert lhs == sum(int(np.sum(x * g)) for x, g in zip(xs, Aty))
+    Bf = o_rl.reduce_scatter(ys, axis)
+    gs = [shard_like(r) for r in range(P)]
+    lhs = sum(int(np.sum(b * g)) for b, g in zip(Bf, gs))
+    Btg = o_rl.reduce_scatter_adjoint(gs, axis)
+    assert lhs == sum(int(np.sum(y * t)) for y, t in zip(ys, Btg))
+    halves = o_rl.all_gather_adjoint([y.astype(np.float64) for y in ys], axis, scale_backward=2)
+    for h, g in zip(halves, Aty):
+        assert np.array_equal(h, g / 2)
