@@ -494,9 +494,11 @@ def test_all_gather_and_reduce_scatter_layers(P, shape, axis, dtype):
         fin = torch.from_numpy(fulls[r]).to(dtype).cuda().requires_grad_(True)
         z = ReduceScatter(P_x, axes_reduce_scatter=(axis,))(fin)
         z.backward(torch.from_numpy(dzs[r]).to(dtype).cuda())
+        xs = torch.from_numpy(shards[r]).to(dtype).cuda().requires_grad_(True)
+        AllGather(P_x, axes_all_gather=(axis,), scale_backward=4)(xs).backward(torch.from_numpy(dys[r]).to(dtype).cuda())
         torch.cuda.synchronize()
         return (y.detach().float().cpu().numpy(), xin.grad.float().cpu().numpy(),
-                z.detach().float().cpu().numpy(), fin.grad.float().cpu().numpy())
+                z.detach().float().cpu().numpy(), fin.grad.float().cpu().numpy(), xs.grad.float().cpu().numpy())
 
     outs = SimWorld(n).run(body)
     want_dx = o_rep.scatter(sum(dys), P)
@@ -507,7 +509,9 @@ def test_all_gather_and_reduce_scatter_layers(P, shape, axis, dtype):
     o_dx = o_rl.all_gather_adjoint(dys, axis)
     o_z = o_rl.reduce_scatter(fulls, axis)
     o_dfull = o_rl.reduce_scatter_adjoint(dzs, axis)
-    for r, (y, dx, z, dfull) in enumerate(outs):
+    o_dx_scaled = o_rl.all_gather_adjoint(dys, axis, scale_backward=4)      # quarters of small integers: exact in bf16 too
+    for r, (y, dx, z, dfull, dx_scaled) in enumerate(outs):
+        assert np.array_equal(dx_scaled, o_dx_scaled[r])
         assert np.array_equal(y, x) and np.array_equal(y, o_y)
         assert np.array_equal(dx, want_dx[r]) and np.array_equal(dx, o_dx[r])
         assert np.array_equal(z, want_z[r]) and np.array_equal(z, o_z[r])
