@@ -1032,6 +1032,34 @@ def build_reduce_scatter_relayout(torch, lib, _lib, nsets):
     return steps, keep, 9 * 4 * 2048 * 1024 * 2
 
 
+def cpu_all_gather_relayout(budget_s=3.0):
+    """The oracle's restatement of the reference's gather + rearrange on the
+    eight pieces of the workload, bf16 moved as int16 as the reference moves it."""
+    import numpy as np
+    from oracle import relayout as o_rl
+    rng = np.random.default_rng(8004)
+    parts = [rng.integers(-2 ** 15, 2 ** 15, size=(4, 2048, 1024), dtype=np.int16) for _ in range(8)]
+    n, dt = timed_cpu(lambda: o_rl.all_gather(parts, 2), budget_s)
+    return {"value": 2 * 4 * 2048 * 8192 * 2 * n / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{n} gathers of eight [4,2048,1024] int16 pieces into [4,2048,8192] (np.stack, np.concatenate), {dt:.1f} s"}
+
+
+def cpu_reduce_scatter_relayout(budget_s=3.0):
+    """The oracle's reduce-scatter over all eight workers on a sixteenth of the
+    rows, in float32 (NumPy has no bfloat16; the reference would add the int16
+    views): eight slabs of the sum of eight tensors, i.e. eight workers' shares
+    per run, counted as such."""
+    import numpy as np
+    from oracle import relayout as o_rl
+    rng = np.random.default_rng(8104)
+    fulls = [rng.standard_normal((4, 128, 8192), dtype=np.float32) for _ in range(8)]
+    n, dt = timed_cpu(lambda: o_rl.reduce_scatter(fulls, 2), budget_s)
+    work = 8 * 9 * 4 * 128 * 1024 * 4            # per worker: eight slabs read, one written
+    return {"value": work * n / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{n} reduce-scatters of eight [4,128,8192] float32 tensors over 8 simulated workers (split, pad-free "
+                      f"flatten, rank-order sum), {dt:.1f} s"}
+
+
 # ----------------------------------------------------------------------------
 # measurement aids
 # ----------------------------------------------------------------------------
@@ -1123,8 +1151,8 @@ WORKLOADS = {
     "halo_interior": (build_halo_interior, 4, 1, "hbm", None, None, None, None),
     "halo_slabs": (build_halo_slabs, 8, 6, "hbm", None, None, None, None),
     "halo_slabs_interior": (build_halo_slabs_interior, 8, 6, "hbm", None, None, None, None),
-    "all_gather_relayout": (build_all_gather_relayout, 3, 1, "hbm", "sum", None, None, None),
-    "reduce_scatter_relayout": (build_reduce_scatter_relayout, 2, 1, "hbm", "sum", None, None, None),
+    "all_gather_relayout": (build_all_gather_relayout, 3, 1, "hbm", "sum", None, cpu_all_gather_relayout, None),
+    "reduce_scatter_relayout": (build_reduce_scatter_relayout, 2, 1, "hbm", "sum", None, cpu_reduce_scatter_relayout, None),
     "layernorm_bwd": (build_layernorm_bwd, 32, 2, "hbm", None, None, None, None),
     "layernorm_bwd_one_pass": (_build_layernorm_bwd_one_pass(16 * 512, 256, 4), 32, 2, "hbm", None, None, None, None),
     "layernorm_local_bwd": (_build_layernorm_bwd_one_pass(16 * 512, 1024, 1), 8, 2, "hbm", None, None, None, None),
@@ -1281,7 +1309,8 @@ def main():
     }
     if "cpu_baseline" in head:
         cpu = dict(head["cpu_baseline"])
-        cpu["configs"] = {f"cfg{r['baseline_config']}_{name}": {k: r["cpu_baseline"][k] for k in ("value", "unit", "cores")}
+        cpu["configs"] = {(f"cfg{r['baseline_config']}_{name}" if r["baseline_config"] else name):
+                          {k: r["cpu_baseline"][k] for k in ("value", "unit", "cores")}
                           for name, r in results.items() if "cpu_baseline" in r}
         line["cpu_baseline"] = cpu
     if not args.skip_cpu:
