@@ -245,7 +245,23 @@ __device__ inline void sort_bucket_long(int32_t* stage, int32_t* bucket, int32_t
     __syncthreads();   // the bucket is in order for every wavefront of the workgroup; stage may be refilled
 }
 
+// Elements: uint16_t holds bf16 bits, f16_bits fp16 bits; both are summed in fp32 and rounded once on the way out.
+struct f16_bits {
+    uint16_t u;
+};
+__device__ inline float f16_to_f32(uint16_t u) {
+    _Float16 h;
+    __builtin_memcpy(&h, &u, 2);
+    return static_cast<float>(h);
+}
+__device__ inline uint16_t f32_to_f16(float f) {
+    const _Float16 h = static_cast<_Float16>(f);
+    uint16_t u;
+    __builtin_memcpy(&u, &h, 2);
+    return u;
+}
 __device__ inline float load_as_f32(const uint16_t* p) { return __uint_as_float(static_cast<uint32_t>(*p) << 16); }
+__device__ inline float load_as_f32(const f16_bits* p) { return f16_to_f32(p->u); }
 __device__ inline float load_as_f32(const float* p) { return *p; }
 
 __device__ inline void store_from_f32(uint16_t* p, float f) {
@@ -257,6 +273,7 @@ __device__ inline void store_from_f32(uint16_t* p, float f) {
     }
     *p = b;
 }
+__device__ inline void store_from_f32(f16_bits* p, float f) { p->u = f32_to_f16(f); }
 __device__ inline void store_from_f32(float* p, float f) { *p = f; }
 
 // Order of the tokens of a bucket of at most 64: lane i holds one token and
@@ -347,12 +364,12 @@ __global__ __launch_bounds__(kBlock) void emb_bwd_reduce(const T* __restrict__ d
     }
 }
 
-// The same for bf16 rows that can be moved 16 bytes at a time: a lane owns the
+// The same for bf16 or fp16 (HALF) rows that can be moved 16 bytes at a time: a lane owns the
 // eight consecutive columns chunk * kChunk + 8 lane .. + 7, so one load
 // instruction of the wavefront covers a chunk, and an item is a group of CPW
 // chunks of its row so that the loads of a token overlap and the walk through
 // the bucket is paid once for all of them.
-template <int CPW>
+template <int CPW, bool HALF>
 __global__ __launch_bounds__(kBlock) void emb_bwd_reduce_bf16x8(const uint16_t* __restrict__ dy, int64_t dim, int64_t ld_dy,
                                                                 const int32_t* __restrict__ count, const int32_t* __restrict__ begin,
                                                                 int32_t* bucket, int64_t rows, int groups, int rows_per_block,
@@ -385,8 +402,8 @@ __global__ __launch_bounds__(kBlock) void emb_bwd_reduce_bf16x8(const uint16_t* 
                     const uint32_t w4[4] = {q[j].x, q[j].y, q[j].z, q[j].w};
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        acc[j][2 * e] += __uint_as_float(w4[e] << 16);
-                        acc[j][2 * e + 1] += __uint_as_float(w4[e] & 0xFFFF0000u);
+                        acc[j][2 * e] += HALF ? f16_to_f32(static_cast<uint16_t>(w4[e])) : __uint_as_float(w4[e] << 16);
+                        acc[j][2 * e + 1] += HALF ? f16_to_f32(static_cast<uint16_t>(w4[e] >> 16)) : __uint_as_float(w4[e] & 0xFFFF0000u);
                     }
                 }
             }
@@ -398,7 +415,12 @@ __global__ __launch_bounds__(kBlock) void emb_bwd_reduce_bf16x8(const uint16_t* 
             if (c0 + j * kChunk >= dim) continue;
             uint16_t o[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) store_from_f32(&o[e], acc[j][e] * scale);
+            for (int e = 0; e < 8; ++e) {
+                if (HALF)
+                    o[e] = f32_to_f16(acc[j][e] * scale);
+                else
+                    store_from_f32(&o[e], acc[j][e] * scale);
+            }
             uint4 q;
             q.x = o[0] | (static_cast<uint32_t>(o[1]) << 16);
             q.y = o[2] | (static_cast<uint32_t>(o[3]) << 16);
@@ -418,12 +440,16 @@ inline int rows_per_block_for(int items_per_row) { return items_per_row >= 3 ? 1
 
 template <int CPW>
 void launch_reduce_x8(const void* dy, int64_t dim, int64_t ld_dy, const int32_t* count, const int32_t* begin, int32_t* bucket,
-                      int64_t rows, int chunks, void* dw, int64_t ld_dw, int scale_by_freq, hipStream_t s) {
+                      int64_t rows, int chunks, void* dw, int64_t ld_dw, int scale_by_freq, bool half, hipStream_t s) {
     const int groups = (chunks + CPW - 1) / CPW;
     const int rpb = rows_per_block_for(groups);
-    hipLaunchKernelGGL((emb_bwd_reduce_bf16x8<CPW>), dim3(static_cast<uint32_t>((rows + rpb - 1) / rpb)), dim3(kBlock), 0, s,
-                       static_cast<const uint16_t*>(dy), dim, ld_dy, count, begin, bucket, rows, groups, rpb,
-                       static_cast<uint16_t*>(dw), ld_dw, scale_by_freq);
+    const dim3 grid(static_cast<uint32_t>((rows + rpb - 1) / rpb));
+    if (half)
+        hipLaunchKernelGGL((emb_bwd_reduce_bf16x8<CPW, true>), grid, dim3(kBlock), 0, s, static_cast<const uint16_t*>(dy), dim, ld_dy, count,
+                           begin, bucket, rows, groups, rpb, static_cast<uint16_t*>(dw), ld_dw, scale_by_freq);
+    else
+        hipLaunchKernelGGL((emb_bwd_reduce_bf16x8<CPW, false>), grid, dim3(kBlock), 0, s, static_cast<const uint16_t*>(dy), dim, ld_dy, count,
+                           begin, bucket, rows, groups, rpb, static_cast<uint16_t*>(dw), ld_dw, scale_by_freq);
 }
 
 template <typename IdT>
@@ -449,14 +475,18 @@ int run(const void* dy, int dtype, int64_t dim, int64_t ld_dy, const IdT* ids, i
                                cursor, bucket);
     }
     const int chunks = static_cast<int>((dim + kChunk - 1) / kChunk);
-    const bool vec = dtype == DDL_DT_BF16 && dim % 8 == 0 && ld_dy % 8 == 0 && ld_dw % 8 == 0 && aligned_to(dy, 16) && aligned_to(dw, 16);
+    const bool half = dtype == DDL_DT_F16;
+    const bool vec = (dtype == DDL_DT_BF16 || half) && dim % 8 == 0 && ld_dy % 8 == 0 && ld_dw % 8 == 0 && aligned_to(dy, 16) && aligned_to(dw, 16);
     if (vec) {
-        if (chunks >= 2) launch_reduce_x8<2>(dy, dim, ld_dy, count, begin, bucket, rows, chunks, dw, ld_dw, scale_by_freq, s);
-        else launch_reduce_x8<1>(dy, dim, ld_dy, count, begin, bucket, rows, chunks, dw, ld_dw, scale_by_freq, s);
+        if (chunks >= 2) launch_reduce_x8<2>(dy, dim, ld_dy, count, begin, bucket, rows, chunks, dw, ld_dw, scale_by_freq, half, s);
+        else launch_reduce_x8<1>(dy, dim, ld_dy, count, begin, bucket, rows, chunks, dw, ld_dw, scale_by_freq, half, s);
     } else {
         const int rpb = rows_per_block_for(chunks);
         const dim3 rgrid(static_cast<uint32_t>((rows + rpb - 1) / rpb));
-        if (dtype == DDL_DT_BF16)
+        if (half)
+            hipLaunchKernelGGL((emb_bwd_reduce<f16_bits>), rgrid, dim3(kBlock), 0, s, static_cast<const f16_bits*>(dy), dim, ld_dy, count,
+                               begin, bucket, rows, chunks, rpb, static_cast<f16_bits*>(dw), ld_dw, scale_by_freq);
+        else if (dtype == DDL_DT_BF16)
             hipLaunchKernelGGL((emb_bwd_reduce<uint16_t>), rgrid, dim3(kBlock), 0, s, static_cast<const uint16_t*>(dy), dim, ld_dy, count,
                                begin, bucket, rows, chunks, rpb, static_cast<uint16_t*>(dw), ld_dw, scale_by_freq);
         else
@@ -519,12 +549,13 @@ extern "C" int ddl_embedding_backward(const void* dy, int dtype, int64_t dim, in
     if (dim < 0 || ld_dy < dim || ld_dw < dim || n_ids < 0 || hi < lo)
         return fail(DDL_E_ARG, "embedding backward: dim=%lld ld_dy=%lld ld_dw=%lld n_ids=%lld window=[%lld,%lld)", (long long)dim,
                     (long long)ld_dy, (long long)ld_dw, (long long)n_ids, (long long)lo, (long long)hi);
-    if (dtype != DDL_DT_BF16 && dtype != DDL_DT_F32) return fail(DDL_E_UNSUPP, "embedding backward: dtype %d (bf16 and f32 only)", dtype);
+    if (dtype != DDL_DT_BF16 && dtype != DDL_DT_F16 && dtype != DDL_DT_F32)
+        return fail(DDL_E_UNSUPP, "embedding backward: dtype %d (bf16, f16 and f32 only)", dtype);
     const int64_t rows = hi - lo;
     if (rows == 0 || dim == 0) return 0;
     if (n_ids > 0x7FFFFFFFll || rows > 0x3FFFFFFFll) return fail(DDL_E_UNSUPP, "embedding backward: more than 2^31 tokens or 2^30 rows");
     if (!dweight || !workspace || (n_ids > 0 && (!dy || !ids))) return fail(DDL_E_ARG, "embedding backward: null pointer");
-    const int es = dtype == DDL_DT_BF16 ? 2 : 4;
+    const int es = dtype == DDL_DT_F32 ? 4 : 2;
     if (!aligned_to(dy, es) || !aligned_to(dweight, es) || !aligned_to(workspace, 4) || !aligned_to(ids, ids_is_i64 ? 8 : 4))
         return fail(DDL_E_ALIGN, "embedding backward: pointer misaligned");
     const int64_t need = 3 * rows + 1 + n_ids;

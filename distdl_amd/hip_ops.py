@@ -642,8 +642,8 @@ def embedding_backward(grad_output, ids, lo, hi, padding_idx=None, scale_grad_by
     table; with ``scale_grad_by_freq`` every row's sum is divided by the number
     of tokens that looked the row up."""
     _require_gpu(grad_output, ids)
-    if grad_output.dtype not in (torch.bfloat16, torch.float32):
-        raise ValueError("embedding_backward: bfloat16 or float32 gradients only")
+    if grad_output.dtype not in _LN_DTYPES:
+        raise ValueError("embedding_backward: bfloat16, float16 or float32 gradients only")
     if ids.dtype not in (torch.int64, torch.int32):
         raise ValueError("embedding_backward: ids must be int32 or int64")
     dim = grad_output.shape[-1]
@@ -656,7 +656,7 @@ def embedding_backward(grad_output, ids, lo, hi, padding_idx=None, scale_grad_by
     rows, n_ids = int(hi) - int(lo), ids_c.numel()
     dw = torch.empty((rows, dim), dtype=grad_output.dtype, device=grad_output.device)
     work = torch.empty(3 * rows + 1 + n_ids, dtype=torch.int32, device=grad_output.device)
-    dt = _lib.DDL_DT_BF16 if grad_output.dtype == torch.bfloat16 else _lib.DDL_DT_F32
+    dt = _LN_DTYPES[grad_output.dtype]
     rc = _lib.load().ddl_embedding_backward(dy.data_ptr(), dt, dim, dy.stride(0) if n_ids > 1 else dim, ids_c.data_ptr(),
                                             1 if ids.dtype == torch.int64 else 0, n_ids, int(lo), int(hi),
                                             -1 if padding_idx is None else int(padding_idx), 1 if scale_grad_by_freq else 0,

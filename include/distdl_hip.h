@@ -408,8 +408,8 @@ int ddl_embedding_renorm(void* weight, int dtype, int64_t dim, int64_t ldw,
  *   dweight[r, :] = sum over t with ids[t] - lo == r and ids[t] != padding_idx
  *                   of dy[t, :]                        for every r in [0, hi-lo)
  * (what autograd derives for torch.nn.functional.embedding,
- * nn/embedding.py:244-246; padding_idx < 0 = none).  dtype = DDL_DT_BF16 or
- * DDL_DT_F32 for dy and dweight alike; sums are accumulated in fp32 in
+ * nn/embedding.py:244-246; padding_idx < 0 = none).  dtype = DDL_DT_BF16,
+ * DDL_DT_F16 or DDL_DT_F32 for dy and dweight alike; sums are accumulated in fp32 in
  * ascending token order whatever the length of a row's token list, so the
  * result is the same on every run.  With scale_grad_by_freq != 0 each row's
  * sum is divided by the number of tokens that contributed to it

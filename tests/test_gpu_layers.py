@@ -951,7 +951,7 @@ def test_embedding_training_step_reference_cases(P, table_shape):
         assert np.allclose(grad, want_grad[r], rtol=rtol, atol=atol)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("dim,rows,tokens", [(1, 1, 1), (8, 10, 50), (100, 37, 300), (512, 64, 1000), (1000, 5, 4000),
                                               (4100, 20, 100)])
 @pytest.mark.parametrize("idt", [torch.int64, torch.int32])
@@ -996,7 +996,7 @@ def test_embedding_backward_matches_torch_autograd_on_random_data(ops):
     assert np.allclose(got, tw.grad.double().numpy(), rtol=2.0 ** -7, atol=1e-4)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_embedding_backward_long_buckets_are_summed_in_token_order(ops, dtype):
     """Rows looked up 65 to several thousand times with random float gradients:
     the sums run in ascending token order whatever order the bucket fill
@@ -1022,11 +1022,11 @@ def test_embedding_backward_long_buckets_are_summed_in_token_order(ops, dtype):
     assert torch.equal(first, want.to(dtype))
     for _ in range(3):
         again = ops.embedding_backward(dy.cuda(), ids.cuda(), 4, 4 + rows).cpu()
-        assert torch.equal(again.view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
-                           first.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+        as_bits = torch.int32 if dtype == torch.float32 else torch.int16
+        assert torch.equal(again.view(as_bits), first.view(as_bits))
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_embedding_backward_scale_grad_by_freq(ops, dtype):
     """Each row's sum divided by its number of contributing tokens, against the
     oracle (pinned to torch autograd) and through the layer's autograd path."""
@@ -1036,7 +1036,7 @@ def test_embedding_backward_scale_grad_by_freq(ops, dtype):
     dy = torch.randn(6, 50, 96, generator=gen).to(dtype)
     got = ops.embedding_backward(dy.cuda(), ids.cuda(), 5, 30, padding_idx=7, scale_grad_by_freq=True)
     want = o_emb.backward(dy.double().numpy(), ids.numpy(), 5, 30, padding_idx=7, scale_grad_by_freq=True)
-    tol = 2.0 ** -7 if dtype == torch.bfloat16 else 1e-5
+    tol = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10, torch.float32: 1e-5}[dtype]
     assert (np.abs(got.cpu().double().numpy() - want) <= tol * np.abs(want) + 1e-6).all()
     w = torch.zeros(25, 96, dtype=dtype, device="cuda", requires_grad=True)
     _EmbeddingShard.apply(w, ids.cuda(), 5, 30, 7, True).backward(dy.cuda())
